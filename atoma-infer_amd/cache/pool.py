@@ -1,0 +1,133 @@
+"""Device memory of the cache, laid out from a model's run order.
+
+Every layer call that owns a cache entry is put into the group of its ``CacheSpec`` (KV heads, head size,
+window); a group has one pool of pages, and a page holds ``page_size`` tokens of every entry of its group, so
+one page number serves all those layers (the reference does the same for its single group:
+backends/vllm/src/worker.rs:570-598).  Keys of an entry are [pages, kv_heads, page_size, head] and values
+[pages, kv_heads, head, page_size]: a (page, head) tile is contiguous, keys along the head axis and values
+along the token axis, which is how the attention kernels read them.
+
+Mixers that declare a ``StateSpec`` get a float32 tensor [slots, *shape] per layer call, indexed by the
+request's state slot.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..parts.base import CacheSpec
+from .manager import CacheManager, GroupGeometry
+
+
+@dataclasses.dataclass
+class GroupPlan:
+    spec: CacheSpec
+    calls: List[int]          # run-order positions that own an entry of this group
+
+    def bytes_per_token(self, elem: int) -> int:
+        return 2 * len(self.calls) * self.spec.kv_heads * self.spec.head_size * elem
+
+
+@dataclasses.dataclass
+class CachePlan:
+    groups: List[GroupPlan]
+    #: run-order position -> (group, entry within group, writable); absent for calls whose mixer keeps no cache
+    where: Dict[int, Tuple[int, int, bool]]
+    #: run-order position -> state shape
+    states: Dict[int, Tuple[int, ...]]
+
+    def bytes_per_token(self, elem: int) -> int:
+        return sum(g.bytes_per_token(elem) for g in self.groups)
+
+
+def plan_cache(spec) -> CachePlan:
+    groups: List[GroupPlan] = []
+    index: Dict[CacheSpec, int] = {}
+    where: Dict[int, Tuple[int, int, bool]] = {}
+    states: Dict[int, Tuple[int, ...]] = {}
+    for pos, call in enumerate(spec.run_order):
+        mixer = spec.layers[call.layer][1].mixer
+        st = mixer.state_spec()
+        if st is not None:
+            states[pos] = tuple(st.shape)
+        cs = mixer.cache_spec()
+        if cs is None:
+            continue
+        if call.kv_from is not None:
+            g, e, _ = where[call.kv_from]
+            where[pos] = (g, e, False)
+            continue
+        if cs not in index:
+            index[cs] = len(groups)
+            groups.append(GroupPlan(cs, []))
+        g = index[cs]
+        where[pos] = (g, len(groups[g].calls), True)
+        groups[g].calls.append(pos)
+    return CachePlan(groups, where, states)
+
+
+@dataclasses.dataclass
+class LayerCache:
+    """What one layer call sees of the cache in one step."""
+    k: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None
+    page_size: int = 1
+    writable: bool = True
+    group: int = -1
+    slot_mapping: Optional[torch.Tensor] = None     # [T] int32: page * page_size + offset of each token
+    block_tables: Optional[torch.Tensor] = None     # [S, blocks] int32
+    state: Optional[torch.Tensor] = None            # [slots, *shape] float32
+
+
+class CachePool:
+    """Pages and state tensors on the device, with the manager that hands them out."""
+
+    def __init__(self, plan: CachePlan, page_size: int, num_pages: List[int], num_state_slots: int,
+                 dtype: torch.dtype, device: torch.device):
+        if len(num_pages) != len(plan.groups):
+            raise ValueError("one page count per group is needed")
+        self.plan, self.page_size, self.dtype, self.device = plan, int(page_size), dtype, device
+        self.num_state_slots = int(num_state_slots)
+        self.k: List[torch.Tensor] = []
+        self.v: List[torch.Tensor] = []
+        geometry = []
+        for g, n in zip(plan.groups, num_pages):
+            cs = g.spec
+            # zero-filled, so that pages never written hold finite numbers
+            self.k.append(torch.zeros((len(g.calls), n, cs.kv_heads, page_size, cs.head_size), dtype=dtype,
+                                      device=device))
+            self.v.append(torch.zeros((len(g.calls), n, cs.kv_heads, cs.head_size, page_size), dtype=dtype,
+                                      device=device))
+            geometry.append(GroupGeometry(page_size, n, cs.window))
+        self.states = {pos: torch.zeros((num_state_slots, *shape), dtype=torch.float32, device=device)
+                       for pos, shape in plan.states.items()}
+        self.manager = CacheManager(geometry, num_state_slots)
+
+    def layer_cache(self, pos: int, slot_mappings, block_tables) -> LayerCache:
+        lc = LayerCache(state=self.states.get(pos))
+        if pos in self.plan.where:
+            g, e, writable = self.plan.where[pos]
+            lc.k, lc.v, lc.page_size, lc.writable, lc.group = self.k[g][e], self.v[g][e], self.page_size, writable, g
+            lc.slot_mapping, lc.block_tables = slot_mappings[g], block_tables[g]
+        return lc
+
+    def bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.k + self.v)
+
+
+def pages_for_tokens(plan: CachePlan, page_size: int, max_tokens: int, max_requests: int) -> List[int]:
+    """Pages per group so that ``max_tokens`` tokens, each request's count rounded up to whole pages, fit."""
+    per_group = -(-max_tokens // page_size)
+    return [max(per_group, 1) for _ in plan.groups]
+
+
+def pages_for_memory(plan: CachePlan, page_size: int, elem: int, budget_bytes: int) -> List[int]:
+    """Pages per group from a byte budget, the same number in each group
+    (the reference: floor(free x utilization / bytes per page), backends/vllm/src/config.rs:195-208, 708-718)."""
+    per_page = plan.bytes_per_token(elem) * page_size
+    if per_page == 0:
+        return []
+    n = max(int(budget_bytes // per_page), 1)
+    return [n for _ in plan.groups]

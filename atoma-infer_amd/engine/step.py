@@ -1,0 +1,222 @@
+"""The step function: run one batch of (request, its next tokens) from the cache and return logits.
+
+A step's entries may be portions of prompts beside single decoded tokens, in any order and cut anywhere.  The
+step runs only the tokens it is given, as one batch; keys and values of those tokens are written to the cache
+first, then every token at position p attends keys 0..p of its own request through the block table.  Logits
+come back only for the places asked for, in float32.
+
+The reference's counterpart is ``ModelWorker::execute_model`` with ``prepare_input_tensors``
+(backends/vllm/src/worker.rs:111-191, 224-460); unlike it, a later portion of a prompt sees the earlier ones.
+All integer metadata of a step travels to the device in one pinned buffer and one copy.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.pool import CachePool, LayerCache
+
+
+class StepError(ValueError):
+    pass
+
+
+@dataclasses.dataclass
+class StepEntry:
+    """The next tokens of one request.
+
+    ``start`` is the position of ``tokens[0]``: the number of tokens of this request already in the cache.
+    ``want`` lists the indices into ``tokens`` whose logits are asked for.
+    """
+    request: int
+    tokens: Sequence[int]
+    start: int
+    want: Sequence[int] = ()
+
+
+@dataclasses.dataclass
+class StepContext:
+    """Device-side description of one step, as the parts see it."""
+    n_tokens: int
+    n_entries: int
+    n_want: int
+    tokens: torch.Tensor            # [T] int32
+    positions: torch.Tensor         # [T] int32 absolute positions
+    token_seq: torch.Tensor         # [T] int32: the entry (row of the block tables) of each token
+    q_start: torch.Tensor           # [S+1] int32: first token of each entry
+    seq_lens: torch.Tensor          # [S] int32: tokens of each request after this step
+    state_slots: torch.Tensor       # [S] int32
+    want_rows: Optional[torch.Tensor]   # [n_want] int32 rows of the step
+    # host copies, for launch decisions
+    h_starts: np.ndarray            # [S] position of each entry's first token
+    h_counts: np.ndarray            # [S] tokens of each entry
+    h_state_slots: np.ndarray
+    max_count: int
+    max_seq_len: int
+    slot_mappings: List[torch.Tensor] = dataclasses.field(default_factory=list)   # per group [T]
+    block_tables: List[torch.Tensor] = dataclasses.field(default_factory=list)    # per group [S, blocks]
+    pool: Optional[CachePool] = None
+    scratch: Dict[str, object] = dataclasses.field(default_factory=dict)          # per-step notes of kernels
+
+    def layer_cache(self, pos: int) -> LayerCache:
+        return self.pool.layer_cache(pos, self.slot_mappings, self.block_tables)
+
+
+class _Staging:
+    """A pinned host buffer and its device twin, grown on demand."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self.host: Optional[torch.Tensor] = None
+        self.dev: Optional[torch.Tensor] = None
+
+    def ensure(self, n: int):
+        if self.host is None or self.host.numel() < n:
+            cap = max(1024, 1 << (n - 1).bit_length())
+            self.host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+            self.dev = torch.empty(cap, dtype=torch.int32, device=self.device)
+        return self.host.numpy()
+
+
+class ModelRunner:
+    """Owns the model and the cache pool of one GPU and steps batches through them."""
+
+    def __init__(self, model, pool: CachePool):
+        self.model, self.pool = model, pool
+        self.manager = pool.manager
+        self._stage = _Staging(model.device)
+        self._pending = None
+        self._computed: Dict[int, int] = {}       # request -> tokens in the cache
+
+    # -- requests ------------------------------------------------------------------------------------
+    def add_request(self, request: int) -> int:
+        slot = self.manager.add(request)
+        self._computed[request] = 0
+        for st in self.pool.states.values():
+            st[slot].zero_()
+        return slot
+
+    def has_request(self, request: int) -> bool:
+        return request in self._computed
+
+    def computed_len(self, request: int) -> int:
+        return self._computed[request]
+
+    def free_request(self, request: int) -> None:
+        self.manager.free(request)
+        del self._computed[request]
+
+    def reset_request(self, request: int) -> None:
+        """Drop what a request holds but keep it registered (recompute-preemption)."""
+        self.free_request(request)
+        self.add_request(request)
+
+    # -- the step ------------------------------------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        vocab, max_pos = self.model.vocab_size, self.model.spec.max_positions
+        for e in entries:
+            if e.request in seen:
+                raise StepError(f"request {e.request} appears twice in one step")
+            seen.add(e.request)
+            if e.request not in self._computed:
+                raise StepError(f"request {e.request} is not registered")
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.request}: an entry needs at least one token")
+            if e.start != self._computed[e.request]:
+                raise StepError(f"request {e.request}: tokens start at position {e.start}, but the cache holds "
+                                f"{self._computed[e.request]} tokens")
+            if e.start + n > max_pos:
+                raise StepError(f"request {e.request}: position {e.start + n - 1} exceeds max_position_embeddings "
+                                f"{max_pos}")
+            lo, hi = min(e.tokens), max(e.tokens)
+            if lo < 0 or hi >= vocab:
+                raise StepError(f"request {e.request}: token id {lo if lo < 0 else hi} outside the vocabulary "
+                                f"of {vocab}")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise StepError(f"request {e.request}: wanted place {w} outside its {n} tokens")
+
+    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Reserve pages and build the step's metadata on the device."""
+        self._validate(entries)
+        self.wait_staging()
+        mgr = self.manager
+        for e in entries:
+            mgr.reserve(e.request, e.start + len(e.tokens))
+        s = len(entries)
+        counts = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=s)
+        starts = np.fromiter((e.start for e in entries), dtype=np.int32, count=s)
+        ids = np.fromiter((e.request for e in entries), dtype=np.int64, count=s)
+        t = int(counts.sum())
+        n_want = sum(len(e.want) for e in entries)
+        n_groups = len(self.pool.plan.groups)
+        max_seq = int((starts + counts).max())
+        max_blocks = -(-max_seq // self.pool.page_size)
+        # layout of the one staging buffer
+        o_tok, o_pos, o_seq = 0, t, 2 * t
+        o_qs, o_len, o_slot = 3 * t, 3 * t + s + 1, 3 * t + 2 * s + 1
+        o_want = 3 * t + 3 * s + 1
+        o_sm = o_want + n_want
+        o_bt = o_sm + n_groups * t
+        total = o_bt + n_groups * s * max_blocks
+        buf = self._stage.ensure(total)
+        q_start = np.zeros(s + 1, dtype=np.int32)
+        np.cumsum(counts, out=q_start[1:])
+        row = 0
+        wi = o_want
+        for i, e in enumerate(entries):
+            n = counts[i]
+            buf[o_tok + row: o_tok + row + n] = e.tokens
+            buf[o_pos + row: o_pos + row + n] = np.arange(e.start, e.start + n, dtype=np.int32)
+            buf[o_seq + row: o_seq + row + n] = i
+            for w in e.want:
+                buf[wi] = row + w
+                wi += 1
+            row += n
+        buf[o_qs: o_qs + s + 1] = q_start
+        buf[o_len: o_len + s] = starts + counts
+        slots = np.fromiter((mgr.state_slot(e.request) for e in entries), dtype=np.int32, count=s)
+        buf[o_slot: o_slot + s] = slots
+        for g in range(n_groups):
+            sm = buf[o_sm + g * t: o_sm + (g + 1) * t]
+            bt = buf[o_bt + g * s * max_blocks: o_bt + (g + 1) * s * max_blocks].reshape(s, max_blocks)
+            mgr.fill_step(g, ids, starts, counts, sm, bt)
+        dev = self._stage.dev
+        dev[:total].copy_(self._stage.host[:total], non_blocking=True)
+        self._pending = torch.cuda.Event()
+        self._pending.record()
+        ctx = StepContext(
+            n_tokens=t, n_entries=s, n_want=n_want,
+            tokens=dev[o_tok: o_tok + t], positions=dev[o_pos: o_pos + t], token_seq=dev[o_seq: o_seq + t],
+            q_start=dev[o_qs: o_qs + s + 1], seq_lens=dev[o_len: o_len + s], state_slots=dev[o_slot: o_slot + s],
+            want_rows=dev[o_want: o_want + n_want] if n_want else None,
+            h_starts=starts, h_counts=counts, h_state_slots=slots, max_count=int(counts.max()), max_seq_len=max_seq,
+            slot_mappings=[dev[o_sm + g * t: o_sm + (g + 1) * t] for g in range(n_groups)],
+            block_tables=[dev[o_bt + g * s * max_blocks: o_bt + (g + 1) * s * max_blocks].view(s, max_blocks)
+                          for g in range(n_groups)],
+            pool=self.pool)
+        return ctx
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one batch; returns float32 logits [wanted places, vocab] (order: entries, then ``want``) or None."""
+        ctx = self.prepare(entries)
+        logits = self.model.forward(ctx)
+        for e in entries:
+            done = e.start + len(e.tokens)
+            self._computed[e.request] = done
+            self.manager.release_behind(e.request, done)
+        return logits
+
+    def wait_staging(self):
+        """The pinned metadata buffer is reused by every step: wait until the last copy out of it has been read."""
+        ev = getattr(self, "_pending", None)
+        if ev is not None:
+            ev.synchronize()
+            self._pending = None

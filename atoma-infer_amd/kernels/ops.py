@@ -1,0 +1,239 @@
+"""Python face of the HIP kernels: argument checks on the host, then one C call per op on the current stream.
+
+Every function takes device tensors and writes into tensors the caller passes or that it allocates with torch
+(torch is the allocator and the stream owner; it computes nothing here).  Shapes, strides and dtypes are checked
+before a launch, because a kernel that reads outside a tensor can take the GPU down.  A missing or unbuildable
+library raises ``KernelBuildError``; there is no other code path.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .library import load_hip_module
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise KernelError(f"{what}: dtype {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _p(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc: int, op: str):
+    if rc == 0:
+        return
+    if rc == -2:
+        raise KernelError(f"{op}: unsupported combination of element types")
+    if rc == -3:
+        raise KernelError(f"{op}: the kernel refuses these sizes")
+    raise KernelError(f"{op}: HIP error {rc}")
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None:
+            _need(t.is_cuda, "kernels run on device tensors only; got a CPU tensor")
+
+
+def _i32(t: torch.Tensor, what: str, n: Optional[int] = None):
+    _need(t.dtype is torch.int32 and t.is_contiguous(), f"{what} must be a contiguous int32 tensor")
+    if n is not None:
+        _need(t.numel() >= n, f"{what} has {t.numel()} entries, {n} are needed")
+
+
+_core = None
+
+
+def core():
+    global _core
+    if _core is None:
+        _core = load_hip_module("core")
+    return _core
+
+
+# ------------------------------------------------------------------------------------------------------------
+
+def embed(tokens: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = table[tokens[t]] as float32.  The caller guarantees 0 <= token < table rows."""
+    _dev(tokens, table)
+    _i32(tokens, "tokens")
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, width]")
+    n, width = tokens.numel(), table.shape[1]
+    if out is None:
+        out = torch.empty((n, width), dtype=torch.float32, device=table.device)
+    _need(out.dtype is torch.float32 and out.is_contiguous() and tuple(out.shape) == (n, width), "embed: bad out")
+    _check(core().atoma_embed(_p(tokens), _p(table), _code(table, "embedding table"), _p(out), n, width, _stream()),
+           "embed")
+    return out
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """resid += delta (in place, float32); return rmsnorm(resid) * weight in ``out_dtype``.
+
+    With ``rows`` (int32 row numbers) only those rows are summed and normed, into a result of len(rows) rows,
+    and resid is left as it is.
+    """
+    _dev(resid, delta, weight, rows)
+    _need(resid.dtype is torch.float32 and resid.dim() == 2 and resid.is_contiguous(), "resid must be float32 [T, W]")
+    t, width = resid.shape
+    _need(weight.is_contiguous() and weight.numel() == width, "norm weight must have one entry per column")
+    if delta is not None:
+        _need(delta.is_contiguous() and tuple(delta.shape) == (t, width), "delta must match resid")
+    n = t
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.numel()
+    if out is None:
+        out = torch.empty((n, width), dtype=out_dtype, device=resid.device)
+    _need(out.is_contiguous() and tuple(out.shape) == (n, width) and out.dtype is out_dtype, "add_rmsnorm: bad out")
+    _check(core().atoma_add_rmsnorm(_p(resid), _p(delta), _code(delta, "delta") if delta is not None else F32,
+                                    _p(weight), _code(weight, "norm weight"), _p(out), _code(out, "out"), _p(rows),
+                                    n, width, ctypes.c_float(eps), _stream()), "add_rmsnorm")
+    return out
+
+
+def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torch.Tensor],
+                     sin: Optional[torch.Tensor], rotary_dim: int, kcache: Optional[torch.Tensor],
+                     vcache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], page_size: int, nh: int,
+                     nkv: int, hd: int) -> None:
+    """Rotate q and k of ``qkv`` [T, (nh + 2 nkv) hd] (q in place), store rotated k and v at ``slot_mapping``.
+
+    kcache is [pages, nkv, page_size, hd], vcache [pages, nkv, hd, page_size].  Null caches: rotate q only.
+    """
+    _dev(qkv, positions, cos, sin, kcache, vcache, slot_mapping)
+    t = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= (nh + 2 * nkv) * hd, "qkv: bad shape")
+    _i32(positions, "positions", t)
+    if cos is not None:
+        _need(sin is not None and cos.dtype is torch.float32 and sin.dtype is torch.float32 and cos.is_contiguous()
+              and sin.is_contiguous() and cos.shape == sin.shape and cos.shape[1] == rotary_dim // 2,
+              "rotary tables must be float32 [positions, rotary_dim/2]")
+    cache_code = _code(qkv, "qkv")
+    if kcache is not None:
+        _need(vcache is not None and slot_mapping is not None, "cache write needs k, v and slots")
+        _i32(slot_mapping, "slot_mapping", t)
+        pages = kcache.shape[0]
+        _need(kcache.is_contiguous() and vcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size, hd)
+              and tuple(vcache.shape) == (pages, nkv, hd, page_size) and kcache.dtype is vcache.dtype,
+              "cache tensors must be [pages, nkv, page, hd] and [pages, nkv, hd, page]")
+        cache_code = _code(kcache, "cache")
+    _check(core().atoma_rope_cache_write(_p(qkv), _code(qkv, "qkv"), qkv.stride(0), _p(positions), _p(cos), _p(sin),
+                                         rotary_dim, _p(kcache), _p(vcache), cache_code, _p(slot_mapping), page_size,
+                                         t, nh, nkv, hd, _stream()), "rope_cache_write")
+
+
+def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, out: torch.Tensor,
+                            block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
+                            scale: float, window: int, page_size: int, nh: int, nkv: int, hd: int) -> None:
+    """Attention of every token of ``q`` [T, >= nh hd] (row stride free) over its request's cached keys.
+
+    Token t belongs to row ``token_seq[t]`` of ``block_tables`` and sits at absolute position ``positions[t]``;
+    it sees keys max(0, p - window + 1) .. p (window 0: all).  ``out`` is [T, nh hd].
+    """
+    _dev(q, kcache, vcache, out, block_tables, token_seq, positions)
+    t = q.shape[0]
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nh * hd, "q: bad shape")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == t and out.shape[1] >= nh * hd
+          and out.dtype is q.dtype, "out: bad shape")
+    pages = kcache.shape[0]
+    _need(kcache.is_contiguous() and vcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size, hd)
+          and tuple(vcache.shape) == (pages, nkv, hd, page_size) and kcache.dtype is vcache.dtype,
+          "cache tensors must be [pages, nkv, page, hd] and [pages, nkv, hd, page]")
+    _need(block_tables.dim() == 2 and block_tables.dtype is torch.int32 and block_tables.is_contiguous(),
+          "block_tables must be contiguous int32 [requests, blocks]")
+    _i32(token_seq, "token_seq", t)
+    _i32(positions, "positions", t)
+    _check(core().atoma_paged_attention_generic(
+        _p(q), q.stride(0), _p(kcache), _p(vcache), _p(out), out.stride(0), _code(q, "q"), _code(kcache, "cache"),
+        _p(block_tables), block_tables.shape[1], _p(token_seq), _p(positions), ctypes.c_float(scale), int(window),
+        page_size, t, nh, nkv, hd, _stream()), "paged_attention_generic")
+
+
+def swiglu(gu: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, i] = silu(gu[t, i]) * gu[t, I + i] for gu [T, 2 I]."""
+    _dev(gu)
+    _need(gu.dim() == 2 and gu.is_contiguous() and gu.shape[1] % 2 == 0, "swiglu input must be contiguous [T, 2 I]")
+    t, inter = gu.shape[0], gu.shape[1] // 2
+    if out is None:
+        out = torch.empty((t, inter), dtype=gu.dtype, device=gu.device)
+    _need(out.is_contiguous() and tuple(out.shape) == (t, inter) and out.dtype is gu.dtype, "swiglu: bad out")
+    _check(core().atoma_swiglu(_p(gu), _p(out), _code(gu, "swiglu input"), t, inter, _stream()), "swiglu")
+    return out
+
+
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None,
+                 ) -> torch.Tensor:
+    """a [M, K] times w [N, K] transposed, in true float32 arithmetic; any sizes."""
+    _dev(a, w)
+    _need(a.dim() == 2 and w.dim() == 2 and a.stride(1) == 1 and w.stride(1) == 1 and a.shape[1] == w.shape[1],
+          f"gemm: a {tuple(a.shape)} and w {tuple(w.shape)} do not fit")
+    m, k = a.shape
+    n = w.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    _need(out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (m, n) and out.dtype is out_dtype,
+          "gemm: bad out")
+    _check(core().atoma_gemm_generic(_p(a), _code(a, "a"), _p(w), _code(w, "w"), _p(out), _code(out, "out"), m, n, k,
+                                     a.stride(0) if m > 1 else k, w.stride(0) if n > 1 else k,
+                                     out.stride(0) if m > 1 else n, _stream()), "gemm_generic")
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None):
+    """Per row of float32 ``logits`` [S, V]: argmax where temperature <= 0, else a draw (see sampling.hip).
+
+    Returns (tokens int32 [S], logits of the chosen tokens float32 [S]).
+    """
+    _dev(logits, temperature, top_k, top_p, uniform)
+    _need(logits.dim() == 2 and logits.dtype is torch.float32 and logits.stride(1) == 1, "logits must be float32 [S, V]")
+    s, v = logits.shape
+    for name, x, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                        ("top_p", top_p, torch.float32), ("uniform", uniform, torch.float32)):
+        _need(x.dtype is dt and x.is_contiguous() and x.numel() == s, f"{name} must be {dt} [S]")
+    if workspace is None:
+        workspace = torch.empty((s, v), dtype=torch.float32, device=logits.device)
+    _need(workspace.dtype is torch.float32 and workspace.is_contiguous() and workspace.numel() >= s * v,
+          "sample: workspace too small")
+    tok = torch.empty((s,), dtype=torch.int32, device=logits.device)
+    lg = torch.empty((s,), dtype=torch.float32, device=logits.device)
+    _check(core().atoma_sample(_p(logits), logits.stride(0) if s > 1 else v, s, v, _p(temperature), _p(top_k),
+                               _p(top_p), _p(uniform), _p(workspace), _p(tok), _p(lg), _stream()), "sample")
+    return tok, lg
+
+
+def repeat_penalty(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, penalty: torch.Tensor) -> None:
+    """In place: for each pair (rows[i], tokens[i]) the logit is divided (if >= 0) or multiplied by penalty[row]."""
+    _dev(logits, rows, tokens, penalty)
+    _need(logits.dim() == 2 and logits.dtype is torch.float32 and logits.stride(1) == 1, "logits must be float32 [S, V]")
+    n = rows.numel()
+    _i32(rows, "rows")
+    _i32(tokens, "tokens", n)
+    _need(penalty.dtype is torch.float32 and penalty.numel() == logits.shape[0], "penalty must be float32 [S]")
+    _check(core().atoma_repeat_penalty(_p(logits), logits.stride(0), _p(rows), _p(tokens), _p(penalty), n, _stream()),
+           "repeat_penalty")

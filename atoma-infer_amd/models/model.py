@@ -1,0 +1,65 @@
+"""A model at run time: the parts of a ModelSpec with their weights on the device, and its forward pass.
+
+The forward pass runs only the tokens of one step, as one batch: embedding gather, the layer calls in run order
+(each with its own view of the cache), the final norm on the rows whose logits are wanted, and the head
+(models/src/llama.rs:456-478 of the reference, which norms every row and selects afterwards).
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional
+
+import torch
+
+from ..config.base import ModelConfig
+from ..config.registry import Architecture, load_model_config
+from ..weights.loader import load_into
+from .spec import ModelSpec
+
+_ACT = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+@dataclasses.dataclass
+class Model:
+    arch: Architecture
+    config: ModelConfig
+    spec: ModelSpec
+    device: torch.device
+    act_dtype: torch.dtype
+
+    @property
+    def vocab_size(self) -> int:
+        return self.spec.vocab_size
+
+    def weight_bytes(self) -> int:
+        """Bytes of weights that one step reads (each matrix once; the embedding table only through a tied head)."""
+        return sum(part.device_bytes() for _, part in self.spec.parts())
+
+    def forward(self, ctx) -> Optional[torch.Tensor]:
+        """Logits [wanted rows, vocab] in float32, or None when the step wants none."""
+        spec = self.spec
+        resid = spec.embedding[1].forward(ctx.tokens)
+        delta = None
+        for pos, call in enumerate(spec.run_order):
+            delta = spec.layers[call.layer][1].forward(resid, delta, ctx, ctx.layer_cache(pos))
+        if ctx.n_want == 0:
+            return None
+        x = spec.final_norm[1].add_norm(resid, delta, rows=ctx.want_rows)
+        return spec.head[1].forward(x)
+
+
+def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") -> Model:
+    """Build the model that ``model_dir/config.json`` names and bind ``model_dir``'s weights to it.
+
+    ``dtype`` is the activation and cache dtype: "bfloat16" runs the serving kernels, "float32" everything in
+    true 32-bit arithmetic.  Weights stay as stored (bfloat16 or float32) in both.
+    """
+    if dtype not in _ACT:
+        raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}")
+    dev = torch.device(device)
+    if dev.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError("this engine runs on a GPU only (device 'cuda:N'); no GPU is visible")
+    arch, cfg = load_model_config(model_dir)
+    spec = arch.build(cfg)
+    load_into(spec, model_dir, dev, _ACT[dtype])
+    return Model(arch, cfg, spec, dev, _ACT[dtype])

@@ -1,0 +1,105 @@
+"""Causal self-attention over the paged cache, with grouped KV heads and an optional window.
+
+Projections without bias (models/src/llama.rs:269-271, 311, 322-325), head split by columns (:273-296), rotation
+of q and k (:298-299), keys and values written to the cache before attention (models/src/flash_attention.rs:
+360-361), softmax scale 1/sqrt(head size) (models/src/llama.rs:342), query head h on KV head h // (nh/nkv)
+(csrc/kernels/flash_fwd_kernel.h:593).  Where the reference runs separate kernels for prompt rows and decode rows
+(models/src/flash_attention.rs:380-466), one rule serves here: a token at position p sees keys 0..p (or the
+last ``window`` of them) of its own request through the block table.
+
+The three projection matrices are fused into one [(nh + 2 nkv) hd, width] matrix at load time; results equal
+the separate products.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import CacheSpec, Mixer, PositionEncoding, WeightSpec, register_mixer
+from .linear import linear
+
+
+class PagedAttention(Mixer):
+    def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_size: int,
+                 position: Optional[PositionEncoding] = None, window: Optional[int] = None,
+                 scale: Optional[float] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads cannot be grouped over {num_kv_heads} KV heads")
+        if head_size % 16 or not 16 <= head_size <= 256:
+            raise ValueError(f"head size {head_size} is not supported: the attention kernels take multiples of 16 "
+                             f"from 16 to 256")
+        if window is not None and window <= 0:
+            raise ValueError("window must be positive")
+        self.width, self.nh, self.nkv, self.hd = int(width), int(num_heads), int(num_kv_heads), int(head_size)
+        self.position = position
+        self.window = window
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+        self.act_dtype = torch.float32
+
+    # -- declaration ----------------------------------------------------------------------------------
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        q, kv = self.nh * self.hd, self.nkv * self.hd
+        return {"q_proj.weight": WeightSpec((q, self.width)), "k_proj.weight": WeightSpec((kv, self.width)),
+                "v_proj.weight": WeightSpec((kv, self.width)), "o_proj.weight": WeightSpec((self.width, q))}
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(self.nkv, self.hd, self.window)
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("q_proj.weight"), get("k_proj.weight"), get("v_proj.weight")]
+        dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        self.w_qkv = torch.cat([w.to(device=device, dtype=dt) for w in ws], dim=0).contiguous()
+        self.w_o = get("o_proj.weight").to(device).contiguous()
+        self.act_dtype = act_dtype
+        if self.position is not None:
+            self.position.load(get, device, act_dtype)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
+
+    # -- execution ------------------------------------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        nh, nkv, hd = self.nh, self.nkv, self.hd
+        t = x.shape[0]
+        writes = cache.writable
+        # a call that reads another call's cache needs its queries only
+        w = self.w_qkv if writes else self.w_qkv[: nh * hd]
+        qkv = linear(x, w)
+        k_cache, v_cache = cache.k, cache.v
+        tables = self.position.rotary_tables() if self.position is not None else None
+        if tables is not None or self.position is None:
+            cos, sin, rd = tables if tables is not None else (None, None, 0)
+            if writes:
+                ops.rope_cache_write(qkv, ctx.positions, cos, sin, rd, k_cache, v_cache, cache.slot_mapping,
+                                     cache.page_size, nh, nkv, hd)
+            else:
+                ops.rope_cache_write(qkv, ctx.positions, cos, sin, rd, None, None, None, 1, nh, 0, hd)
+        else:
+            q = qkv[:, : nh * hd].view(t, nh, hd)
+            if writes:
+                k = qkv[:, nh * hd: (nh + nkv) * hd].view(t, nkv, hd)
+                self.position.apply(q, k, ctx.positions)
+                ops.rope_cache_write(qkv, ctx.positions, None, None, 0, k_cache, v_cache, cache.slot_mapping,
+                                     cache.page_size, nh, nkv, hd)
+            else:
+                self.position.apply(q, q[:, :0], ctx.positions)
+        out = torch.empty((t, nh * hd), dtype=qkv.dtype, device=qkv.device)
+        self.attend(qkv, k_cache, v_cache, out, ctx, cache)
+        return linear(out, self.w_o)
+
+    def attend(self, q, k_cache, v_cache, out, ctx, cache) -> None:
+        if q.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16:
+            from ..kernels import attention_bf16
+            if attention_bf16.try_attention(q, k_cache, v_cache, out, ctx, cache, self.scale, self.window or 0,
+                                            self.nh, self.nkv, self.hd):
+                return
+        ops.paged_attention_generic(q, k_cache, v_cache, out, cache.block_tables, ctx.token_seq, ctx.positions,
+                                    self.scale, self.window or 0, cache.page_size, self.nh, self.nkv, self.hd)
+
+
+register_mixer("attention", PagedAttention)

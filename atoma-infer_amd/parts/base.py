@@ -1,0 +1,156 @@
+"""Interfaces of the parts a layer is put together from.
+
+A part is built from its own sizes and constants only; it never sees the model
+configuration and does not know which model it is in.  Every part
+
+* declares the checkpoint tensors it binds, by name relative to its prefix
+  (``weight_specs``), which serves the loader's checks and the random-weights
+  writer alike;
+* takes them in ``load`` (where it may fuse or re-lay them for its kernels);
+* runs on device tensors with the step's ``StepContext``.
+
+Kinds of parts are registered by name (``register_mixer`` and friends) so that a
+model builder, or a test, can choose them layer by layer.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Callable, Dict, Optional, Tuple
+
+import torch
+
+
+@dataclasses.dataclass(frozen=True)
+class WeightSpec:
+    """One checkpoint tensor: its shape, and how the random-weights writer fills it.
+
+    ``init``: "linear" and "embedding" draw N(0, 0.02); "norm" is 1 (plus N(0, norm_jitter) on request);
+    "int_table" draws integers in [0, high).  Integer tables are kept as int32 on the device.
+    """
+    shape: Tuple[int, ...]
+    init: str = "linear"
+    high: int = 0
+
+    @property
+    def is_int(self) -> bool:
+        return self.init == "int_table"
+
+
+@dataclasses.dataclass(frozen=True)
+class CacheSpec:
+    """What a mixer keeps per token: keys and values of ``kv_heads`` heads of ``head_size``.
+
+    ``window``: None keeps every token; w keeps the last w.  Layers whose specs are equal share one
+    group of pages and one block table per request.
+    """
+    kv_heads: int
+    head_size: int
+    window: Optional[int] = None
+
+
+@dataclasses.dataclass(frozen=True)
+class StateSpec:
+    """Per-request state of fixed size that a mixer keeps: ``shape`` float32 numbers per request."""
+    shape: Tuple[int, ...]
+
+
+WeightGetter = Callable[[str], torch.Tensor]
+
+
+class Part:
+    """Base of all parts."""
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {}
+
+    def load(self, get: WeightGetter, device: torch.device, act_dtype: torch.dtype) -> None:
+        """Take the tensors named in ``weight_specs`` (``get(name)`` returns the CPU tensor as stored)."""
+
+    def device_bytes(self) -> int:
+        """Bytes of weights this part reads once per step (for the roofline)."""
+        return 0
+
+
+class Norm(Part):
+    def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
+                 ) -> torch.Tensor:
+        """``resid += delta`` (float32, in place; skipped when delta is None), return norm(resid) in the activation dtype.
+
+        With ``rows`` the sum and norm are taken at those rows only, ``resid`` stays unchanged and the result
+        has one row per entry of ``rows``.
+        """
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Encodes positions into queries and keys."""
+
+    def prepare(self, device: torch.device) -> None:
+        """Build device tables."""
+
+    def rotary_tables(self):
+        """(cos, sin, rotary_dim) float32 tables [positions, rotary_dim/2] if this encoding is a rotation of
+        half-split pairs, else None.  Mixers with a fused rotate-and-store kernel use them."""
+        return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
+        """Encode in place: q [T, heads, hd], k [T, kv_heads, hd], positions [T] int32."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request (attention here)."""
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        """x [T, width] in the activation dtype -> [T, width].  ``cache`` is this layer call's ``LayerCache``."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of norms, a mixer and a feed-forward around the residual stream."""
+
+    mixer: Mixer
+
+    def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], ctx, cache) -> torch.Tensor:
+        """Consume the pending ``delta`` into ``resid`` (float32 [T, width], in place) and return the new pending delta."""
+        raise NotImplementedError
+
+
+_KINDS: Dict[str, Dict[str, Callable]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}}
+
+
+def _register(family: str, name: str, factory: Callable, replace: bool):
+    table = _KINDS[family]
+    if name in table and not replace:
+        raise ValueError(f"{family} kind '{name}' is already registered")
+    table[name] = factory
+
+
+def register_mixer(name, factory, *, replace=False): _register("mixer", name, factory, replace)
+def register_feed_forward(name, factory, *, replace=False): _register("feed_forward", name, factory, replace)
+def register_norm(name, factory, *, replace=False): _register("norm", name, factory, replace)
+def register_position(name, factory, *, replace=False): _register("position", name, factory, replace)
+def register_block(name, factory, *, replace=False): _register("block", name, factory, replace)
+
+
+def make_part(family: str, kind: str, **params):
+    """Build a part of ``family`` ("mixer", "feed_forward", "norm", "position", "block") by its registered kind."""
+    table = _KINDS[family]
+    if kind not in table:
+        raise KeyError(f"unknown {family} kind '{kind}'; registered: {', '.join(sorted(table)) or 'none'}")
+    return table[kind](**params)
+
+
+def registered_kinds(family: str) -> Tuple[str, ...]:
+    return tuple(sorted(_KINDS[family]))

@@ -1,0 +1,40 @@
+"""Arrangements of parts around the residual stream.
+
+``PreNormBlock``: ``h = x + mixer(norm1(x))``, ``y = h + ffn(norm2(h))`` (models/src/llama.rs:393-410).  The residual
+stream is float32; each sum is fused with the norm that follows it, so a block receives the previous block's
+output as a pending ``delta`` and returns its own.
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+from .base import Block, FeedForward, Mixer, Norm, WeightSpec, register_block
+
+
+class PreNormBlock(Block):
+    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm, feed_forward: FeedForward,
+                 names=("input_layernorm", "self_attn", "post_attention_layernorm", "mlp")):
+        self.norm1, self.mixer, self.norm2, self.feed_forward = norm1, mixer, norm2, feed_forward
+        self.names = tuple(names)
+
+    def _children(self):
+        return zip(self.names, (self.norm1, self.mixer, self.norm2, self.feed_forward))
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {f"{n}.{k}": ws for n, part in self._children() for k, ws in part.weight_specs().items()}
+
+    def load(self, get, device, act_dtype) -> None:
+        for n, part in self._children():
+            part.load(lambda rel, _n=n: get(f"{_n}.{rel}"), device, act_dtype)
+
+    def device_bytes(self) -> int:
+        return sum(part.device_bytes() for _, part in self._children())
+
+    def forward(self, resid, delta, ctx, cache):
+        x = self.norm1.add_norm(resid, delta)
+        a = self.mixer.forward(x, ctx, cache)
+        x = self.norm2.add_norm(resid, a)
+        return self.feed_forward.forward(x, ctx)
+
+
+register_block("pre_norm", PreNormBlock)

@@ -1,0 +1,29 @@
+"""Matrix products ``x @ W^T`` with weights [out, in] as checkpoints store them.
+
+Which kernel runs is decided by the operands, never by the model:
+
+* any float32 operand -> the true float32 kernel (plain FMAs, no matrix-core mode);
+* bfloat16 x bfloat16 -> the hand-written MFMA kernels where their shape conditions hold (skinny products that
+  stream the weight once, and float32-output products for logits), the library product (hipBLASLt through
+  ``torch.matmul``, as the reference uses cuBLAS through candle for its linears: models/src/llama.rs:269-271,
+  311, 364-365) for large bfloat16-output products, and the float32 kernel for whatever is left.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [M, K] (row stride free) times w [N, K] transposed -> [M, N] in ``out_dtype`` (default: x's dtype)."""
+    out_dtype = out_dtype or x.dtype
+    if x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16:
+        from ..kernels import gemm_bf16
+        y = gemm_bf16.try_linear(x, w, out_dtype, out)
+        if y is not None:
+            return y
+    return ops.gemm_generic(x, w, out_dtype, out)

@@ -1,0 +1,201 @@
+"""The engine against the plain implementation: whole prompts, decoding, portions, mixed batches with few pages.
+
+Every schedule must give, for every (request, position), the logits of the plain float32 model run on the whole
+sequence: float32 within accumulation-order noise, bfloat16 within its rounding.
+"""
+import random
+
+import pytest
+import torch
+
+import plain_llama
+from util import (NORM_JITTER, TINY, TOL_BF16, TOL_F32, frob_err, make_model_dir, plain_config, plain_weights,
+                  random_tokens, rel_err)
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+PAGE = {"A": 4, "B": 16, "C": 16}
+
+
+@pytest.fixture(scope="module")
+def model_dirs(tmp_path_factory):
+    out = {}
+    for name, cfg in TINY.items():
+        # bfloat16 storage: both dtypes then compute from exactly the same numbers
+        out[name] = make_model_dir(str(tmp_path_factory.mktemp(f"tiny_{name}")), cfg, seed=11 + len(name),
+                                   dtype="bfloat16", norm_jitter=NORM_JITTER[name])
+    return out
+
+
+_plain_cache = {}
+
+
+def plain_logits(model_dir, tokens):
+    key = (model_dir, tuple(tokens))
+    if key not in _plain_cache:
+        _plain_cache[key] = plain_llama.forward(list(tokens), plain_weights(model_dir), plain_config(model_dir))
+    return _plain_cache[key]
+
+
+def make_runner(model_dir, dtype, page_size, num_pages, slots=8):
+    from atoma_infer_amd.cache import CachePool, plan_cache
+    from atoma_infer_amd.engine import ModelRunner
+    from atoma_infer_amd.models import load_model
+    model = load_model(model_dir, dtype)
+    plan = plan_cache(model.spec)
+    pool = CachePool(plan, page_size, [num_pages] * len(plan.groups), slots, model.act_dtype, model.device)
+    return ModelRunner(model, pool)
+
+
+def run_schedule(runner, requests, steps):
+    """``steps``: list of (entries, end); entries are (name, n_tokens).  Returns {(name, position): logits row}."""
+    from atoma_infer_amd.engine import StepEntry
+    ids, out = {}, {}
+    for entries, end in steps:
+        batch, places = [], []
+        for name, n in entries:
+            if name not in ids:
+                ids[name] = len(ids)
+                runner.add_request(ids[name])
+            start = runner.computed_len(ids[name])
+            toks = requests[name][start:start + n]
+            assert len(toks) == n, (name, start, n)
+            batch.append(StepEntry(ids[name], toks, start, list(range(n))))
+            places += [(name, start + i) for i in range(n)]
+        logits = runner.step(batch).cpu()
+        assert logits.shape[0] == len(places)
+        for row, key in enumerate(places):
+            out[key] = logits[row]
+        for name in end:
+            runner.free_request(ids[name])
+        runner.manager.check()
+    return out
+
+
+def check_against_plain(model_dir, requests, got, dtype):
+    worst = 0.0
+    for name, toks in requests.items():
+        rows = [p for (n, p) in got if n == name]
+        if not rows:
+            continue
+        want = plain_logits(model_dir, toks)
+        mine = torch.stack([got[(name, p)] for p in sorted(rows)])
+        ref = want[sorted(rows)]
+        if dtype == "float32":
+            err = rel_err(mine, ref)
+            assert err < TOL_F32, f"request {name}: float32 logits differ by {err:.3e} of the largest"
+        else:
+            err = frob_err(mine, ref)
+            assert err < TOL_BF16, f"request {name}: bfloat16 logits differ by {err:.3e} of the norm"
+            # row by row too, so that one bad position cannot hide among many good ones
+            for i, p in enumerate(sorted(rows)):
+                e = frob_err(mine[i], ref[i])
+                assert e < 2.5 * TOL_BF16, f"request {name} position {p}: {e:.3e}"
+        worst = max(worst, err)
+    return worst
+
+
+def lengths(name):
+    return {"A": [100, 37, 64, 5], "B": [200, 1, 77, 130], "C": [150, 48, 97, 16]}[name]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(TINY))
+def test_whole_prompts(model_dirs, name, dtype):
+    vocab = TINY[name]["vocab_size"]
+    requests = {f"r{i}": random_tokens(n, vocab, 100 + i) for i, n in enumerate(lengths(name))}
+    runner = make_runner(model_dirs[name], dtype, PAGE[name], 64)
+    steps = [([(r, len(t))], [r]) for r, t in requests.items()]
+    got = run_schedule(runner, requests, steps)
+    check_against_plain(model_dirs[name], requests, got, dtype)
+    assert runner.manager.num_free_pages(0) == 64
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(TINY))
+def test_last_32_one_by_one(model_dirs, name, dtype):
+    vocab = TINY[name]["vocab_size"]
+    n = lengths(name)[0]
+    requests = {"r": random_tokens(n, vocab, 7)}
+    runner = make_runner(model_dirs[name], dtype, PAGE[name], 64)
+    steps = [([("r", n - 32)], [])] + [([("r", 1)], []) for _ in range(32)]
+    got = run_schedule(runner, requests, steps)
+    assert len(got) == n
+    check_against_plain(model_dirs[name], requests, got, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(TINY))
+def test_portions_of_changing_size(model_dirs, name, dtype):
+    vocab = TINY[name]["vocab_size"]
+    n = lengths(name)[0]
+    requests = {"r": random_tokens(n, vocab, 8)}
+    runner = make_runner(model_dirs[name], dtype, PAGE[name], 64)
+    sizes, left, cycle = [], n, [17, 2, 31, 3, 16, 2, 5, 33, 1, 4]
+    i = 0
+    while left:
+        s = min(cycle[i % len(cycle)], left)
+        sizes.append(s)
+        left -= s
+        i += 1
+    got = run_schedule(runner, requests, [([("r", s)], []) for s in sizes])
+    check_against_plain(model_dirs[name], requests, got, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(TINY))
+def test_mixed_batches_with_few_pages(model_dirs, name, dtype):
+    """Up to four live requests, portions of some beside decoded tokens of others; the pool is so small that
+    pages freed by finished requests are used again at once."""
+    vocab = TINY[name]["vocab_size"]
+    lens = {"A": [60, 33, 47, 21, 58, 40, 9, 52], "B": [120, 1, 77, 90, 45, 130, 18, 66],
+            "C": [90, 48, 97, 16, 70, 33, 80, 25]}[name]
+    requests = {f"r{i}": random_tokens(n, vocab, 300 + i) for i, n in enumerate(lens)}
+    page = PAGE[name]
+    rng = random.Random(5)
+    # pool: what the four longest need at once, nothing more
+    need = sum(sorted(-(-n // page) for n in lens)[-4:])
+    runner = make_runner(model_dirs[name], dtype, page, need, slots=4)
+    waiting = list(requests)
+    live, done_tokens, steps = [], {r: 0 for r in requests}, []
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            left = len(requests[r]) - done_tokens[r]
+            # the last 8 tokens of every request are "decoded" one at a time; before that portions of 2..24
+            if left <= 8:
+                n = 1
+            else:
+                n = min(rng.choice([2, 3, 5, 8, 13, 24]), left - 8)
+            if rng.random() < 0.15 and len(live) > 1:
+                continue  # a request may sit out a step
+            entries.append((r, n))
+            done_tokens[r] += n
+            if done_tokens[r] == len(requests[r]):
+                end.append(r)
+        if not entries:
+            continue
+        rng.shuffle(entries)
+        steps.append((entries, end))
+        live = [r for r in live if r not in end]
+    got = run_schedule(runner, requests, steps)
+    assert len(got) == sum(lens)
+    check_against_plain(model_dirs[name], requests, got, dtype)
+    assert runner.manager.num_free_pages(0) == need and runner.manager.num_requests() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_first_tokens_and_long_decoding(model_dirs, dtype):
+    """A one-token prompt, then everything decoded token by token up to the model's last position."""
+    name = "A"
+    vocab, n = TINY[name]["vocab_size"], TINY[name]["max_position_embeddings"]
+    requests = {"r": random_tokens(n, vocab, 9)}
+    runner = make_runner(model_dirs[name], dtype, PAGE[name], 40)
+    got = run_schedule(runner, requests, [([("r", 1)], []) for _ in range(n)])
+    check_against_plain(model_dirs[name], requests, got, dtype)
+    from atoma_infer_amd.engine import StepEntry, StepError
+    with pytest.raises(StepError):
+        runner.step([StepEntry(0, [1], n, [0])])  # beyond max_position_embeddings

@@ -1,0 +1,75 @@
+"""Shared pieces of the tests: the tiny configurations, model folders with random weights, comparisons."""
+from __future__ import annotations
+
+import json
+import os
+from typing import Dict, List
+
+import torch
+
+# Two tiny configurations that differ in every size and option: layers, width, heads, KV heads (one shared head
+# against no grouping), head size, feed-forward width, vocabulary (none a power of two in B), eps, theta,
+# scaling (none against llama3 with all three branches hit), tied against untied head.
+TINY_A = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 64, "intermediate_size": 160, "vocab_size": 512, "num_hidden_layers": 2,
+    "num_attention_heads": 4, "num_key_value_heads": 1, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
+    "max_position_embeddings": 128, "tie_word_embeddings": True, "eos_token_id": 2,
+}
+TINY_B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 96, "intermediate_size": 256, "vocab_size": 1000, "num_hidden_layers": 3,
+    "num_attention_heads": 3, "num_key_value_heads": 3, "rms_norm_eps": 1e-6, "rope_theta": 500000.0,
+    "rope_scaling": {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 64, "rope_type": "llama3"},
+    "max_position_embeddings": 256, "tie_word_embeddings": False, "eos_token_id": [1, 7],
+}
+# a third shape: grouped heads (2 per KV head), head size 48 (a multiple of 16 that is no power of two)
+TINY_C = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 192, "intermediate_size": 150, "vocab_size": 331, "num_hidden_layers": 2,
+    "num_attention_heads": 4, "num_key_value_heads": 2, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
+    "max_position_embeddings": 512, "tie_word_embeddings": True,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+NORM_JITTER = {"A": 0.0, "B": 0.1, "C": 0.1}
+
+
+def make_model_dir(path: str, cfg: dict, seed: int, dtype: str, norm_jitter: float = 0.0) -> str:
+    from atoma_infer_amd.weights import write_random_model
+    return write_random_model(path, cfg, seed=seed, dtype=dtype, norm_jitter=norm_jitter)
+
+
+def plain_weights(model_dir: str) -> Dict[str, torch.Tensor]:
+    """The checkpoint as float32 CPU tensors, read with the safetensors package (not with the framework's reader)."""
+    from safetensors.torch import load_file
+    return {k: v.to(torch.float32) for k, v in load_file(os.path.join(model_dir, "model.safetensors")).items()}
+
+
+def plain_config(model_dir: str) -> dict:
+    with open(os.path.join(model_dir, "config.json")) as f:
+        return json.load(f)
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """Largest absolute difference relative to the largest wanted magnitude."""
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+def frob_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).norm() / want.norm().clamp_min(1e-30))
+
+
+# Tolerances, fixed before the first run.  float32: every value is a sum of at most a few thousand float32
+# products whose order differs between the engine and the yardstick; 2e-5 of the largest logit covers that with
+# room and is far below any real fault.  bfloat16: activations are rounded to 8 bits of mantissa (relative
+# 2^-9) about eight times a layer; for at most 16 layers the errors add up to about 1e-2 of the logits' norm.
+TOL_F32 = 2e-5
+TOL_BF16 = 2e-2
+
+
+def random_tokens(n: int, vocab: int, seed: int) -> List[int]:
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
