@@ -32,13 +32,15 @@ extern "C" int atoma_embed(const int32_t* tokens, const void* table, int table_d
 
 // ---------------------------------------------------------------------------------------------
 // resid += delta; out = resid * rsqrt(mean(resid^2) + eps) * w.
-// One block per row.  With `rows`, block r reads row rows[r], leaves resid untouched and writes out row r.
+// delta may come as several planes [planes][rows][width] (the slices of a K-split product); they are added in
+// order of their index.  One block per row.  With `rows`, block r reads row rows[r], leaves resid untouched and writes out row r.
 // The sum of squares is reduced in an order fixed by (width, block size) alone.
 // Reference: models/src/llama.rs:401-408 (norm placement and residual sums), :416-421 (eps).
 template <typename TD, typename TW, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
                                    const TW* __restrict__ w, TO* __restrict__ out,
-                                   const int32_t* __restrict__ rows, int width, float eps) {
+                                   const int32_t* __restrict__ rows, int width, float eps, int planes,
+                                   size_t plane_stride) {
   __shared__ float scratch[4];
   const int r = blockIdx.x;
   const size_t src = (size_t)(rows ? rows[r] : r) * width, dst = (size_t)r * width;
@@ -46,7 +48,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   for (int i = threadIdx.x; i < width; i += 256) {
     float v = resid[src + i];
     if (delta) {
-      v += to_f32(delta[src + i]);
+      for (int p = 0; p < planes; ++p) v += to_f32(delta[p * plane_stride + src + i]);
       if (!rows) resid[src + i] = v;
     }
     ss += v * v;
@@ -55,21 +57,23 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
   for (int i = threadIdx.x; i < width; i += 256) {
     float v = resid[src + i];
-    if (delta && rows) v += to_f32(delta[src + i]);
+    if (delta && rows)
+      for (int p = 0; p < planes; ++p) v += to_f32(delta[p * plane_stride + src + i]);
     out[dst + i] = from_f32<TO>(v * inv * to_f32(w[i]));
   }
 }
 
 template <typename TD, typename TW>
 static int add_rmsnorm_out(float* resid, const TD* delta, const TW* w, void* out, int out_dtype, const int32_t* rows,
-                           int n_rows, int width, float eps, hipStream_t stream) {
+                           int n_rows, int width, float eps, int planes, size_t plane_stride,
+                           hipStream_t stream) {
   dim3 grid(n_rows), block(256);
   if (out_dtype == kF32)
     hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, float>), grid, block, 0, stream, resid, delta, w, (float*)out,
-                       rows, width, eps);
+                       rows, width, eps, planes, plane_stride);
   else if (out_dtype == kBF16)
     hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, bf16_t>), grid, block, 0, stream, resid, delta, w,
-                       (bf16_t*)out, rows, width, eps);
+                       (bf16_t*)out, rows, width, eps, planes, plane_stride);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();
@@ -78,25 +82,26 @@ static int add_rmsnorm_out(float* resid, const TD* delta, const TW* w, void* out
 
 template <typename TD>
 static int add_rmsnorm_w(float* resid, const TD* delta, const void* w, int w_dtype, void* out, int out_dtype,
-                         const int32_t* rows, int n_rows, int width, float eps, hipStream_t stream) {
+                         const int32_t* rows, int n_rows, int width, float eps, int planes, size_t plane_stride,
+                           hipStream_t stream) {
   if (w_dtype == kF32)
-    return add_rmsnorm_out<TD, float>(resid, delta, (const float*)w, out, out_dtype, rows, n_rows, width, eps, stream);
+    return add_rmsnorm_out<TD, float>(resid, delta, (const float*)w, out, out_dtype, rows, n_rows, width, eps, planes, plane_stride, stream);
   if (w_dtype == kBF16)
     return add_rmsnorm_out<TD, bf16_t>(resid, delta, (const bf16_t*)w, out, out_dtype, rows, n_rows, width, eps,
-                                       stream);
+                                       planes, plane_stride, stream);
   return ATOMA_ERR_DTYPE;
 }
 
 extern "C" int atoma_add_rmsnorm(float* resid, const void* delta, int delta_dtype, const void* w, int w_dtype,
                                  void* out, int out_dtype, const int32_t* rows, int n_rows, int width, float eps,
-                                 hipStream_t stream) {
+                                 int planes, size_t plane_stride, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (delta_dtype == kF32)
     return add_rmsnorm_w<float>(resid, (const float*)delta, w, w_dtype, out, out_dtype, rows, n_rows, width, eps,
-                                stream);
+                                planes, plane_stride, stream);
   if (delta_dtype == kBF16)
     return add_rmsnorm_w<bf16_t>(resid, (const bf16_t*)delta, w, w_dtype, out, out_dtype, rows, n_rows, width, eps,
-                                 stream);
+                                 planes, plane_stride, stream);
   return ATOMA_ERR_DTYPE;
 }
 

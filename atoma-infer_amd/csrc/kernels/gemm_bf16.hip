@@ -1,0 +1,173 @@
+// bfloat16 x bfloat16 products on the matrix cores for few rows of activations (decode and short portions):
+// C[M, N] = A[M, K] * W[N, K]^T with float32 accumulation, W streamed from HBM once.
+//
+// The product is bound by the bytes of W.  A wave owns RT tiles of 16 rows of W and multiplies them against up to
+// MT tiles of 16 rows of A with v_mfma_f32_16x16x32_bf16: the W tile is the MFMA's A operand (lane l: row l%16,
+// eight consecutive k at (l/16)*8), the activations its B operand (lane l: row of A l%16, the same eight k), so
+// both are 16-byte loads straight from global memory and nothing passes through LDS on the way in.
+// The four waves of a workgroup either take different rows of W (WK = 1) or split K four ways for the same rows
+// and add their accumulators in LDS (WK = 4), which keeps enough workgroups in flight when N is small.
+// K can additionally be split across blockIdx.y; then each slice writes its own float32 plane
+// C[slice][M][N] and the consumer adds the planes (the fused residual-add + RMSNorm kernel does).
+// Each output's sum order depends only on (K, WK, slices), never on M or on the row's place in the batch.
+//
+// Needs K % (32 * WK * slices) == 0 and 16-byte aligned rows; the host wrapper checks and otherwise refuses.
+#include "common.h"
+
+using namespace atoma;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+template <int MT, int RT, int WK, typename TC>
+__global__ void __launch_bounds__(256)
+gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
+                   int K, int lda, int ldw, int ldc, size_t plane) {
+  constexpr int WN = 4 / WK;  // waves along N
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wn = wave % WN, wk = wave / WN;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int n_base = (blockIdx.x * WN + wn) * (RT * 16);
+  const int k_slices = gridDim.y * WK;
+  const int k_len = K / k_slices;
+  const int k_begin = (blockIdx.y * WK + wk) * k_len;
+
+  // row pointers; rows past the end are clamped to the last valid row and never stored
+  const uint16_t* wp[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    int n = n_base + r * 16 + r16;
+    if (n > N - 1) n = N - 1;
+    wp[r] = w + (size_t)n * ldw + k_begin + kg * 8;
+  }
+  const uint16_t* ap[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    int row = m * 16 + r16;
+    if (row > M - 1) row = M - 1;
+    ap[m] = a + (size_t)row * lda + k_begin + kg * 8;
+  }
+
+  f32x4 acc[RT][MT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[r][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll 4
+  for (int k = 0; k < k_len; k += 32) {
+    bf16x8 wf[RT], af[MT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) wf[r] = *reinterpret_cast<const bf16x8*>(wp[r] + k);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) af[m] = *reinterpret_cast<const bf16x8*>(ap[m] + k);
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+        acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[r], af[m], acc[r][m], 0, 0, 0);
+  }
+
+  if constexpr (WK > 1) {
+    // add the WK partial accumulators of the same rows: wave wk > 0 writes, wave wk == 0 sums in fixed order
+    __shared__ float red[(WK - 1) * WN * RT * MT * 4 * 64];
+    constexpr int per_wave = RT * MT * 4 * 64;
+    if (wk > 0) {
+      float* dst = red + ((wk - 1) * WN + wn) * per_wave;
+#pragma unroll
+      for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[((r * MT + m) * 4 + i) * 64 + lane] = acc[r][m][i];
+    }
+    __syncthreads();
+    if (wk > 0) return;
+#pragma unroll
+    for (int s = 0; s < WK - 1; ++s) {
+      const float* src = red + (s * WN + wn) * per_wave;
+#pragma unroll
+      for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[r][m][i] += src[((r * MT + m) * 4 + i) * 64 + lane];
+    }
+  }
+
+  // D[n = kg*4 + i][row of A = r16]: four consecutive columns of C per lane
+  TC* cp = c + (size_t)blockIdx.y * plane;
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int n0 = n_base + r * 16 + kg * 4;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const int row = m * 16 + r16;
+      if (row >= M) continue;
+      TC* dst = cp + (size_t)row * ldc + n0;
+      if (n0 + 3 < N && (ldc & 3) == 0) {
+        if (sizeof(TC) == 4) {
+          *reinterpret_cast<f32x4*>(dst) = acc[r][m];
+        } else {
+          uint2 v;
+          v.x = (uint32_t)f32_to_bf16_bits(acc[r][m][0]) | ((uint32_t)f32_to_bf16_bits(acc[r][m][1]) << 16);
+          v.y = (uint32_t)f32_to_bf16_bits(acc[r][m][2]) | ((uint32_t)f32_to_bf16_bits(acc[r][m][3]) << 16);
+          *reinterpret_cast<uint2*>(dst) = v;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n0 + i < N) dst[i] = from_f32<TC>(acc[r][m][i]);
+      }
+    }
+  }
+}
+
+template <int MT, int RT, int WK>
+static int launch(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc,
+                  int slices, hipStream_t stream) {
+  constexpr int WN = 4 / WK;
+  dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), slices), block(256);
+  const size_t plane = (size_t)M * ldc;
+  if (c_dtype == kF32)
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WK, float>), grid, block, 0, stream, (const uint16_t*)a,
+                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane);
+  else if (c_dtype == kBF16)
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WK, bf16_t>), grid, block, 0, stream, (const uint16_t*)a,
+                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane);
+  else
+    return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int MT>
+static int launch_mt(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, int lda, int ldw,
+                     int ldc, int rt, int wk, int slices, hipStream_t stream) {
+#define ATOMA_CASE(R, W_)                                                                                   \
+  if (rt == R && wk == W_) return launch<MT, R, W_>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, slices, stream)
+  ATOMA_CASE(1, 1);
+  ATOMA_CASE(2, 1);
+  ATOMA_CASE(4, 1);
+  ATOMA_CASE(1, 4);
+  ATOMA_CASE(2, 4);
+#undef ATOMA_CASE
+  return ATOMA_ERR_SHAPE;
+}
+
+// a [M <= 64, K] bf16, w [N, K] bf16 -> c [slices][M, N] (bf16 only with slices == 1, or float32).
+// rt: tiles of 16 rows of W per wave (1, 2, 4); wk: 1 or 4 (waves split K); slices: K split across the grid.
+extern "C" int atoma_gemm_bf16_skinny(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
+                                      int lda, int ldw, int ldc, int rt, int wk, int slices, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || slices <= 0 || K % (32 * wk * slices) || (lda & 7) || (ldw & 7) || lda < K || ldw < K ||
+      ldc < N || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || (slices > 1 && c_dtype != kF32) || slices > 65535)
+    return ATOMA_ERR_SHAPE;
+  const int mt = (M + 15) / 16;
+  switch (mt) {
+    case 1: return launch_mt<1>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
+    case 2: return launch_mt<2>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
+    case 3: return launch_mt<3>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
+    default: return launch_mt<4>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
+  }
+}

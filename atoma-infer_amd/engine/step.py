@@ -81,6 +81,29 @@ class _Staging:
         return self.host.numpy()
 
 
+class RunnerCache:
+    """The cache manager as the scheduler sees it, with the runner's own books kept in step.
+
+    Same methods as ``CacheManager`` (has, add, free, can_reserve, reserve, fits_at_all, num_free_slots,
+    num_free_pages), so the scheduler runs against either.
+    """
+
+    def __init__(self, runner: "ModelRunner"):
+        self._runner, self._mgr = runner, runner.manager
+
+    def has(self, request: int) -> bool:
+        return self._runner.has_request(request)
+
+    def add(self, request: int) -> int:
+        return self._runner.add_request(request)
+
+    def free(self, request: int) -> None:
+        self._runner.free_request(request)
+
+    def __getattr__(self, name):
+        return getattr(self._mgr, name)
+
+
 class ModelRunner:
     """Owns the model and the cache pool of one GPU and steps batches through them."""
 

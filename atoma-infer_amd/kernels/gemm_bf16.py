@@ -1,12 +1,106 @@
-"""bfloat16 x bfloat16 products on the matrix cores."""
+"""bfloat16 x bfloat16 products on the matrix cores.
+
+``try_linear`` picks, for x [M, K] and w [N, K]:
+
+* the hand-written weight-streaming MFMA kernel when M is small (decode steps, short portions) or when float32
+  output is wanted (logits), running it over blocks of 64 rows of x;
+* the library product (hipBLASLt through ``torch.mm``) for large bfloat16-output products, as the reference uses
+  a library for its linears;
+* nothing (None) when the shape fits neither: the caller then runs the float32 FMA kernel.
+"""
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
 import torch
+
+from .library import load_hip_module
+from .ops import BF16, F32, KernelError, _check, _p, _stream
+
+SKINNY_MAX_M = 64
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = load_hip_module("gemm_bf16")
+    return _lib
+
+
+def _aligned(t: torch.Tensor) -> bool:
+    return t.data_ptr() % 16 == 0 and (t.shape[0] == 1 or t.stride(0) % 8 == 0) and t.stride(1) == 1
+
+
+def _plan(n: int, k: int, allow_slices: bool):
+    """(rows-of-16 per wave, waves splitting K, K slices over the grid) for a product with N outputs."""
+    tiles = -(-n // 16)
+    if tiles >= 4096:
+        rt, wk = 4, 1
+    elif tiles >= 2048:
+        rt, wk = 2, 1
+    elif tiles >= 512:
+        rt, wk = 2, 4
+    else:
+        rt, wk = 1, 4
+    if k % (32 * wk):
+        wk = 1
+    slices = 1
+    if allow_slices:
+        groups = -(-tiles // ((4 // wk) * rt))
+        slices = max(1, min(8, 256 // max(groups, 1)))
+        while slices > 1 and (k % (32 * wk * slices) or k // (wk * slices) < 256):
+            slices -= 1
+    return rt, wk, slices
+
+
+def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16 and x.dim() == 2 and w.dim() == 2
+            and x.shape[1] == w.shape[1] and x.shape[1] % 32 == 0 and _aligned(x) and _aligned(w))
+
+
+def skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, slices: int = 1, rt: int = 0, wk: int = 0) -> None:
+    """out [M, N] (or [slices, M, N] float32 planes) = x [M <= 64, K] @ w [N, K]^T."""
+    m, k = x.shape
+    n = w.shape[0]
+    if not rt:
+        rt, wk, _ = _plan(n, k, False)
+        if k % (32 * wk * slices):
+            wk = 1
+    ldc = out.stride(-2) if m > 1 else n
+    code = {torch.float32: F32, torch.bfloat16: BF16}[out.dtype]
+    _check(lib().atoma_gemm_bf16_skinny(_p(x), _p(w), _p(out), code, m, n, k, x.stride(0) if m > 1 else k,
+                                        w.stride(0) if n > 1 else k, ldc, rt, wk, slices, _stream()),
+           "gemm_bf16_skinny")
 
 
 def try_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None,
                ) -> Optional[torch.Tensor]:
     """x [M, K] @ w [N, K]^T if a fast kernel takes the shape, else None (the caller falls back to float32 FMAs)."""
+    m, n = x.shape[0], w.shape[0]
+    ok = skinny_ok(x, w)
+    if ok and (m <= SKINNY_MAX_M or out_dtype is torch.float32):
+        if out is None:
+            out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        for lo in range(0, m, SKINNY_MAX_M):
+            hi = min(lo + SKINNY_MAX_M, m)
+            skinny(x[lo:hi], w, out[lo:hi])
+        return out
+    if out_dtype is torch.bfloat16 and m > SKINNY_MAX_M:
+        if out is None:
+            return torch.mm(x, w.t())
+        return torch.mm(x, w.t(), out=out)
     return None
+
+
+def linear_planes(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
+    """For M <= 64: float32 planes [slices, M, N] whose sum is x @ w^T (K split over the grid), else None."""
+    m, k = x.shape
+    n = w.shape[0]
+    if m > SKINNY_MAX_M or not skinny_ok(x, w):
+        return None
+    rt, wk, slices = _plan(n, k, True)
+    out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+    skinny(x, w, out, slices, rt, wk)
+    return out

@@ -43,6 +43,7 @@ class KernelBuildError(RuntimeError):
 # name -> (sources relative to csrc/kernels, fixed definitions)
 HIP_MODULES: Dict[str, Tuple[Sequence[str], Sequence[str]]] = {
     "core": (("elementwise.hip", "attention_generic.hip", "gemm_generic.hip", "sampling.hip"), ()),
+    "gemm_bf16": (("gemm_bf16.hip",), ()),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

@@ -102,8 +102,13 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     _need(resid.dtype is torch.float32 and resid.dim() == 2 and resid.is_contiguous(), "resid must be float32 [T, W]")
     t, width = resid.shape
     _need(weight.is_contiguous() and weight.numel() == width, "norm weight must have one entry per column")
+    planes, plane_stride = 1, 0
     if delta is not None:
-        _need(delta.is_contiguous() and tuple(delta.shape) == (t, width), "delta must match resid")
+        if delta.dim() == 3:  # planes of a K-split product, summed here
+            planes, plane_stride = delta.shape[0], t * width
+            _need(delta.is_contiguous() and tuple(delta.shape[1:]) == (t, width), "delta planes must match resid")
+        else:
+            _need(delta.is_contiguous() and tuple(delta.shape) == (t, width), "delta must match resid")
     n = t
     if rows is not None:
         _i32(rows, "rows")
@@ -113,7 +118,8 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     _need(out.is_contiguous() and tuple(out.shape) == (n, width) and out.dtype is out_dtype, "add_rmsnorm: bad out")
     _check(core().atoma_add_rmsnorm(_p(resid), _p(delta), _code(delta, "delta") if delta is not None else F32,
                                     _p(weight), _code(weight, "norm weight"), _p(out), _code(out, "out"), _p(rows),
-                                    n, width, ctypes.c_float(eps), _stream()), "add_rmsnorm")
+                                    n, width, ctypes.c_float(eps), planes, ctypes.c_size_t(plane_stride),
+                                    _stream()), "add_rmsnorm")
     return out
 
 

@@ -13,7 +13,7 @@ import torch
 
 from ..config.base import ModelConfig
 from ..config.registry import Architecture, load_model_config
-from ..weights.loader import load_into
+from ..weights.loader import load_into, load_random_into
 from .spec import ModelSpec
 
 _ACT = {"bfloat16": torch.bfloat16, "float32": torch.float32}
@@ -62,4 +62,22 @@ def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") 
     arch, cfg = load_model_config(model_dir)
     spec = arch.build(cfg)
     load_into(spec, model_dir, dev, _ACT[dtype])
+    return Model(arch, cfg, spec, dev, _ACT[dtype])
+
+
+def random_model(config, seed: int = 0, dtype: str = "bfloat16", stored: str = "bfloat16", device: str = "cuda:0",
+                 norm_jitter: float = 0.0) -> Model:
+    """A model with the weights that the random-weights mode would write for (config, seed), built without files.
+
+    ``config`` is a typed configuration or the JSON object of a config.json.
+    """
+    from ..config.registry import resolve_architecture
+    obj = config.to_dict() if isinstance(config, ModelConfig) else dict(config)
+    arch = resolve_architecture(obj)
+    cfg = arch.config_cls.from_dict(obj)
+    dev = torch.device(device)
+    if dev.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError("this engine runs on a GPU only (device 'cuda:N'); no GPU is visible")
+    spec = arch.build(cfg)
+    load_random_into(spec, seed, _ACT[stored], dev, _ACT[dtype], norm_jitter)
     return Model(arch, cfg, spec, dev, _ACT[dtype])

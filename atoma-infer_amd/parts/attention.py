@@ -19,7 +19,7 @@ import torch
 
 from ..kernels import ops
 from .base import CacheSpec, Mixer, PositionEncoding, WeightSpec, register_mixer
-from .linear import linear
+from .linear import linear, linear_delta
 
 
 class PagedAttention(Mixer):
@@ -90,7 +90,7 @@ class PagedAttention(Mixer):
                 self.position.apply(q, q[:, :0], ctx.positions)
         out = torch.empty((t, nh * hd), dtype=qkv.dtype, device=qkv.device)
         self.attend(qkv, k_cache, v_cache, out, ctx, cache)
-        return linear(out, self.w_o)
+        return linear_delta(out, self.w_o)
 
     def attend(self, q, k_cache, v_cache, out, ctx, cache) -> None:
         if q.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16:

@@ -10,7 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, WeightSpec, register_feed_forward
-from .linear import linear
+from .linear import linear, linear_delta
 
 
 class SwiGLU(FeedForward):
@@ -34,7 +34,7 @@ class SwiGLU(FeedForward):
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        return linear(ops.swiglu(linear(x, self.w_gate_up)), self.w_down)
+        return linear_delta(ops.swiglu(linear(x, self.w_gate_up)), self.w_down)
 
 
 register_feed_forward("swiglu", SwiGLU)

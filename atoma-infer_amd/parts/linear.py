@@ -27,3 +27,17 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         if y is not None:
             return y
     return ops.gemm_generic(x, w, out_dtype, out)
+
+
+def linear_delta(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """A product whose result is only ever added to the residual stream by ``Norm.add_norm``.
+
+    For few rows it comes back as float32 planes [slices, M, N] of a K-split product, which ``add_norm`` sums:
+    the split keeps the whole GPU busy on a small product and costs no extra kernel.
+    """
+    if x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16:
+        from ..kernels import gemm_bf16
+        y = gemm_bf16.linear_planes(x, w)
+        if y is not None:
+            return y
+    return linear(x, w)

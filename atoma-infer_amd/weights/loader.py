@@ -147,3 +147,15 @@ def load_into(spec, model_dir: str, device: torch.device, act_dtype: torch.dtype
             part.load(get, device, act_dtype)
     finally:
         ckpt.close()
+
+
+def load_random_into(spec, seed: int, stored: torch.dtype, device: torch.device, act_dtype: torch.dtype,
+                     norm_jitter: float = 0.0) -> None:
+    """Give every part the tensors that ``write_random_model`` would have stored, without a file."""
+    from .random_init import random_tensor
+    want = expected_tensors(spec)
+    for prefix, part in spec.parts():
+        def get(rel: str, _p=prefix) -> torch.Tensor:
+            name = f"{_p}.{rel}" if _p else rel
+            return random_tensor(name, want[name], seed, stored, norm_jitter)
+        part.load(get, device, act_dtype)
