@@ -145,8 +145,9 @@ def _compile(name: str, compiler: str, sources: Sequence[str], flags: Sequence[s
 
 def _module_plan(name: str, sources: Sequence[str], defines: Sequence[str]):
     paths = [os.path.join(_KERNELS, s) for s in sources]
-    flags = HIP_FLAGS + [f"-D{d}" for d in defines] + ["-I" + _KERNELS]
-    return paths, flags, _hash(paths, flags)
+    flags = HIP_FLAGS + [f"-D{d}" for d in defines]
+    # the include path is left out of the hash: it differs between checkouts of the same sources
+    return paths, flags + ["-I" + _KERNELS], _hash(paths, flags)
 
 
 def load_hip_module(name: str, sources: Optional[Sequence[str]] = None, defines: Sequence[str] = (),

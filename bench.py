@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at Llama-3.2-1B sizes with random weights, on one GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 16]
+
+A "step" is one decode step of the whole engine (scheduler, step function, sampler).  The default run has the
+layer sizes of Llama-3.2-1B (16 layers, width 2048, 32 heads over 8 KV heads of 64, feed-forward 8192, vocabulary
+128256, llama3 rope scaling, tied head), bfloat16, random weights N(0, 0.02), 2048-token prompts of uniform random
+token ids, a batch of 8, and a maximum context of 8192.  It prints ONE JSON line: decoded tokens a second as
+``value``, plus the 2048-token prefill, the decode step's roofline fraction (bytes it has to read / time / 8 TB/s)
+and decode throughput at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+LLAMA_1B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 2048, "intermediate_size": 8192, "vocab_size": 128256, "num_hidden_layers": 16,
+    "num_attention_heads": 32, "num_key_value_heads": 8, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192, "rope_type": "llama3"},
+    "max_position_embeddings": 131072, "tie_word_embeddings": True,
+}
+FULL_LAYERS = 16
+
+
+def log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def make_engine(model, batch, context, page=16):
+    from atoma_infer_amd.config import CacheConfig, SchedulerConfig, ValidationConfig
+    from atoma_infer_amd.engine.engine import LlmEngine
+    pages = batch * (-(-context // page)) + 8
+    return LlmEngine(model, cache=CacheConfig(block_size=page, num_gpu_blocks_override=pages),
+                     scheduler=SchedulerConfig(max_num_batched_tokens=max(2048, batch), max_num_sequences=max(batch, 1),
+                                               max_model_len=context, enable_chunked_prefill=True),
+                     validation=ValidationConfig(max_input_length=context - 1, max_total_tokens=context))
+
+
+def decode_run(model, batch, prompt_len, steps, warmup, context, seed=0):
+    """Prefill ``batch`` prompts (untimed), then time ``steps`` decode steps.  Returns (seconds, mean context)."""
+    import torch
+    from atoma_infer_amd.sampling import GenerateParameters
+    eng = make_engine(model, batch, context)
+    g = torch.Generator().manual_seed(seed)
+    vocab = model.vocab_size
+    params = GenerateParameters(do_sample=False, max_new_tokens=steps + warmup + batch + 8, ignore_eos_token=True)
+    for _ in range(batch):
+        eng.add_request(torch.randint(0, vocab, (prompt_len,), generator=g).tolist(), params)
+    while any(r.in_prefill for r in eng.scheduler.running) or eng.scheduler.waiting:
+        eng.step()
+    for _ in range(warmup):
+        eng.step()
+    ctx0 = sum(r.length for r in eng.scheduler.running)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        eng.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx1 = sum(r.length for r in eng.scheduler.running)
+    assert len(eng.scheduler.running) == batch, "a request ended or was preempted during the timed steps"
+    mean_ctx = (ctx0 + ctx1) / 2.0 / batch
+    del eng
+    torch.cuda.empty_cache()
+    return dt, mean_ctx
+
+
+def prefill_run(model, n_tokens, reps, context):
+    import torch
+    from atoma_infer_amd.cache import CachePool, plan_cache
+    from atoma_infer_amd.engine import ModelRunner, StepEntry
+    plan = plan_cache(model.spec)
+    pool = CachePool(plan, 16, [(-(-n_tokens // 16)) + 4] * len(plan.groups), 4, model.act_dtype, model.device)
+    runner = ModelRunner(model, pool)
+    g = torch.Generator().manual_seed(1)
+    toks = torch.randint(0, model.vocab_size, (n_tokens,), generator=g).tolist()
+    times = []
+    for i in range(reps + 1):
+        runner.add_request(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step([StepEntry(i, toks, 0, [n_tokens - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        runner.free_request(i)
+    del runner, pool
+    torch.cuda.empty_cache()
+    return min(times[1:])
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 runs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
+        return 2
+    if int(os.environ.get("WORLD_SIZE", "1")) > 1:
+        print("bench.py: started with WORLD_SIZE > 1; this engine runs on one GPU", flush=True)
+        return 2
+    if args.prompt_len + args.steps + args.warmup + 72 > args.context:
+        print("bench.py: prompt + steps exceed the context", file=sys.stderr)
+        return 1
+
+    import torch
+    import atoma_infer_amd  # noqa: F401
+    from atoma_infer_amd.cache import plan_cache
+    from atoma_infer_amd.models import random_model
+
+    cfg = dict(LLAMA_1B, num_hidden_layers=args.layers)
+    log(f"building the model ({args.layers} layers, random weights) ...")
+    t0 = time.time()
+    model = random_model(cfg, seed=0, dtype="bfloat16", stored="bfloat16")
+    log(f"model ready in {time.time() - t0:.1f} s; weights read per step: {model.weight_bytes() / 1e6:.1f} MB")
+    kv_bytes_per_token = plan_cache(model.spec).bytes_per_token(2)
+
+    log(f"prefill of {args.prefill_tokens} tokens ...")
+    pre_s = prefill_run(model, args.prefill_tokens, 3, args.context)
+    c = model.config
+    hd = c.head_size
+    layer_params = (c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * hd
+                    + c.num_attention_heads * hd * c.hidden_size + 3 * c.hidden_size * c.intermediate_size)
+    t = args.prefill_tokens
+    pre_flops = (2.0 * t * layer_params * c.num_hidden_layers
+                 + 4.0 * (t * (t + 1) / 2.0) * hd * c.num_attention_heads * c.num_hidden_layers
+                 + 2.0 * c.hidden_size * c.vocab_size)
+    prefill = {"value": round(t / pre_s, 1), "tokens": t, "ms": round(pre_s * 1e3, 3),
+               "frac": round(pre_flops / pre_s / PEAK_FLOPS["bf16"], 4)}
+
+    log(f"decode at batch {args.batch}: {args.warmup} warm-up + {args.steps} timed steps ...")
+    dt, mean_ctx = decode_run(model, args.batch, args.prompt_len, args.steps, args.warmup, args.context)
+    ms_per_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    step_bytes = model.weight_bytes() + kv_bytes_per_token * mean_ctx * args.batch
+    achieved = step_bytes / (dt / args.steps) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4)}
+
+    points = {}
+    if not args.no_points:
+        for b, st in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
+            log(f"decode at batch {b} ...")
+            d, _ = decode_run(model, b, args.prompt_len, st, min(args.warmup, 4), args.context)
+            points[f"decode_b{b}"] = round(b * st / d, 1)
+
+    line = {
+        "metric": "decode tok/s at batch 8 (Llama-3.2-1B sizes, 2048-token prompts); points: batch 1 and 64; "
+                  "prefill tok/s at 2048 tokens",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (uniform random token ids, random weights N(0, 0.02))",
+        "config": {"model": "Llama-3.2-1B sizes", "layers": args.layers, "layers_full": FULL_LAYERS,
+                   "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
+                   "head_dim": hd, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
+                   "global_batch": args.batch, "seq_len": args.prompt_len, "context": args.context,
+                   "mean_decode_context": round(mean_ctx, 1), "kv_block": 16, "tied_embeddings": True,
+                   "parallelism": "single GPU"},
+        "prefill": prefill, "roofline": roofline, "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
