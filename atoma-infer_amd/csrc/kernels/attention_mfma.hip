@@ -1,0 +1,278 @@
+// bfloat16 attention over the paged cache on the matrix cores, for prompts, portions and decoded tokens alike.
+// Compiled once per head size: -DATOMA_HD=<multiple of 16, at most 256>.  Pages hold 16 tokens.
+//
+// Work is cut on the host into tasks, one per wave: 32 query rows against a range of keys.  A row is a
+// (token, query head) pair of one request and one KV head: row r of a tile is head r / qt, token tok0 + r % qt,
+// so the heads of a group share every key and value that is read (the reference does this only for some of its
+// kernels: csrc/src/lib.rs:69-100).  The four waves of a workgroup run four consecutive tasks; the host orders
+// tasks so that these read the same keys (the heads of one tile, or neighbouring key ranges of one request) and
+// meet in the L1 cache.  A task either covers all keys its rows may see and writes the output, or covers one
+// 256-key chunk and writes a partial result (normalised output and log-sum-exp) that the combine kernel merges:
+// the split keeps the GPU busy when few rows face many keys (csrc/kernels/flash_fwd_kernel.h:1131-1310 is the
+// reference's combine).  The cut depends only on the request's own lengths, never on the rest of the batch.
+//
+// Per block of 32 keys (two pages), with v_mfma_f32_32x32x16_bf16:
+//   S^T[key, row] = K[key, :] . Q[row, :]     K page rows are the A operand straight from global memory,
+//                                             Q the B operand, kept in registers for the whole task;
+//   online softmax down the keys of each row in float32 (exp2 with the scale folded in), masked by the row's
+//   own position and window (bottom-right aligned causal mask, csrc/kernels/mask.h:171-192);
+//   O^T[d, row] += V^T[d, key] . P^T[key, row]  S^T's accumulator layout is already the B operand layout, so
+//                                             P goes from registers to the MFMA as bfloat16 without a
+//                                             transpose, and V^T is how the cache stores values.
+#include "common.h"
+
+using namespace atoma;
+
+#ifndef ATOMA_HD
+#error "compile with -DATOMA_HD=<head size>"
+#endif
+
+constexpr int HD = ATOMA_HD;
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
+constexpr int KSTEPS = HD / 16;        // MFMA steps over the head dimension for S
+constexpr int DTILES = (HD + 31) / 32; // 32-row tiles of O^T
+constexpr int PAGE = 16;
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+struct Task {
+  int32_t entry;    // row of the block tables; < 0: nothing to do
+  int32_t tok0;     // first token of the tile, counted inside the entry
+  int32_t qt;       // tokens per head in the tile
+  int32_t row0;     // first of this task's 32 rows inside the tile
+  int32_t k_begin;  // keys [k_begin, k_end) by absolute position; k_begin is a multiple of 32
+  int32_t k_end;
+  int32_t dest;     // < 0: write the output; else index of the partial result
+  int32_t n_parts;  // combine tasks: number of partial results starting at dest
+};
+
+__device__ __forceinline__ bf16x8 pack8(const float* v) {
+  bf16x8 r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = (__bf16)v[i];
+  return r;
+}
+
+__global__ void __launch_bounds__(256)
+attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
+                      const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
+                      float* __restrict__ part_o, float* __restrict__ part_lse, const Task* __restrict__ tasks,
+                      int n_tasks, const int32_t* __restrict__ block_tables, int max_blocks,
+                      const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions, float scale,
+                      int window, int nh, int nkv) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ti = blockIdx.x * 4 + wave;
+  if (ti >= n_tasks) return;
+  const Task task = tasks[ti];
+  if (task.entry < 0) return;
+  const int kvh = blockIdx.y;
+  const int g = nh / nkv;
+  const int c = lane & 31, hg = lane >> 5;
+
+  // this lane's row
+  const int r = task.row0 + c;
+  const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
+  const int tok_base = q_start[task.entry];
+  const int count = q_start[task.entry + 1] - tok_base;
+  const bool row_ok = hq < g && tok < count;
+  const int trow = tok_base + (row_ok ? tok : 0);
+  const int p_row = row_ok ? positions[trow] : -1;
+  const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
+  const int head = kvh * g + (row_ok ? hq : 0);
+
+  // Q fragments: B operand, lane (row c, k half hg) holds 8 consecutive d per step
+  bf16x8 qf[KSTEPS];
+  {
+    const uint16_t* qp = q + (size_t)trow * q_stride + (size_t)head * HD + hg * 8;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
+  }
+
+  const int32_t* table = block_tables + (size_t)task.entry * max_blocks;
+  const float sc2 = scale * kLog2e;
+  float m = -INFINITY, l = 0.f;
+  f32x16 o[DTILES];
+#pragma unroll
+  for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
+
+  const size_t kv_head_stride = (size_t)PAGE * HD;            // one (page, head) tile
+  const size_t page_stride = (size_t)nkv * kv_head_stride;
+
+  for (int kb = task.k_begin; kb < task.k_end; kb += 32) {
+    int b0 = kb / PAGE, b1 = b0 + 1;
+    if (b0 > max_blocks - 1) b0 = max_blocks - 1;
+    if (b1 > max_blocks - 1) b1 = max_blocks - 1;
+    const int pg0 = table[b0], pg1 = table[b1];
+
+    // S^T = K Q^T
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    {
+      const int pg = (c < 16) ? pg0 : pg1;
+      const uint16_t* kp = kcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride + (size_t)(c & 15) * HD +
+                           hg * 8;
+#pragma unroll
+      for (int st = 0; st < KSTEPS; ++st) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + st * 16);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
+      }
+    }
+
+    // V^T fragments for both pages, issued before the softmax so that their latency hides behind it
+    bf16x8 vf[2][DTILES];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int pg = j ? pg1 : pg0;
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt) {
+        const int d = dt * 32 + c;
+        if (HD % 32 == 0 || d < HD) {
+          const uint16_t* vp = vcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride + (size_t)d * PAGE +
+                               hg * 4;
+          const bf16x4 a = *reinterpret_cast<const bf16x4*>(vp);
+          const bf16x4 b = *reinterpret_cast<const bf16x4*>(vp + 8);
+          vf[j][dt] = bf16x8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) vf[j][dt][i] = (__bf16)0.f;
+        }
+      }
+    }
+
+    // mask and online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4
+    float bmax = -INFINITY;
+    float sv[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
+      const bool ok = key <= p_row && key >= lo_row && key < task.k_end;
+      sv[i] = ok ? s[i] * sc2 : -INFINITY;
+      bmax = fmaxf(bmax, sv[i]);
+    }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    const float m_new = fmaxf(m, bmax);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = __builtin_amdgcn_exp2f(m - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sv[i] = __builtin_amdgcn_exp2f(sv[i] - m_use);
+      psum += sv[i];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = m_new;
+
+    // O^T = O^T * corr + V^T P^T
+    const bf16x8 p0 = pack8(sv), p1 = pack8(sv + 8);
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[0][dt], p0, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[1][dt], p1, o[dt], 0, 0, 0);
+    }
+  }
+
+  // accumulator element i of tile dt is d = dt*32 + (i/4)*8 + hg*4 + i%4 of row c
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  if (task.dest < 0) {
+    if (!row_ok) return;
+    uint16_t* op = out + (size_t)trow * out_stride + (size_t)head * HD;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d = dt * 32 + q4 * 8 + hg * 4;
+        if (HD % 32 == 0 || d < HD) {
+          uint2 v;
+          v.x = (uint32_t)f32_to_bf16_bits(o[dt][q4 * 4 + 0] * inv) |
+                ((uint32_t)f32_to_bf16_bits(o[dt][q4 * 4 + 1] * inv) << 16);
+          v.y = (uint32_t)f32_to_bf16_bits(o[dt][q4 * 4 + 2] * inv) |
+                ((uint32_t)f32_to_bf16_bits(o[dt][q4 * 4 + 3] * inv) << 16);
+          *reinterpret_cast<uint2*>(op + d) = v;
+        }
+      }
+  } else {
+    float* po = part_o + (((size_t)task.dest * nkv + kvh) * 32 + c) * HD;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d = dt * 32 + q4 * 8 + hg * 4;
+        if (HD % 32 == 0 || d < HD) {
+          float4 v = make_float4(o[dt][q4 * 4 + 0] * inv, o[dt][q4 * 4 + 1] * inv, o[dt][q4 * 4 + 2] * inv,
+                                 o[dt][q4 * 4 + 3] * inv);
+          *reinterpret_cast<float4*>(po + d) = v;
+        }
+      }
+    if (hg == 0) part_lse[((size_t)task.dest * nkv + kvh) * 32 + c] = l > 0.f ? m + __builtin_amdgcn_logf(l) : -INFINITY;
+  }
+}
+
+// Merge partial results: out = sum_s w_s O_s / sum_s w_s with w_s = exp2(lse_s - max lse).
+// One block per (combine task, KV head): 32 rows x 8 threads, each thread HD/8 values of its row.
+__global__ void __launch_bounds__(256)
+attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
+                         uint16_t* __restrict__ out, int out_stride, const Task* __restrict__ tasks,
+                         const int32_t* __restrict__ q_start, int nh, int nkv) {
+  const Task task = tasks[blockIdx.x];
+  if (task.entry < 0) return;
+  const int kvh = blockIdx.y, g = nh / nkv;
+  const int c = threadIdx.x >> 3, sub = threadIdx.x & 7;
+  const int r = task.row0 + c;
+  const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
+  const int tok_base = q_start[task.entry];
+  const int count = q_start[task.entry + 1] - tok_base;
+  if (hq >= g || tok >= count) return;
+  float mx = -INFINITY;
+  for (int s = 0; s < task.n_parts; ++s)
+    mx = fmaxf(mx, part_lse[((size_t)(task.dest + s) * nkv + kvh) * 32 + c]);
+  float acc[HD / 8];
+#pragma unroll
+  for (int i = 0; i < HD / 8; ++i) acc[i] = 0.f;
+  float wsum = 0.f;
+  for (int s = 0; s < task.n_parts; ++s) {
+    const size_t base = ((size_t)(task.dest + s) * nkv + kvh) * 32 + c;
+    const float w = __builtin_amdgcn_exp2f(part_lse[base] - mx);  // lse = -inf gives weight 0
+    wsum += w;
+    const float* po = part_o + base * HD;
+#pragma unroll
+    for (int i = 0; i < HD / 8; ++i) acc[i] += w * po[sub + i * 8];
+  }
+  const float inv = 1.0f / wsum;
+  uint16_t* op = out + (size_t)(tok_base + tok) * out_stride + (size_t)(kvh * g + hq) * HD;
+#pragma unroll
+  for (int i = 0; i < HD / 8; ++i) op[sub + i * 8] = f32_to_bf16_bits(acc[i] * inv);
+}
+
+extern "C" int atoma_attention_mfma_head_size() { return HD; }
+
+// tasks: device array of n_tasks Task records (main kernel), followed by n_combine records for the combine kernel.
+extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kcache, const void* vcache, void* out,
+                                    int out_stride, float* part_o, float* part_lse, const int32_t* tasks, int n_tasks,
+                                    int n_combine, const int32_t* block_tables, int max_blocks,
+                                    const int32_t* q_start, const int32_t* positions, float scale, int window,
+                                    int nh, int nkv, hipStream_t stream) {
+  if (n_tasks <= 0) return 0;
+  if (nkv <= 0 || nh % nkv || nkv > 65535 || max_blocks <= 0 || (q_stride & 7) || (out_stride & 3) ||
+      ((uintptr_t)q & 15) || ((uintptr_t)out & 7))
+    return ATOMA_ERR_SHAPE;
+  const Task* t = reinterpret_cast<const Task*>(tasks);
+  hipLaunchKernelGGL(attention_mfma_kernel, dim3((n_tasks + 3) / 4, nkv), dim3(256), 0, stream, (const uint16_t*)q,
+                     q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride, part_o,
+                     part_lse, t, n_tasks, block_tables, max_blocks, q_start, positions, scale, window, nh, nkv);
+  ATOMA_LAUNCH_CHECK();
+  if (n_combine > 0) {
+    hipLaunchKernelGGL(attention_combine_kernel, dim3(n_combine, nkv), dim3(256), 0, stream, part_o, part_lse,
+                       (uint16_t*)out, out_stride, t + n_tasks, q_start, nh, nkv);
+    ATOMA_LAUNCH_CHECK();
+  }
+  return 0;
+}

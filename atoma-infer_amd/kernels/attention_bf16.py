@@ -1,7 +1,113 @@
-"""bfloat16 attention over the paged cache on the matrix cores."""
+"""bfloat16 attention over the paged cache on the matrix cores: task lists on the host, kernels per head size.
+
+``try_attention`` runs ``attention_mfma.hip`` (compiled for the model's head size on first use) when the cache
+has 16-token pages; otherwise it returns False and the caller runs the general kernel.
+
+The step's entries are cut into tasks of 32 query rows (row = token x query head of one KV group) against a key
+range.  An entry with few tokens and many keys (a decoded token, a short portion late in a prompt) is split into
+256-key chunks whose partial results a second kernel merges; everything else runs each tile against all its
+keys.  The cut depends only on the entry's own start and length.  The task list is built once per step and
+shared by all layers with the same grouping and window.
+"""
 from __future__ import annotations
+
+import ctypes
+from typing import Dict, Tuple
+
+import numpy as np
+import torch
+
+from .library import load_hip_module
+from .ops import _check, _p, _stream
+
+PAGE = 16
+CHUNK = 256          # keys per partial task
+SPLIT_MAX_TOKENS = 16  # entries with at most this many tokens may be split along the keys
+SPLIT_MIN_KEYS = 2 * CHUNK
+_libs: Dict[int, ctypes.CDLL] = {}
+
+
+def module_name(hd: int) -> str:
+    return f"attention_hd{hd}"
+
+
+def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
+    if hd not in _libs or force_build:
+        _libs[hd] = load_hip_module(module_name(hd), ("attention_mfma.hip",), (f"ATOMA_HD={hd}",),
+                                    force_build=force_build)
+        assert _libs[hd].atoma_attention_mfma_head_size() == hd
+    return _libs[hd]
+
+
+def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int) -> Tuple[np.ndarray, int, int, int]:
+    """Task records [n, 8] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials).
+
+    Main tasks are padded to a multiple of 4 (one workgroup runs 4) and ordered so that tasks sharing keys are
+    neighbours and long tasks come first.
+    """
+    qt_max = max(1, 128 // group)
+    direct, split, combine = [], [], []
+    n_part = 0
+    for e in range(len(starts)):
+        start, count = int(starts[e]), int(counts[e])
+        k_end_all = start + count
+        qt = min(qt_max, count)
+        rows = qt * group
+        first_key = max(0, start - window + 1) if window > 0 else 0
+        do_split = count <= SPLIT_MAX_TOKENS and (k_end_all - first_key) >= SPLIT_MIN_KEYS
+        for tok0 in range(0, count, qt):
+            last = min(tok0 + qt, count)
+            k_end = start + last
+            lo = max(0, start + tok0 - window + 1) if window > 0 else 0
+            if do_split:
+                c0 = (lo // CHUNK) * CHUNK
+                chunks = list(range(c0, k_end, CHUNK))
+                for row0 in range(0, rows, 32):
+                    combine.append((e, tok0, qt, row0, 0, 0, n_part, len(chunks)))
+                    for kb in chunks:
+                        split.append((e, tok0, qt, row0, kb, min(kb + CHUNK, k_end), n_part, 0))
+                        n_part += 1
+            else:
+                kb = (lo // 32) * 32
+                wave_tasks = [(e, tok0, qt, row0, kb, k_end, -1, 0) for row0 in range(0, rows, 32)]
+                while len(wave_tasks) % 4:
+                    wave_tasks.append((-1, 0, 1, 0, 0, 0, -1, 0))
+                direct.append((k_end - kb, wave_tasks))
+    direct.sort(key=lambda x: -x[0])
+    main = [t for _, ws in direct for t in ws] + split
+    while len(main) % 4:
+        main.append((-1, 0, 1, 0, 0, 0, -1, 0))
+    arr = np.asarray(main + combine, dtype=np.int32).reshape(-1, 8)
+    return arr, len(main), len(combine), n_part
 
 
 def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, hd) -> bool:
     """Run the fast kernels if they take this shape; False sends the caller to the general kernel."""
-    return False
+    if cache.page_size != PAGE or hd % 16 or not 16 <= hd <= 256:
+        return False
+    if q.stride(0) % 8 or q.data_ptr() % 16 or out.stride(0) % 4:
+        return False
+    group = nh // nkv
+    key = ("attention_tasks", group, window)
+    plan = ctx.scratch.get(key)
+    if plan is None:
+        arr, n_main, n_comb, n_part = build_tasks(ctx.h_starts, ctx.h_counts, group, window)
+        tasks = torch.from_numpy(arr).to(q.device, non_blocking=False)
+        plan = (tasks, n_main, n_comb, n_part)
+        ctx.scratch[key] = plan
+    tasks, n_main, n_comb, n_part = plan
+    part_o = part_lse = None
+    if n_part:
+        ws_key = ("attention_partials", nkv, hd)
+        ws = ctx.scratch.get(ws_key)
+        if ws is None or ws[0].shape[0] < n_part:
+            ws = (torch.empty((n_part, nkv, 32, hd), dtype=torch.float32, device=q.device),
+                  torch.empty((n_part, nkv, 32), dtype=torch.float32, device=q.device))
+            ctx.scratch[ws_key] = ws
+        part_o, part_lse = ws
+    bt = cache.block_tables
+    _check(lib(hd).atoma_attention_mfma(_p(q), q.stride(0), _p(k_cache), _p(v_cache), _p(out), out.stride(0),
+                                        _p(part_o), _p(part_lse), _p(tasks), n_main, n_comb, _p(bt), bt.shape[1],
+                                        _p(ctx.q_start), _p(ctx.positions), ctypes.c_float(scale), int(window), nh,
+                                        nkv, _stream()), "attention_mfma")
+    return True

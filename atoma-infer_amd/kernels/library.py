@@ -48,6 +48,16 @@ HIP_MODULES: Dict[str, Tuple[Sequence[str], Sequence[str]]] = {
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
+_module_locks: Dict[str, threading.Lock] = {}
+
+# head sizes whose attention module the build check compiles ahead of time; any other multiple of 16 up to 256
+# is compiled when a model with that head size is first used
+STANDARD_HEAD_SIZES = (16, 32, 48, 64, 80, 96, 128, 256)
+
+
+def _lock_for(name: str) -> threading.Lock:
+    with _lock:
+        return _module_locks.setdefault(name, threading.Lock())
 
 
 def _say(msg: str) -> None:
@@ -75,9 +85,8 @@ def _writable_lib_dir() -> str:
     for d in _lib_dirs():
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, f".probe_{os.getpid()}")
-            with open(probe, "w"):
-                pass
+            fd, probe = tempfile.mkstemp(prefix=".probe_", dir=d)
+            os.close(fd)
             os.remove(probe)
             return d
         except OSError:
@@ -153,7 +162,7 @@ def _module_plan(name: str, sources: Sequence[str], defines: Sequence[str]):
 def load_hip_module(name: str, sources: Optional[Sequence[str]] = None, defines: Sequence[str] = (),
                     *, force_build: bool = False) -> ctypes.CDLL:
     """Load HIP module ``name``, compiling it first if no built library matches its sources."""
-    with _lock:
+    with _lock_for(name):
         if name in _loaded and not force_build:
             return _loaded[name]
         if sources is None:
@@ -177,7 +186,7 @@ def load_hip_module(name: str, sources: Optional[Sequence[str]] = None, defines:
 def load_host_library(*, force_build: bool = False) -> ctypes.CDLL:
     """The host library (cache manager); needs no GPU and no ROCm."""
     name = "host"
-    with _lock:
+    with _lock_for(name):
         if name in _loaded and not force_build:
             return _loaded[name]
         paths = sorted(os.path.join(_HOST, f) for f in os.listdir(_HOST) if f.endswith(".cpp"))
@@ -193,12 +202,17 @@ def load_host_library(*, force_build: bool = False) -> ctypes.CDLL:
         return lib
 
 
-def build_all(head_sizes: Sequence[int] = ()) -> List[str]:
+def build_all(head_sizes: Sequence[int] = STANDARD_HEAD_SIZES) -> List[str]:
     """Compile every module from scratch (the build check); returns the names built."""
+    from . import attention_bf16
     built = []
     load_host_library(force_build=True)
     built.append("host")
-    for name in HIP_MODULES:
-        load_hip_module(name, force_build=True)
-        built.append(name)
+    jobs = [(name, None, ()) for name in HIP_MODULES]
+    jobs += [(attention_bf16.module_name(hd), ("attention_mfma.hip",), (f"ATOMA_HD={hd}",)) for hd in head_sizes]
+    with ThreadPoolExecutor(min(8, len(jobs))) as pool:
+        futs = [pool.submit(load_hip_module, n, src, d, force_build=True) for n, src, d in jobs]
+        for (n, _, _), f in zip(jobs, futs):
+            f.result()
+            built.append(n)
     return built

@@ -135,3 +135,184 @@ def test_gemm_bf16_float32_out_for_many_rows():
     cb = gemm_bf16.try_linear(a, w, torch.bfloat16)   # the library product
     assert (cb.double().cpu() - want).abs().max() <= 1e-2 * want.abs().max()
     assert gemm_bf16.try_linear(a[:, :40], w[:, :40], torch.float32) is None   # K no multiple of 32: refused
+
+
+# ----------------------------------------------------------------------------------------------------------
+# attention kernels against plain softmax(QK^T)V
+
+
+class FakeCtx:
+    """Only what the attention wrappers read of a StepContext."""
+
+    def __init__(self, starts, counts):
+        import numpy as np
+        self.h_starts = np.asarray(starts, dtype=np.int32)
+        self.h_counts = np.asarray(counts, dtype=np.int32)
+        qs = [0]
+        for c in counts:
+            qs.append(qs[-1] + c)
+        self.q_start = torch.tensor(qs, dtype=torch.int32, device=DEV)
+        pos, seq = [], []
+        for e, (s, c) in enumerate(zip(starts, counts)):
+            pos += list(range(s, s + c))
+            seq += [e] * c
+        self.positions = torch.tensor(pos, dtype=torch.int32, device=DEV)
+        self.token_seq = torch.tensor(seq, dtype=torch.int32, device=DEV)
+        self.scratch = {}
+
+
+class FakeCache:
+    def __init__(self, block_tables, page):
+        self.block_tables, self.page_size = block_tables, page
+
+
+def paged_setup(lens, nkv, hd, page, dtype, seed=0):
+    """Random keys/values for requests of the given lengths, laid into shuffled pages.  Returns
+    (k list, v list as float32 [len, nkv, hd]), kcache, vcache, block_tables."""
+    g = torch.Generator().manual_seed(seed)
+    ks = [torch.randn(n, nkv, hd, generator=g).to(dtype) for n in lens]
+    vs = [torch.randn(n, nkv, hd, generator=g).to(dtype) for n in lens]
+    blocks = [-(-n // page) for n in lens]
+    total = sum(blocks) + 3
+    perm = torch.randperm(total, generator=g).tolist()
+    kc = torch.randn(total, nkv, page, hd, generator=g).to(dtype)    # unused slots hold noise, not zeros
+    vc = torch.randn(total, nkv, hd, page, generator=g).to(dtype)
+    bt = torch.zeros(len(lens), max(blocks), dtype=torch.int32)
+    nxt = 0
+    for e, n in enumerate(lens):
+        for b in range(blocks[e]):
+            pg = perm[nxt]
+            nxt += 1
+            bt[e, b] = pg
+            lo, hi = b * page, min((b + 1) * page, n)
+            kc[pg, :, : hi - lo, :] = ks[e][lo:hi].permute(1, 0, 2)
+            vc[pg, :, :, : hi - lo] = vs[e][lo:hi].permute(1, 2, 0)
+    return ks, vs, kc.to(DEV), vc.to(DEV), bt.to(DEV)
+
+
+def plain_attention(q, k, v, start, scale, window, group):
+    """q [c, nh, hd] at positions start..start+c-1 over k, v [len, nkv, hd] (float64)."""
+    c, nh, hd = q.shape
+    k = k.double().repeat_interleave(group, dim=1)
+    v = v.double().repeat_interleave(group, dim=1)
+    att = torch.einsum("qhd,khd->hqk", q.double(), k) * scale
+    pos = torch.arange(start, start + c)[:, None]
+    key = torch.arange(k.shape[0])[None, :]
+    keep = key <= pos
+    if window:
+        keep &= key > pos - window
+    att = att.masked_fill(~keep[None], float("-inf")).softmax(-1)
+    return torch.einsum("hqk,khd->qhd", att, v)
+
+
+ATTN_CASES = [
+    # (nh, nkv, hd, page, window, [(start, count), ...])
+    (4, 1, 16, 16, 0, [(0, 40), (0, 1), (39, 1)]),
+    (3, 3, 32, 16, 0, [(0, 70), (5, 9), (64, 2)]),
+    (8, 2, 64, 16, 0, [(0, 130), (600, 1), (1030, 3), (511, 1), (512, 1)]),
+    (6, 2, 48, 16, 0, [(0, 33), (100, 20)]),
+    (4, 4, 80, 16, 0, [(10, 50)]),
+    (16, 2, 128, 16, 0, [(0, 64), (700, 1)]),
+    (2, 1, 256, 16, 0, [(0, 35), (520, 2)]),
+    (8, 2, 64, 16, 48, [(0, 130), (600, 1), (1030, 3), (40, 20)]),
+    (4, 2, 32, 16, 600, [(0, 100), (900, 1), (640, 5)]),
+]
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,window,entries", ATTN_CASES)
+@pytest.mark.parametrize("kind", ["generic_f32", "generic_bf16", "mfma"])
+def test_paged_attention(nh, nkv, hd, page, window, entries, kind):
+    from atoma_infer_amd.kernels import attention_bf16, ops
+    dtype = torch.float32 if kind == "generic_f32" else torch.bfloat16
+    starts, counts = [s for s, _ in entries], [c for _, c in entries]
+    lens = [s + c for s, c in entries]
+    ks, vs, kc, vc, bt = paged_setup(lens, nkv, hd, page, dtype, seed=hd + nh)
+    t = sum(counts)
+    g = torch.Generator().manual_seed(1)
+    qkv = (torch.randn(t, (nh + 2 * nkv) * hd, generator=g) * 1.5).to(dtype).to(DEV)   # q lives inside a wider row
+    out = torch.empty(t, nh * hd, dtype=dtype, device=DEV)
+    ctx, cache = FakeCtx(starts, counts), FakeCache(bt, page)
+    scale = 1.0 / math.sqrt(hd)
+    if kind == "mfma":
+        assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, cache, scale, window, nh, nkv, hd)
+    else:
+        ops.paged_attention_generic(qkv, kc, vc, out, bt, ctx.token_seq, ctx.positions, scale, window, page, nh,
+                                    nkv, hd)
+    row = 0
+    for e, (s, c) in enumerate(entries):
+        q = qkv[row:row + c, : nh * hd].cpu().view(c, nh, hd)
+        want = plain_attention(q, ks[e], vs[e], s, scale, window, nh // nkv).reshape(c, nh * hd)
+        got = out[row:row + c].double().cpu()
+        tol = 2e-5 if dtype is torch.float32 else 2e-2
+        err = (got - want).abs().max() / want.abs().max()
+        assert err < tol, f"entry {e} ({s}, {c}): {err:.3e}"
+        row += c
+
+
+def test_attention_reference_vectors():
+    """The reference's own golden values: csrc/tests/flash_attn_tests.rs:31-93 (no mask, as a one-token decode of the
+    second row is not what they test, the unmasked case is rebuilt as two single-key requests...) and the causal
+    ones of models/src/flash_attention.rs:632-705: q = arange(48)/30, k = /40, v = /50 shaped (3 heads, 2 tokens,
+    8), scale 0.5; row 0 of every head equals v[0]."""
+    from atoma_infer_amd.kernels import ops
+    base = torch.arange(48, dtype=torch.float32).reshape(3, 2, 8).half().float()
+    q, k, v = (base / 30).half().float(), (base / 40).half().float(), (base / 50).half().float()
+    causal = torch.tensor([
+        [[0.0, 0.02, 0.04, 0.06, 0.08, 0.1, 0.12, 0.14],
+         [0.0922, 0.1122, 0.1322, 0.1522, 0.1721, 0.1921, 0.2122, 0.2322]],
+        [[0.3201, 0.3401, 0.3601, 0.3801, 0.4001, 0.4202, 0.4402, 0.4602],
+         [0.428, 0.448, 0.468, 0.488, 0.5083, 0.5283, 0.5483, 0.5684]],
+        [[0.6401, 0.6602, 0.6802, 0.7002, 0.7202, 0.7402, 0.7603, 0.7803],
+         [0.7622, 0.7822, 0.8022, 0.8223, 0.8423, 0.8623, 0.8823, 0.9023]]])
+    # head size 8 is below what the kernels take: embed each head into 16 columns, the upper 8 zero
+    hd, nh, page = 16, 3, 16
+    qq = torch.zeros(2, nh, hd)
+    qq[:, :, :8] = q.permute(1, 0, 2)
+    kc = torch.zeros(1, nh, page, hd)
+    vc = torch.zeros(1, nh, hd, page)
+    kc[0, :, :2, :8] = k
+    vc[0, :, :8, :2] = v.permute(0, 2, 1)
+    out = torch.empty(2, nh * hd, device=DEV)
+    bt = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
+    ctx = FakeCtx([0], [2])
+    ops.paged_attention_generic(qq.reshape(2, nh * hd).to(DEV), kc.to(DEV), vc.to(DEV), out, bt, ctx.token_seq,
+                                ctx.positions, 0.5, 0, page, nh, nh, hd)
+    got = out.cpu().view(2, nh, hd)[:, :, :8].permute(1, 0, 2)
+    # the goldens were computed in float16 and rounded to 4 places
+    assert (got - causal).abs().max() < 1.5e-3
+    assert torch.allclose(got[:, 0], v[:, 0], atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_cache_write(dtype):
+    from atoma_infer_amd.kernels import ops
+    nh, nkv, hd, page, t = 5, 2, 48, 4, 9
+    g = torch.Generator().manual_seed(3)
+    qkv = torch.randn(t, (nh + 2 * nkv) * hd, generator=g).to(dtype)
+    pos = torch.tensor([0, 1, 2, 3, 4, 50, 51, 7, 8], dtype=torch.int32)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))
+    ang = torch.arange(64).float()[:, None] * inv[None]
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    slots = torch.tensor([8, 9, 10, 11, 0, 1, -1, 30, 31], dtype=torch.int32)
+    kc = torch.zeros(8, nkv, page, hd, dtype=dtype)
+    vc = torch.zeros(8, nkv, hd, page, dtype=dtype)
+    d_qkv, d_kc, d_vc = qkv.to(DEV), kc.to(DEV), vc.to(DEV)
+    ops.rope_cache_write(d_qkv, pos.to(DEV), cos.to(DEV), sin.to(DEV), hd, d_kc, d_vc, slots.to(DEV), page, nh, nkv, hd)
+    x = qkv.float().view(t, nh + 2 * nkv, hd)
+    c, s = cos[pos.long()][:, None, :], sin[pos.long()][:, None, :]
+    x1, x2 = x[..., : hd // 2], x[..., hd // 2:]
+    rot = torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], -1)
+    tol = 1e-6 if dtype is torch.float32 else 1e-2
+    got = d_qkv.float().cpu().view(t, nh + 2 * nkv, hd)
+    assert torch.allclose(got[:, :nh], rot[:, :nh], atol=tol, rtol=tol)
+    assert torch.equal(got[:, nh + nkv:], x[:, nh + nkv:])          # v untouched in place
+    for i in range(t):
+        sl = int(slots[i])
+        if sl < 0:
+            continue
+        assert torch.allclose(d_kc.float().cpu()[sl // page, :, sl % page, :], rot[i, nh:nh + nkv], atol=tol, rtol=tol)
+        assert torch.equal(d_vc.cpu()[sl // page, :, :, sl % page].float(), x[i, nh + nkv:].to(dtype).float())
+    # slot -1 wrote nothing: pages 2..6 stay zero
+    assert torch.count_nonzero(d_kc[3:7]) == 0 and torch.count_nonzero(d_vc[3:7]) == 0
+    # position 0 is the identity
+    assert torch.allclose(got[0, :nh], x[0, :nh], atol=tol)
