@@ -1,0 +1,179 @@
+"""The cache manager: no page lost, held twice or freed twice, under random orders of requests; windows; slots."""
+import random
+
+import numpy as np
+import pytest
+from hypothesis import given, settings
+from hypothesis import strategies as st
+
+from atoma_infer_amd.cache import CacheError, CacheManager, GroupGeometry, OutOfPages
+
+
+def test_allocate_grow_free():
+    """Mirrors backends/vllm/src/block_manager.rs:1162-1552 (allocate, append, free) for one group."""
+    m = CacheManager([GroupGeometry(4, 6)], 2)
+    assert m.add(10) == 0
+    m.reserve(10, 9)                       # 3 pages
+    assert m.table(10) == [0, 1, 2] and m.num_free_pages() == 3
+    m.reserve(10, 9)                       # idempotent
+    m.reserve(10, 12)                      # still 3 pages
+    assert m.num_free_pages() == 3
+    m.reserve(10, 13)                      # a 4th
+    assert m.table(10) == [0, 1, 2, 3] and m.reserved_len(10) == 13
+    m.check()
+    assert m.can_reserve(10, 24) and not m.can_reserve(10, 25)
+    with pytest.raises(OutOfPages):
+        m.reserve(10, 25)
+    assert m.table(10) == [0, 1, 2, 3]     # nothing taken by the failed call
+    m.free(10)
+    assert m.num_free_pages() == 6 and m.num_free_slots() == 2 and m.num_requests() == 0
+    m.check()
+
+
+def test_double_free_and_unknown_requests_are_errors():
+    """backends/vllm/src/block_allocator.rs:147-229: freeing twice is an error."""
+    m = CacheManager([GroupGeometry(4, 4)], 1)
+    m.add(1)
+    m.reserve(1, 5)
+    m.free(1)
+    with pytest.raises(CacheError):
+        m.free(1)
+    with pytest.raises(CacheError):
+        m.reserve(2, 4)
+    with pytest.raises(CacheError):
+        m.table(2)
+    m.add(3)
+    with pytest.raises(CacheError):
+        m.add(3)
+    with pytest.raises(OutOfPages):
+        m.add(4)                           # the only slot is taken
+    m.check()
+
+
+def test_freed_pages_are_used_again_last_freed_first():
+    m = CacheManager([GroupGeometry(2, 4)], 4)
+    m.add(1)
+    m.reserve(1, 4)                        # pages 0, 1
+    m.add(2)
+    m.reserve(2, 2)                        # page 2
+    m.free(1)
+    m.add(3)
+    m.reserve(3, 6)
+    assert m.table(3) == [0, 1, 3]         # the freed pages first, in ascending order of position
+    m.check()
+
+
+def test_groups_reserve_together_or_not_at_all():
+    m = CacheManager([GroupGeometry(4, 8), GroupGeometry(4, 2)], 2)
+    m.add(1)
+    with pytest.raises(OutOfPages):
+        m.reserve(1, 12)                   # group 1 has only 2 pages
+    assert m.num_free_pages(0) == 8 and m.num_free_pages(1) == 2
+    m.reserve(1, 8)
+    assert m.table(1, 0) == [0, 1] and m.table(1, 1) == [0, 1]
+    assert m.fits_at_all(8) and not m.fits_at_all(9)
+
+
+def test_window_gives_pages_back_while_running():
+    m = CacheManager([GroupGeometry(4, 16, None), GroupGeometry(4, 4, 6)], 1)
+    m.add(1)
+    length = 0
+    for step in range(40):
+        length += 1
+        m.reserve(1, length)
+        m.release_behind(1, length)
+        m.check()
+        # a window of 6 tokens over pages of 4 never needs more than 3 live pages
+        live = [p for p in m.table(1, 1) if p >= 0]
+        assert len(live) <= 3
+        first_needed = max(0, length - 6 + 1)
+        assert all(p >= 0 for p in m.table(1, 1)[first_needed // 4:])
+    assert len(m.table(1, 0)) == 10 and all(p >= 0 for p in m.table(1, 0))
+    m.free(1)
+    assert m.num_free_pages(1) == 4 and m.num_free_pages(0) == 16
+    m.check()
+
+
+def test_fill_step_slots_and_tables():
+    m = CacheManager([GroupGeometry(4, 8)], 4)
+    m.add(7)
+    m.add(9)
+    m.reserve(9, 3)
+    m.reserve(7, 10)
+    ids = np.array([7, 9], dtype=np.int64)
+    starts, counts = np.array([6, 0], dtype=np.int32), np.array([4, 3], dtype=np.int32)
+    sm = np.full(7, -9, dtype=np.int32)
+    bt = np.full((2, 3), -9, dtype=np.int32)
+    m.fill_step(0, ids, starts, counts, sm, bt)
+    t7, t9 = m.table(7), m.table(9)
+    assert bt.tolist() == [t7, t9 + [0, 0]]
+    want = [t7[p // 4] * 4 + p % 4 for p in range(6, 10)] + [t9[0] * 4 + p for p in range(3)]
+    assert sm.tolist() == want
+    with pytest.raises(CacheError):
+        m.fill_step(0, ids, np.array([9, 0], dtype=np.int32), counts, sm, bt)   # position 12 has no page
+
+
+@settings(max_examples=60, deadline=None)
+@given(seed=st.integers(0, 10_000), page=st.sampled_from([1, 4, 16]), pages=st.integers(4, 40),
+       window=st.sampled_from([None, 3, 17]))
+def test_random_orders_keep_the_books(seed, page, pages, window):
+    rng = random.Random(seed)
+    m = CacheManager([GroupGeometry(page, pages), GroupGeometry(page, pages, window)], 5)
+    live = {}
+    next_id = 0
+    for _ in range(200):
+        op = rng.random()
+        if op < 0.25 and m.num_free_slots() > 0:
+            m.add(next_id)
+            live[next_id] = 0
+            next_id += 1
+        elif op < 0.75 and live:
+            r = rng.choice(list(live))
+            new = live[r] + rng.randint(1, 3 * page)
+            if m.can_reserve(r, new):
+                m.reserve(r, new)
+                live[r] = new
+                if rng.random() < 0.7:
+                    m.release_behind(r, new)
+            else:
+                with pytest.raises(OutOfPages):
+                    m.reserve(r, new)
+        elif live:
+            r = rng.choice(list(live))
+            m.free(r)
+            del live[r]
+        m.check()
+        held = sum(-(-n // page) for n in live.values())
+        assert m.num_free_pages(0) == pages - held
+        assert m.num_free_pages(1) >= pages - held
+        assert m.num_requests() == len(live) and m.num_free_slots() == 5 - len(live)
+    for r in list(live):
+        m.free(r)
+    m.check()
+    assert m.num_free_pages(0) == pages and m.num_free_pages(1) == pages and m.num_free_slots() == 5
+
+
+def test_plan_cache_groups_layers_by_their_needs():
+    from atoma_infer_amd.cache import plan_cache
+    from atoma_infer_amd.config import LlamaConfig
+    from atoma_infer_amd.models import LayerCall
+    from atoma_infer_amd.models.llama import build_llama
+    from util import TINY_B
+    spec = build_llama(LlamaConfig.from_dict(TINY_B))
+    plan = plan_cache(spec)
+    assert len(plan.groups) == 1 and plan.groups[0].calls == [0, 1, 2]
+    assert plan.bytes_per_token(2) == 2 * 3 * 3 * 32 * 2
+    # a layer named twice has two entries; a call that reads another call's cache has none of its own
+    spec.run_order = [LayerCall(0), LayerCall(1), LayerCall(1), LayerCall(2, kv_from=0)]
+    spec.__post_init__()
+    plan = plan_cache(spec)
+    assert plan.groups[0].calls == [0, 1, 2]
+    assert plan.where[3] == (0, 0, False) and plan.where[2] == (0, 2, True)
+    # a window makes a group of its own
+    spec.layers[2][1].mixer.window = 8
+    spec.run_order = [LayerCall(0), LayerCall(1), LayerCall(2)]
+    plan = plan_cache(spec)
+    assert [g.spec.window for g in plan.groups] == [None, 8] and plan.where[2] == (1, 0, True)
+    with pytest.raises(ValueError):
+        spec.run_order = [LayerCall(0), LayerCall(2, kv_from=0)]   # needs differ
+        spec.__post_init__()
