@@ -1,0 +1,244 @@
+"""Generation through the entry points: greedy tokens against the plain implementation, sampling kernels against
+the plain sampling functions, the scheduler under page pressure on the GPU, and bin/trace_run as a program."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+from util import (NORM_JITTER, TINY, TOL_BF16, TOL_F32, frob_err, make_model_dir, plain_config, plain_weights,
+                  random_tokens, rel_err)
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def model_dirs(tmp_path_factory):
+    return {name: make_model_dir(str(tmp_path_factory.mktemp(f"gen_{name}")), cfg, seed=21, dtype="bfloat16",
+                                 norm_jitter=NORM_JITTER[name]) for name, cfg in TINY.items()}
+
+
+def engine(model_dir, dtype, page, pages, **sched):
+    from atoma_infer_amd.config import CacheConfig, SchedulerConfig
+    from atoma_infer_amd.engine.engine import LlmEngine
+    sched.setdefault("max_num_batched_tokens", 64)
+    sched.setdefault("max_num_sequences", 4)
+    sched.setdefault("max_model_len", 128)
+    return LlmEngine(model_dir, dtype, cache=CacheConfig(block_size=page, num_gpu_blocks_override=pages),
+                     scheduler=SchedulerConfig(**sched))
+
+
+def test_greedy_generation_tiny_a_workload(model_dirs):
+    """BASELINE's Tiny A workload: 2 prompts of 8 and 5 ids, 8 greedy steps each, float32, block size 4."""
+    from atoma_infer_amd.sampling import GenerateParameters
+    d = model_dirs["A"]
+    w, cfg = plain_weights(d), plain_config(d)
+    prompts = [random_tokens(8, 512, 1), random_tokens(5, 512, 2)]
+    want = [plain_llama.greedy_generate(p, 8, w, cfg) for p in prompts]
+    eng = engine(d, "float32", 4, 16)
+    outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=8, ignore_eos_token=True))
+    assert [o.inference_outputs[0].token_ids for o in outs] == want
+    assert all(o.is_finished and o.inference_outputs[0].finish_reason == "length_capped" for o in outs)
+    assert eng.runner.manager.num_free_pages() == 16 and eng.runner.manager.num_requests() == 0
+    # the function-style entry point gives the same
+    from atoma_infer_amd import generate
+    from atoma_infer_amd.config import CacheConfig
+    outs2 = generate(d, prompts, GenerateParameters(do_sample=False, max_new_tokens=8, ignore_eos_token=True),
+                     dtype="float32", cache=CacheConfig(block_size=4, num_gpu_blocks_override=16))
+    assert [o.inference_outputs[0].token_ids for o in outs2] == want
+
+
+def test_tiny_b_workload_portions_beside_decodes_with_temperature(model_dirs):
+    """BASELINE's Tiny B workload: prompts of 37, 1 and 20 ids in 16-token portions alongside decodes, temperature
+    0.7 with a fixed seed.  The sampled tokens must be what the plain model and plain sampler give for the same
+    uniform numbers, and must not depend on how requests were batched."""
+    from atoma_infer_amd.sampling import GenerateParameters, uniform
+    d = model_dirs["B"]
+    w, cfg = plain_weights(d), plain_config(d)
+    prompts = [random_tokens(37, 1000, 3), random_tokens(1, 1000, 4), random_tokens(20, 1000, 5)]
+    params = GenerateParameters(temperature=0.7, random_seed=99, max_new_tokens=6, ignore_eos_token=True)
+    eng = engine(d, "float32", 16, 12, max_num_batched_tokens=16, max_prefill_chunk=16)
+    outs = eng.generate(prompts, params)
+    got = [o.inference_outputs[0].token_ids for o in outs]
+    for p, toks in zip(prompts, got):
+        seq = list(p)
+        for step, tok in enumerate(toks):
+            logits = plain_llama.forward(seq, w, cfg)[-1]
+            dist = plain_llama.sampling_distribution(logits, 0.7)
+            u = uniform(99, step)
+            want = plain_llama.draw(dist, u)
+            if tok != want:
+                # allowed only when u lands on the boundary between the two tokens within float32 rounding
+                c = torch.cumsum(dist.double(), 0) / dist.double().sum()
+                lo, hi = sorted((tok, want))
+                assert abs(float(c[lo:hi].max()) - u) < 1e-5 or abs(float(c[lo]) - u) < 1e-5, (step, tok, want)
+            seq.append(tok)
+    # alone, each request samples the same tokens
+    for p, toks in zip(prompts, got):
+        eng1 = engine(d, "float32", 16, 12)
+        alone = eng1.generate([p], params)[0].inference_outputs[0].token_ids
+        assert alone == toks
+    assert eng.stats["steps"] > 3
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_preemption_under_page_pressure_keeps_results(model_dirs, dtype):
+    """So few pages that running requests are preempted and recomputed: the tokens stay what they are alone."""
+    from atoma_infer_amd.sampling import GenerateParameters
+    d = model_dirs["C"]
+    prompts = [random_tokens(n, 331, 40 + i) for i, n in enumerate([30, 45, 20, 33, 12])]
+    params = GenerateParameters(do_sample=False, max_new_tokens=40, ignore_eos_token=True)
+    roomy = engine(d, dtype, 16, 64, max_model_len=256)
+    want = [o.inference_outputs[0].token_ids for o in roomy.generate(prompts, params)]
+    tight = engine(d, dtype, 16, 12, max_model_len=256)
+    outs = tight.generate(prompts, params)
+    got = [o.inference_outputs[0].token_ids for o in outs]
+    assert tight.stats["preemptions"] > 0
+    assert tight.runner.manager.num_free_pages() == 12
+    if dtype == "float32":
+        assert got == want
+    else:
+        # bfloat16 logits may differ in the last bits between batch shapes; a flipped argmax changes what follows
+        same = sum(a == b for g, x in zip(got, want) for a, b in zip(g, x))
+        assert same >= 0.9 * sum(len(x) for x in want)
+
+
+def test_eos_stops_and_too_long_is_ignored(model_dirs):
+    from atoma_infer_amd.sampling import GenerateParameters
+    d = model_dirs["A"]
+    w, cfg = plain_weights(d), plain_config(d)
+    prompt = random_tokens(6, 512, 9)
+    free_run = plain_llama.greedy_generate(prompt, 10, w, cfg)
+    eng = engine(d, "float32", 4, 32, max_model_len=64)
+    eng.eos_ids = {free_run[3]}
+    out = eng.generate([prompt], GenerateParameters(do_sample=False, max_new_tokens=10))[0].inference_outputs[0]
+    stop_at = free_run.index(free_run[3])
+    assert out.token_ids == free_run[:stop_at + 1] and out.finish_reason == "stopped" and out.stop_reason == free_run[3]
+    outs = eng.generate([random_tokens(70, 512, 1)], GenerateParameters(do_sample=False, max_new_tokens=2))
+    assert outs[0].inference_outputs[0].finish_reason == "ignored" and outs[0].inference_outputs[0].token_ids == []
+    from atoma_infer_amd.sampling import ValidationError
+    with pytest.raises(ValidationError):
+        eng.add_request([1, 2, 9999])
+    with pytest.raises(ValidationError):
+        eng.add_request("text without a tokenizer")
+
+
+# ----------------------------------------------------------------------------------------------------------
+# the sampling kernel against the plain sampling functions
+
+
+@pytest.mark.parametrize("vocab", [331, 1000, 5000])
+def test_sample_kernel(vocab):
+    from atoma_infer_amd.kernels import ops
+    g = torch.Generator().manual_seed(vocab)
+    rows = [(0.0, 0, 1.0), (0.7, 0, 1.0), (1.3, 5, 1.0), (0.7, 0, 0.6), (0.9, 20, 0.8), (0.5, 1, 1.0), (2.0, 0, 0.999)]
+    logits = torch.randn(len(rows), vocab, generator=g) * 2.0
+    logits[2, 10] = logits[2, 20] = logits[2].max() + 1.0        # ties at the top
+    for u in (0.0, 0.013, 0.25, 0.5, 0.77, 0.999):
+        dev = lambda x, dt: torch.tensor(x, dtype=dt, device="cuda:0")
+        tok, lg = ops.sample(logits.cuda(), dev([r[0] for r in rows], torch.float32),
+                             dev([r[1] for r in rows], torch.int32), dev([r[2] for r in rows], torch.float32),
+                             dev([u] * len(rows), torch.float32))
+        tok, lg = tok.cpu().tolist(), lg.cpu()
+        for i, (t, k, p) in enumerate(rows):
+            if t == 0.0:
+                assert tok[i] == int(torch.argmax(logits[i]))
+                continue
+            dist = plain_llama.sampling_distribution(logits[i], t, k, p)
+            want = plain_llama.draw(dist, u)
+            assert dist[tok[i]] > 0, f"row {i}: token {tok[i]} is outside the kept set"
+            if tok[i] != want:
+                c = torch.cumsum(dist.double(), 0) / dist.double().sum()
+                lo, hi = sorted((tok[i], want))
+                assert abs(float(c[lo]) - u) < 1e-5 or abs(float(c[hi - 1]) - u) < 1e-5, (i, u, tok[i], want)
+            assert float(lg[i]) == float(logits[i, tok[i]])
+
+
+def test_sample_kernel_kept_sets_and_ties():
+    from atoma_infer_amd.kernels import ops
+    vocab = 700
+    logits = torch.zeros(3, vocab)
+    logits[0, [5, 100, 300, 650]] = 3.0                # four tied tokens, top_k = 2 keeps ids 5 and 100
+    logits[1, 7] = 20.0                                # nearly all mass on one token, top_p = 0.5 keeps only it
+    logits[2] = torch.linspace(0, 5, vocab)
+    seen = [set(), set(), set()]
+    for i in range(64):
+        u = (i + 0.5) / 64
+        dev = lambda x, dt: torch.tensor(x, dtype=dt, device="cuda:0")
+        tok, _ = ops.sample(logits.cuda(), dev([1.0, 1.0, 1.0], torch.float32), dev([2, 0, 3], torch.int32),
+                            dev([1.0, 0.5, 1.0], torch.float32), dev([u] * 3, torch.float32))
+        for r, t in enumerate(tok.cpu().tolist()):
+            seen[r].add(t)
+    assert seen[0] == {5, 100} and seen[1] == {7} and seen[2] == {vocab - 3, vocab - 2, vocab - 1}
+
+
+def test_repeat_penalty_kernel_and_temperature_limit():
+    from atoma_infer_amd.kernels import ops
+    from atoma_infer_amd.sampling import Sampler, validate, GenerateParameters
+    logits = torch.tensor([[1.0, -1.0, 2.0, 0.5], [3.0, 1.0, -2.0, 0.0]], device="cuda:0")
+    want0 = plain_llama.repeat_penalty(logits[0].cpu(), 2.0, [0, 1, 1])
+    ops.repeat_penalty(logits, torch.tensor([0, 0], dtype=torch.int32, device="cuda:0"),
+                       torch.tensor([0, 1], dtype=torch.int32, device="cuda:0"),
+                       torch.tensor([2.0, 1.0], device="cuda:0"))
+    assert torch.equal(logits[0].cpu(), want0) and logits[1].cpu().tolist() == [3.0, 1.0, -2.0, 0.0]
+    # through the sampler: the penalty turns the argmax away from a repeated token
+    s = Sampler(torch.device("cuda:0"))
+    lg = torch.tensor([[2.0, 1.9, 0.0]], device="cuda:0")
+    p1 = validate(GenerateParameters(do_sample=False), 3, 100, 200)
+    p2 = validate(GenerateParameters(do_sample=False, repetition_penalty=1.5, repeat_last_n=4), 3, 100, 200)
+    assert s.sample(lg.clone(), [p1], [0], [[0, 0, 0]])[0] == [0]
+    assert s.sample(lg.clone(), [p2], [0], [[0, 0, 0]])[0] == [1]
+    # a very low temperature is greedy in effect
+    p3 = validate(GenerateParameters(temperature=1e-3, random_seed=5), 3, 100, 200)
+    big = torch.randn(1, 2000, generator=torch.Generator().manual_seed(0)).cuda()
+    assert s.sample(big.clone(), [p3], [0], [()])[0] == [int(big.argmax())]
+
+
+# ----------------------------------------------------------------------------------------------------------
+# bin/trace_run as a program
+
+
+def run_trace(model_dir, dtype, steps, out_dir, max_tokens):
+    env = dict(os.environ)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype",
+                           dtype, "--out", out_dir, "--max-tokens", str(max_tokens)],
+                          input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
+                          env=env, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    return proc
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_dirs, tmp_path, dtype):
+    d = model_dirs["B"]
+    vocab = TINY["B"]["vocab_size"]
+    a, b, c = random_tokens(70, vocab, 1), random_tokens(40, vocab, 2), random_tokens(64, vocab, 3)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:33], "want": [0, 32]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[:2], "want": []}, {"id": "a", "tokens": a[33:35], "want": [1]}],
+         "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[35:], "want": [34]}, {"id": "b", "tokens": b[2:], "want": [0, 37]}],
+         "end": ["a", "b"]},
+        {"step": 3, "entries": [{"id": "c", "tokens": c[:63], "want": []}], "end": []},
+        {"step": 4, "entries": [{"id": "c", "tokens": c[63:], "want": [0]}], "end": ["c"]},
+    ]
+    out = str(tmp_path / "out")
+    # a and b round up to 128 + 64 tokens; c reuses their pages
+    run_trace(d, dtype, steps, out, 192)
+    assert sorted(os.listdir(out)) == ["0.f32", "1.f32", "2.f32", "4.f32"]
+    w, cfg = plain_weights(d), plain_config(d)
+    pa, pb, pc = (plain_llama.forward(t, w, cfg) for t in (a, b, c))
+    want = {0: torch.stack([pa[0], pa[32]]), 1: pa[34][None], 2: torch.stack([pa[69], pb[2], pb[39]]), 4: pc[63][None]}
+    for step, ref in want.items():
+        got = torch.from_numpy(np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, vocab))
+        assert got.shape == ref.shape
+        if dtype == "float32":
+            assert rel_err(got, ref) < TOL_F32
+        else:
+            assert frob_err(got, ref) < TOL_BF16

@@ -1,0 +1,397 @@
+"""Each part alone, and the generality of their arrangement: a toy architecture, defined here, whose layers
+differ (attention with and without a window, a mixer with per-request state of its own, another position
+encoding), whose run order names a layer twice and lets a layer read another layer's cache.  It is registered,
+written with random weights, built and stepped without a change to the framework's files."""
+import dataclasses
+import math
+from typing import Dict, List, Optional
+
+import pytest
+import torch
+
+import plain_llama as P
+from util import TINY_B, TOL_BF16, TOL_F32, frob_err, plain_weights, random_tokens, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ----------------------------------------------------------------------------------------------------------
+# parts alone
+
+
+def getter(tensors):
+    return lambda name: tensors[name]
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(act):
+    from atoma_infer_amd.parts import RMSNorm
+    g = torch.Generator().manual_seed(0)
+    w = (1 + 0.1 * torch.randn(100, generator=g)).to(torch.bfloat16)
+    part = RMSNorm(100, 1e-6)
+    assert part.weight_specs()["weight"].shape == (100,)
+    part.load(getter({"weight": w}), torch.device(DEV), act)
+    resid, delta = torch.randn(5, 100, generator=g), torch.randn(5, 100, generator=g).to(act)
+    r = resid.to(DEV)
+    out = part.add_norm(r, delta.to(DEV))
+    want_r = resid + delta.float()
+    assert torch.allclose(r.cpu(), want_r)
+    want = P.rms_norm(want_r, w.float(), 1e-6)
+    assert out.dtype is act
+    assert torch.allclose(out.float().cpu(), want, atol=1e-5 if act is torch.float32 else 2e-2, rtol=1e-2)
+
+
+def test_rotary_part_tables_equal_the_plain_ones():
+    from atoma_infer_amd.parts import RotaryEncoding
+    rs = {k: v for k, v in TINY_B["rope_scaling"].items() if k != "rope_type"}
+    part = RotaryEncoding(32, 500000.0, 256, rs)
+    part.prepare(torch.device(DEV))
+    cos, sin, rd = part.rotary_tables()
+    pc, ps = P.rope_tables(TINY_B, torch.arange(256))
+    assert rd == 32 and torch.equal(cos.cpu(), pc) and torch.equal(sin.cpu(), ps)
+    # apply: equals the plain rotation
+    g = torch.Generator().manual_seed(1)
+    q, k = torch.randn(4, 3, 32, generator=g), torch.randn(4, 2, 32, generator=g)
+    pos = torch.tensor([0, 5, 200, 255], dtype=torch.int32)
+    dq, dk = q.to(DEV), k.to(DEV)
+    part.apply(dq, dk, pos.to(DEV))
+    assert torch.allclose(dq.cpu(), P.apply_rope(q, pc[pos.long()], ps[pos.long()]), atol=1e-6)
+    assert torch.allclose(dk.cpu(), P.apply_rope(k, pc[pos.long()], ps[pos.long()]), atol=1e-6)
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,inter", [(64, 96), (96, 250)])
+def test_swiglu_part(act, width, inter):
+    from atoma_infer_amd.parts import SwiGLU
+    g = torch.Generator().manual_seed(2)
+    ws = {n: (torch.randn(*s, generator=g) * 0.1).to(torch.bfloat16) for n, s in
+          (("gate_proj.weight", (inter, width)), ("up_proj.weight", (inter, width)),
+           ("down_proj.weight", (width, inter)))}
+    part = SwiGLU(width, inter)
+    assert {k: v.shape for k, v in part.weight_specs().items()} == {k: tuple(v.shape) for k, v in ws.items()}
+    part.load(getter(ws), torch.device(DEV), act)
+    x = torch.randn(7, width, generator=g).to(act)
+    y = part.forward(x.to(DEV), None)
+    if y.dim() == 3:
+        y = y.sum(0)
+    want = P.swiglu_mlp(x.float(), {k: v.float() for k, v in ws.items()}, "")
+    err = frob_err(y.float(), want)
+    assert err < (1e-5 if act is torch.float32 else 1e-2), err
+
+
+def test_embedding_and_head_parts():
+    from atoma_infer_amd.parts import OutputHead, TokenEmbedding
+    g = torch.Generator().manual_seed(3)
+    table = (torch.randn(50, 32, generator=g)).to(torch.bfloat16)
+    emb = TokenEmbedding(50, 32)
+    emb.load(getter({"weight": table}), torch.device(DEV), torch.bfloat16)
+    tied = OutputHead(32, 50, tied_to=emb)
+    assert tied.weight_specs() == {}
+    tied.load(getter({}), torch.device(DEV), torch.bfloat16)
+    x = torch.randn(3, 32, generator=g).to(torch.bfloat16)
+    logits = tied.forward(x.to(DEV))
+    assert logits.dtype is torch.float32 and rel_err(logits, x.float() @ table.float().T) < 1e-5
+    own = (torch.randn(50, 32, generator=g)).to(torch.bfloat16)
+    untied = OutputHead(32, 50)
+    assert untied.weight_specs()["weight"].shape == (50, 32)
+    untied.load(getter({"weight": own}), torch.device(DEV), torch.bfloat16)
+    assert rel_err(untied.forward(x.to(DEV)), x.float() @ own.float().T) < 1e-5
+    assert torch.equal(emb.forward(torch.tensor([4, 0, 49], dtype=torch.int32, device=DEV)).cpu(),
+                       table.float()[[4, 0, 49]])
+
+
+def test_part_registries():
+    from atoma_infer_amd.parts import make_part, registered_kinds
+    assert "attention" in registered_kinds("mixer") and "swiglu" in registered_kinds("feed_forward")
+    assert "rmsnorm" in registered_kinds("norm") and {"rotary", "none"} <= set(registered_kinds("position"))
+    with pytest.raises(KeyError):
+        make_part("mixer", "no-such-mixer")
+    with pytest.raises(ValueError):
+        make_part("mixer", "attention", width=64, num_heads=4, num_kv_heads=3, head_size=16)
+    with pytest.raises(ValueError):
+        make_part("mixer", "attention", width=40, num_heads=4, num_kv_heads=4, head_size=10)   # head size refused
+
+
+# ----------------------------------------------------------------------------------------------------------
+# a toy architecture, defined here
+
+
+def _toy_parts():
+    """Parts that exist only in this test: a mixer with state of its own and another position encoding."""
+    from atoma_infer_amd.parts import (Mixer, PositionEncoding, StateSpec, WeightSpec, register_mixer,
+                                       register_position)
+
+    class DecayMixer(Mixer):
+        """state <- decay * state + x W_in (per token, in order); y = state W_out.  State: [inner] per request."""
+
+        def __init__(self, width: int, inner: int, decay: float):
+            self.width, self.inner, self.decay = width, inner, decay
+
+        def weight_specs(self):
+            return {"in_proj.weight": WeightSpec((self.inner, self.width)),
+                    "out_proj.weight": WeightSpec((self.width, self.inner))}
+
+        def state_spec(self):
+            return StateSpec((self.inner,))
+
+        def load(self, get, device, act_dtype):
+            self.w_in = get("in_proj.weight").to(device)
+            self.w_out = get("out_proj.weight").to(device)
+            self.act_dtype = act_dtype
+
+        def forward(self, x, ctx, cache):
+            from atoma_infer_amd.parts import linear
+            u = linear(x, self.w_in, torch.float32)
+            out = torch.empty_like(u)
+            row = 0
+            for e in range(ctx.n_entries):
+                slot, n = int(ctx.h_state_slots[e]), int(ctx.h_counts[e])
+                st = cache.state[slot]
+                for i in range(n):
+                    st.mul_(self.decay).add_(u[row + i])
+                    out[row + i] = st
+                row += n
+            return linear(out.to(self.act_dtype), self.w_out)
+
+    class InterleavedRotary(PositionEncoding):
+        """Rotates neighbouring pairs (2i, 2i+1) instead of half-split ones; no tables for the fused kernel."""
+
+        def __init__(self, head_size: int, theta: float):
+            self.inv = 1.0 / (theta ** (torch.arange(0, head_size, 2).float() / head_size))
+
+        def load(self, get, device, act_dtype):
+            self.inv = self.inv.to(device)
+
+        def apply(self, q, k, positions):
+            ang = positions.float()[:, None] * self.inv[None, :]
+            c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            for x in (q, k):
+                if x.numel() == 0:
+                    continue
+                xf = x.float().clone()   # float() of a float32 tensor is the tensor itself
+                a, b = xf[..., 0::2], xf[..., 1::2]
+                x[..., 0::2] = (a * c - b * s).to(x.dtype)
+                x[..., 1::2] = (b * c + a * s).to(x.dtype)
+
+    register_mixer("toy_decay", DecayMixer, replace=True)
+    register_position("toy_interleaved", InterleavedRotary, replace=True)
+
+
+def _toy_architecture():
+    from atoma_infer_amd.config import ModelConfig, key, register_architecture
+    from atoma_infer_amd.config.base import as_float, as_positive_int
+    from atoma_infer_amd.models import LayerCall, ModelSpec
+    from atoma_infer_amd.parts import OutputHead, TokenEmbedding, make_part
+
+    @dataclasses.dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        architectures = ("ToyMixedForCausalLM",)
+        width: int = key(convert=as_positive_int)
+        vocab: int = key(convert=as_positive_int)
+        heads: int = key(convert=as_positive_int)
+        kv_heads: int = key(convert=as_positive_int)
+        inter: int = key(convert=as_positive_int)
+        eps: float = key(convert=as_float)
+        max_positions: int = key(convert=as_positive_int)
+        layers: tuple = key(convert=lambda v: tuple(dict(x) for x in v))
+        order: tuple = key(convert=lambda v: tuple(dict(x) for x in v))
+
+        def to_dict(self):
+            d = {f.name: getattr(self, f.name) for f in dataclasses.fields(self)}
+            d["layers"], d["order"] = [dict(x) for x in self.layers], [dict(x) for x in self.order]
+            d["architectures"] = ["ToyMixedForCausalLM"]
+            return d
+
+    def build(cfg: ToyConfig) -> ModelSpec:
+        hd = cfg.width // cfg.heads
+        layers = []
+        for i, ld in enumerate(cfg.layers):
+            if ld["mixer"] == "attention":
+                pos = None
+                if ld.get("position") == "rotary":
+                    pos = make_part("position", "rotary", head_size=hd, theta=10000.0, max_positions=cfg.max_positions)
+                elif ld.get("position") == "interleaved":
+                    pos = make_part("position", "toy_interleaved", head_size=hd, theta=100.0)
+                mixer = make_part("mixer", "attention", width=cfg.width, num_heads=cfg.heads,
+                                  num_kv_heads=cfg.kv_heads, head_size=hd, position=pos, window=ld.get("window"))
+            else:
+                mixer = make_part("mixer", "toy_decay", width=cfg.width, inner=ld["inner"], decay=ld["decay"])
+            block = make_part("block", "pre_norm", norm1=make_part("norm", "rmsnorm", width=cfg.width, eps=cfg.eps),
+                              mixer=mixer, norm2=make_part("norm", "rmsnorm", width=cfg.width, eps=cfg.eps),
+                              feed_forward=make_part("feed_forward", "swiglu", width=cfg.width, intermediate=cfg.inter),
+                              names=("norm_a", "mixer", "norm_b", "ffn"))
+            layers.append((f"toy.layers.{i}", block))
+        emb = TokenEmbedding(cfg.vocab, cfg.width)
+        return ModelSpec(width=cfg.width, vocab_size=cfg.vocab, max_positions=cfg.max_positions,
+                         embedding=("toy.embed", emb), layers=layers,
+                         final_norm=("toy.final_norm", make_part("norm", "rmsnorm", width=cfg.width, eps=cfg.eps)),
+                         head=("toy.head", OutputHead(cfg.width, cfg.vocab)),
+                         run_order=[LayerCall(o["layer"], o.get("kv_from")) for o in cfg.order])
+
+    register_architecture("ToyMixedForCausalLM", ToyConfig, build, replace=True)
+
+
+TOY = {
+    "architectures": ["ToyMixedForCausalLM"], "width": 64, "vocab": 211, "heads": 4, "kv_heads": 2, "inter": 96,
+    "eps": 1e-5, "max_positions": 512,
+    "layers": [
+        {"mixer": "attention", "position": "rotary"},                       # 0: all keys
+        {"mixer": "toy_decay", "inner": 40, "decay": 0.9},                  # 1: state of its own
+        {"mixer": "attention", "position": "rotary", "window": 24},         # 2: a window of 24 keys
+        {"mixer": "attention", "position": "interleaved"},                  # 3: another position encoding
+        {"mixer": "attention"},                                             # 4: no position encoding
+    ],
+    # layer 1 runs twice (two states), call 6 reads the cache that call 0 wrote, with layer 4's queries
+    "order": [{"layer": 0}, {"layer": 1}, {"layer": 2}, {"layer": 3}, {"layer": 1}, {"layer": 4},
+              {"layer": 4, "kv_from": 0}],
+}
+
+
+def toy_plain_forward(tokens: List[int], w: Dict[str, torch.Tensor], cfg: dict) -> torch.Tensor:
+    """The toy model on a whole sequence, from the plain implementation's functions."""
+    H, nh, nkv = cfg["width"], cfg["heads"], cfg["kv_heads"]
+    hd, t = H // nh, len(tokens)
+    pos = torch.arange(t)
+    x = w["toy.embed.weight"][torch.tensor(tokens)]
+    kv_of_call = {}
+
+    def encode(ld, q, k):
+        if ld.get("position") == "rotary":
+            c, s = P.rope_tables({"hidden_size": H, "num_attention_heads": nh, "rope_theta": 10000.0}, pos)
+            return P.apply_rope(q, c, s), (P.apply_rope(k, c, s) if k is not None else None)
+        if ld.get("position") == "interleaved":
+            inv = 1.0 / (100.0 ** (torch.arange(0, hd, 2).float() / hd))
+            ang = pos.float()[:, None] * inv[None]
+            c, s = torch.cos(ang)[:, None], torch.sin(ang)[:, None]
+            def rot(z):
+                a, b = z[..., 0::2], z[..., 1::2]
+                out = torch.empty_like(z)
+                out[..., 0::2], out[..., 1::2] = a * c - b * s, b * c + a * s
+                return out
+            return rot(q), (rot(k) if k is not None else None)
+        return q, k
+
+    for ci, call in enumerate(cfg["order"]):
+        li, ld = call["layer"], cfg["layers"][call["layer"]]
+        p = f"toy.layers.{li}."
+        h = P.rms_norm(x, w[p + "norm_a.weight"], cfg["eps"])
+        if ld["mixer"] == "attention":
+            q = (h @ w[p + "mixer.q_proj.weight"].T).view(t, nh, hd)
+            if call.get("kv_from") is None:
+                k = (h @ w[p + "mixer.k_proj.weight"].T).view(t, nkv, hd)
+                v = (h @ w[p + "mixer.v_proj.weight"].T).view(t, nkv, hd)
+                q, k = encode(ld, q, k)
+                kv_of_call[ci] = (k, v)
+            else:
+                q, _ = encode(ld, q, None)
+                k, v = kv_of_call[call["kv_from"]]
+            kk, vv = k.repeat_interleave(nh // nkv, 1), v.repeat_interleave(nh // nkv, 1)
+            o = P.attention_scores_softmax_pv(q.transpose(0, 1), kk.transpose(0, 1), vv.transpose(0, 1),
+                                              1 / math.sqrt(hd), True, ld.get("window"))
+            a = o.transpose(0, 1).reshape(t, H) @ w[p + "mixer.o_proj.weight"].T
+        else:
+            u = h @ w[p + "mixer.in_proj.weight"].T
+            st, ys = torch.zeros(ld["inner"]), []
+            for i in range(t):
+                st = ld["decay"] * st + u[i]
+                ys.append(st)
+            a = torch.stack(ys) @ w[p + "mixer.out_proj.weight"].T
+        x = x + a
+        x = x + P.swiglu_mlp(P.rms_norm(x, w[p + "norm_b.weight"], cfg["eps"]), w, p + "ffn.")
+    return P.rms_norm(x, w["toy.final_norm.weight"], cfg["eps"]) @ w["toy.head.weight"].T
+
+
+@pytest.fixture(scope="module")
+def toy_dir(tmp_path_factory):
+    _toy_parts()
+    _toy_architecture()
+    from atoma_infer_amd.weights import write_random_model
+    d = str(tmp_path_factory.mktemp("toy"))
+    write_random_model(d, TOY, seed=5, dtype="bfloat16", norm_jitter=0.1)
+    yield d
+    from atoma_infer_amd.config import unregister_architecture
+    unregister_architecture("ToyMixedForCausalLM")
+
+
+def test_toy_cache_plan(toy_dir):
+    from atoma_infer_amd.cache import plan_cache
+    from atoma_infer_amd.config import load_model_config
+    arch, cfg = load_model_config(toy_dir)
+    plan = plan_cache(arch.build(cfg))
+    # attention calls 0, 3, 5 keep all keys (one group), call 2 keeps a window (a group of its own),
+    # call 6 reads call 0's entry, calls 1 and 4 each have their own state
+    assert [(g.spec.window, g.calls) for g in plan.groups] == [(None, [0, 3, 5]), (24, [2])]
+    assert plan.where[6] == (0, 0, False) and sorted(plan.states) == [1, 4] and plan.states[1] == (40,)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_steps_like_its_plain_model(toy_dir, dtype):
+    from atoma_infer_amd.cache import CachePool, plan_cache
+    from atoma_infer_amd.engine import ModelRunner, StepEntry
+    from atoma_infer_amd.models import load_model
+    model = load_model(toy_dir, dtype)
+    plan = plan_cache(model.spec)
+    w = plain_weights(toy_dir)
+    reqs = {n: random_tokens(ln, TOY["vocab"], 60 + i) for i, (n, ln) in enumerate([("a", 120), ("b", 75), ("c", 90)])}
+    want = {n: toy_plain_forward(t, w, TOY) for n, t in reqs.items()}
+
+    def run(schedule, pages):
+        pool = CachePool(plan, 16, pages, 3, model.act_dtype, model.device)
+        runner = ModelRunner(model, pool)
+        ids, got = {}, {}
+        for entries, end in schedule:
+            batch, places = [], []
+            for name, n in entries:
+                if name not in ids:
+                    ids[name] = len(ids)
+                    runner.add_request(ids[name])
+                s = runner.computed_len(ids[name])
+                batch.append(StepEntry(ids[name], reqs[name][s:s + n], s, list(range(n))))
+                places += [(name, s + i) for i in range(n)]
+            logits = runner.step(batch).cpu()
+            for r, key in enumerate(places):
+                got[key] = logits[r]
+            for name in end:
+                runner.free_request(ids[name])
+            runner.manager.check()
+        return got, runner
+
+    def check(got):
+        for n in reqs:
+            rows = sorted(p for (m, p) in got if m == n)
+            mine, ref = torch.stack([got[(n, p)] for p in rows]), want[n][rows]
+            if dtype == "float32":
+                assert rel_err(mine, ref) < TOL_F32, n
+            else:
+                assert frob_err(mine, ref) < TOL_BF16, n
+
+    # whole prompts, one request at a time
+    got, _ = run([([(n, len(t))], [n]) for n, t in reqs.items()], [8, 8])
+    check(got)
+    # portions of changing size beside decoded tokens of other requests; the windowed group has so few pages
+    # (12 of 16 tokens, where the three requests would need 19 without giving any back) that it only works because passed pages return
+    sched = [([("a", 50), ("b", 2)], []), ([("a", 1), ("b", 33), ("c", 17)], []), ([("a", 30), ("c", 2)], []),
+             ([("b", 40), ("a", 1), ("c", 1)], ["b"]), ([("a", 38), ("c", 3)], ["a"]), ([("c", 60)], []),
+             ([("c", 1)], []), ([("c", 1)], []), ([("c", 5)], ["c"])]
+    got, runner = run(sched, [19, 12])
+    check(got)
+    assert runner.manager.num_free_pages(0) == 19 and runner.manager.num_free_pages(1) == 12
+
+
+def test_toy_architecture_generates_through_the_engine(toy_dir):
+    from atoma_infer_amd.config import CacheConfig, SchedulerConfig
+    from atoma_infer_amd.engine.engine import LlmEngine
+    from atoma_infer_amd.sampling import GenerateParameters
+    w = plain_weights(toy_dir)
+    prompts = [random_tokens(19, TOY["vocab"], 1), random_tokens(3, TOY["vocab"], 2)]
+    want = []
+    for p in prompts:
+        seq = list(p)
+        for _ in range(5):
+            seq.append(int(torch.argmax(toy_plain_forward(seq, w, TOY)[-1])))
+        want.append(seq[len(p):])
+    eng = LlmEngine(toy_dir, "float32", cache=CacheConfig(block_size=16, num_gpu_blocks_override=8),
+                    scheduler=SchedulerConfig(max_num_batched_tokens=8, max_num_sequences=2, max_model_len=64))
+    outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=5, ignore_eos_token=True))
+    assert [o.inference_outputs[0].token_ids for o in outs] == want
