@@ -7,17 +7,27 @@ come back only for the places asked for, in float32.
 
 The reference's counterpart is ``ModelWorker::execute_model`` with ``prepare_input_tensors``
 (backends/vllm/src/worker.rs:111-191, 224-460); unlike it, a later portion of a prompt sees the earlier ones.
-All integer metadata of a step travels to the device in one pinned buffer and one copy.
+All integer metadata of a step (including what mixers plan for their kernels, such as attention task lists)
+travels to the device in one pinned buffer and one copy.
+
+Steps that only decode (one token per entry, its logits wanted) are launch-bound, so their kernel sequence is
+captured once per (number of entries, context bucket of 256 tokens) into a HIP graph and replayed; between
+replays only the metadata buffer changes.  A shape is run eagerly the first time it is seen and captured the
+second time.
 """
 from __future__ import annotations
 
 import dataclasses
-from typing import Dict, List, Optional, Sequence
+from collections import OrderedDict
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
 from ..cache.pool import CachePool, LayerCache
+
+DECODE_BUCKET = 256      # tokens; a decode graph serves contexts up to a multiple of this
+MAX_GRAPHS = 48
 
 
 class StepError(ValueError):
@@ -59,7 +69,12 @@ class StepContext:
     slot_mappings: List[torch.Tensor] = dataclasses.field(default_factory=list)   # per group [T]
     block_tables: List[torch.Tensor] = dataclasses.field(default_factory=list)    # per group [S, blocks]
     pool: Optional[CachePool] = None
-    scratch: Dict[str, object] = dataclasses.field(default_factory=dict)          # per-step notes of kernels
+    #: what mixers planned for this step: key -> (int32 device tensor, meta)
+    plans: Dict[object, Tuple[torch.Tensor, tuple]] = dataclasses.field(default_factory=dict)
+    #: per-step notes and workspaces of kernels
+    scratch: Dict[object, object] = dataclasses.field(default_factory=dict)
+    #: not None inside a decode graph: the number of 256-token buckets the graph serves
+    decode_bucket: Optional[int] = None
 
     def layer_cache(self, pos: int) -> LayerCache:
         return self.pool.layer_cache(pos, self.slot_mappings, self.block_tables)
@@ -72,13 +87,34 @@ class _Staging:
         self.device = device
         self.host: Optional[torch.Tensor] = None
         self.dev: Optional[torch.Tensor] = None
+        self.pending: Optional[torch.cuda.Event] = None
 
-    def ensure(self, n: int):
+    def ensure(self, n: int) -> np.ndarray:
         if self.host is None or self.host.numel() < n:
+            self.wait()
             cap = max(1024, 1 << (n - 1).bit_length())
             self.host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
             self.dev = torch.empty(cap, dtype=torch.int32, device=self.device)
         return self.host.numpy()
+
+    def wait(self) -> None:
+        """The pinned buffer is reused by every step: wait until the last copy out of it has been read."""
+        if self.pending is not None:
+            self.pending.synchronize()
+            self.pending = None
+
+    def upload(self, n: int) -> None:
+        self.dev[:n].copy_(self.host[:n], non_blocking=True)
+        self.pending = torch.cuda.Event()
+        self.pending.record()
+
+
+@dataclasses.dataclass
+class _Graph:
+    stage: _Staging
+    graph: Optional[torch.cuda.CUDAGraph] = None
+    logits: Optional[torch.Tensor] = None
+    ctx: Optional[StepContext] = None
 
 
 class RunnerCache:
@@ -107,12 +143,20 @@ class RunnerCache:
 class ModelRunner:
     """Owns the model and the cache pool of one GPU and steps batches through them."""
 
-    def __init__(self, model, pool: CachePool):
+    def __init__(self, model, pool: CachePool, use_graphs: bool = True):
         self.model, self.pool = model, pool
         self.manager = pool.manager
+        self.use_graphs = use_graphs
         self._stage = _Staging(model.device)
-        self._pending = None
         self._computed: Dict[int, int] = {}       # request -> tokens in the cache
+        self._graphs: "OrderedDict[Tuple[int, int], _Graph]" = OrderedDict()
+        # planners of the mixers, one per distinct key
+        self._planners: Dict[object, Callable] = {}
+        for _, block in model.spec.layers:
+            plan = getattr(block.mixer, "step_planner", None)
+            got = plan(pool.page_size, pool.dtype) if plan is not None else None
+            if got is not None:
+                self._planners.setdefault(got[0], got[1])
 
     # -- requests ------------------------------------------------------------------------------------
     def add_request(self, request: int) -> int:
@@ -166,13 +210,13 @@ class ModelRunner:
                 if not 0 <= w < n:
                     raise StepError(f"request {e.request}: wanted place {w} outside its {n} tokens")
 
-    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
-        """Reserve pages and build the step's metadata on the device."""
-        self._validate(entries)
-        self.wait_staging()
+    def _build(self, entries: Sequence[StepEntry], stage: _Staging, bucket: Optional[int]) -> StepContext:
+        """Fill ``stage`` with the step's metadata, start its copy to the device and describe it.
+
+        With ``bucket`` (decode graphs) every size is a function of (entries, bucket) alone, so the layout, and
+        with it every device address a captured kernel reads, is the same at every replay.
+        """
         mgr = self.manager
-        for e in entries:
-            mgr.reserve(e.request, e.start + len(e.tokens))
         s = len(entries)
         counts = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=s)
         starts = np.fromiter((e.start for e in entries), dtype=np.int32, count=s)
@@ -181,7 +225,9 @@ class ModelRunner:
         n_want = sum(len(e.want) for e in entries)
         n_groups = len(self.pool.plan.groups)
         max_seq = int((starts + counts).max())
-        max_blocks = -(-max_seq // self.pool.page_size)
+        page = self.pool.page_size
+        max_blocks = -(-max_seq // page) if bucket is None else -(-bucket * DECODE_BUCKET // page)
+        extras = [(key, *fn(starts, counts, bucket)) for key, fn in self._planners.items()]
         # layout of the one staging buffer
         o_tok, o_pos, o_seq = 0, t, 2 * t
         o_qs, o_len, o_slot = 3 * t, 3 * t + s + 1, 3 * t + 2 * s + 1
@@ -189,7 +235,13 @@ class ModelRunner:
         o_sm = o_want + n_want
         o_bt = o_sm + n_groups * t
         total = o_bt + n_groups * s * max_blocks
-        buf = self._stage.ensure(total)
+        ex_off = []
+        for _, arr, _ in extras:
+            total += (-total) % 4                  # every extra starts on a 16-byte boundary
+            ex_off.append(total)
+            total += arr.size
+        stage.wait()
+        buf = stage.ensure(total)
         q_start = np.zeros(s + 1, dtype=np.int32)
         np.cumsum(counts, out=q_start[1:])
         row = 0
@@ -211,10 +263,10 @@ class ModelRunner:
             sm = buf[o_sm + g * t: o_sm + (g + 1) * t]
             bt = buf[o_bt + g * s * max_blocks: o_bt + (g + 1) * s * max_blocks].reshape(s, max_blocks)
             mgr.fill_step(g, ids, starts, counts, sm, bt)
-        dev = self._stage.dev
-        dev[:total].copy_(self._stage.host[:total], non_blocking=True)
-        self._pending = torch.cuda.Event()
-        self._pending.record()
+        for off, (_, arr, _) in zip(ex_off, extras):
+            buf[off: off + arr.size] = arr.reshape(-1)
+        stage.upload(total)
+        dev = stage.dev
         ctx = StepContext(
             n_tokens=t, n_entries=s, n_want=n_want,
             tokens=dev[o_tok: o_tok + t], positions=dev[o_pos: o_pos + t], token_seq=dev[o_seq: o_seq + t],
@@ -224,22 +276,63 @@ class ModelRunner:
             slot_mappings=[dev[o_sm + g * t: o_sm + (g + 1) * t] for g in range(n_groups)],
             block_tables=[dev[o_bt + g * s * max_blocks: o_bt + (g + 1) * s * max_blocks].view(s, max_blocks)
                           for g in range(n_groups)],
-            pool=self.pool)
+            pool=self.pool, decode_bucket=bucket)
+        for off, (key, arr, meta) in zip(ex_off, extras):
+            ctx.plans[key] = (dev[off: off + arr.size].view(arr.shape), meta)
         return ctx
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        """Run one batch; returns float32 logits [wanted places, vocab] (order: entries, then ``want``) or None."""
-        ctx = self.prepare(entries)
-        logits = self.model.forward(ctx)
+    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Check the entries, reserve their pages and build the step's metadata on the device."""
+        self._validate(entries)
+        for e in entries:
+            self.manager.reserve(e.request, e.start + len(e.tokens))
+        return self._build(entries, self._stage, None)
+
+    def _finish(self, entries: Sequence[StepEntry]) -> None:
         for e in entries:
             done = e.start + len(e.tokens)
             self._computed[e.request] = done
             self.manager.release_behind(e.request, done)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one batch; returns float32 logits [wanted places, vocab] (order: entries, then ``want``) or None.
+
+        The tensor returned by a decode step belongs to that step's graph and is overwritten by the next step of
+        the same shape: use it (sample, copy) before stepping again.
+        """
+        self._validate(entries)
+        for e in entries:
+            self.manager.reserve(e.request, e.start + len(e.tokens))
+        logits = None
+        if self.use_graphs and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries):
+            logits = self._decode_with_graph(entries)
+        if logits is None:
+            ctx = self._build(entries, self._stage, None)
+            logits = self.model.forward(ctx)
+        self._finish(entries)
         return logits
 
+    def _decode_with_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        s = len(entries)
+        max_seq = max(e.start for e in entries) + 1
+        key = (s, -(-max_seq // DECODE_BUCKET))
+        g = self._graphs.get(key)
+        if g is None:
+            # first sight of this shape: run it eagerly (which also loads every kernel it needs)
+            self._graphs[key] = _Graph(_Staging(self.model.device))
+            while len(self._graphs) > MAX_GRAPHS:
+                self._graphs.popitem(last=False)
+            return None
+        self._graphs.move_to_end(key)
+        ctx = self._build(entries, g.stage, key[1])
+        if g.graph is None:
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out = self.model.forward(ctx)
+            g.graph, g.logits, g.ctx = graph, out, ctx
+        g.graph.replay()
+        return g.logits
+
     def wait_staging(self):
-        """The pinned metadata buffer is reused by every step: wait until the last copy out of it has been read."""
-        ev = getattr(self, "_pending", None)
-        if ev is not None:
-            ev.synchronize()
-            self._pending = None
+        self._stage.wait()

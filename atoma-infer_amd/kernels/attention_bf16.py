@@ -12,7 +12,7 @@ shared by all layers with the same grouping and window.
 from __future__ import annotations
 
 import ctypes
-from typing import Dict, Tuple
+from typing import Dict, Optional, Tuple
 
 import numpy as np
 import torch
@@ -39,13 +39,16 @@ def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
     return _libs[hd]
 
 
-def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int) -> Tuple[np.ndarray, int, int, int]:
+def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket: Optional[int] = None,
+                ) -> Tuple[np.ndarray, Tuple[int, int, int]]:
     """Task records [n, 8] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials).
 
     Main tasks are padded to a multiple of 4 (one workgroup runs 4) and ordered so that tasks sharing keys are
-    neighbours and long tasks come first.
+    neighbours and long tasks come first.  With ``bucket`` (decode graphs: one token per entry) every entry is
+    split and owns ``bucket`` chunk slots, used or not, so all counts depend on (entries, bucket) alone.
     """
     qt_max = max(1, 128 // group)
+    null = (-1, 0, 1, 0, 0, 0, -1, 0)
     direct, split, combine = [], [], []
     n_part = 0
     for e in range(len(starts)):
@@ -54,31 +57,38 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int)
         qt = min(qt_max, count)
         rows = qt * group
         first_key = max(0, start - window + 1) if window > 0 else 0
-        do_split = count <= SPLIT_MAX_TOKENS and (k_end_all - first_key) >= SPLIT_MIN_KEYS
+        do_split = bucket is not None or (count <= SPLIT_MAX_TOKENS and (k_end_all - first_key) >= SPLIT_MIN_KEYS)
         for tok0 in range(0, count, qt):
             last = min(tok0 + qt, count)
             k_end = start + last
             lo = max(0, start + tok0 - window + 1) if window > 0 else 0
             if do_split:
-                c0 = (lo // CHUNK) * CHUNK
-                chunks = list(range(c0, k_end, CHUNK))
+                c_first, c_last = lo // CHUNK, (k_end - 1) // CHUNK
+                slots = bucket if bucket is not None else c_last + 1
                 for row0 in range(0, rows, 32):
-                    combine.append((e, tok0, qt, row0, 0, 0, n_part, len(chunks)))
-                    for kb in chunks:
-                        split.append((e, tok0, qt, row0, kb, min(kb + CHUNK, k_end), n_part, 0))
-                        n_part += 1
+                    combine.append((e, tok0, qt, row0, 0, 0, n_part + c_first, c_last - c_first + 1))
+                    for c in range(slots):
+                        if c_first <= c <= c_last:
+                            split.append((e, tok0, qt, row0, c * CHUNK, min((c + 1) * CHUNK, k_end), n_part + c, 0))
+                        elif bucket is not None:
+                            split.append(null)
+                    n_part += slots
             else:
                 kb = (lo // 32) * 32
                 wave_tasks = [(e, tok0, qt, row0, kb, k_end, -1, 0) for row0 in range(0, rows, 32)]
                 while len(wave_tasks) % 4:
-                    wave_tasks.append((-1, 0, 1, 0, 0, 0, -1, 0))
+                    wave_tasks.append(null)
                 direct.append((k_end - kb, wave_tasks))
     direct.sort(key=lambda x: -x[0])
     main = [t for _, ws in direct for t in ws] + split
     while len(main) % 4:
-        main.append((-1, 0, 1, 0, 0, 0, -1, 0))
+        main.append(null)
     arr = np.asarray(main + combine, dtype=np.int32).reshape(-1, 8)
-    return arr, len(main), len(combine), n_part
+    return arr, (len(main), len(combine), n_part)
+
+
+def plan_key(group: int, window: int):
+    return ("attention_mfma_tasks", group, window)
 
 
 def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, hd) -> bool:
@@ -88,14 +98,16 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
     if q.stride(0) % 8 or q.data_ptr() % 16 or out.stride(0) % 4:
         return False
     group = nh // nkv
-    key = ("attention_tasks", group, window)
-    plan = ctx.scratch.get(key)
+    plan = getattr(ctx, "plans", {}).get(plan_key(group, window))
     if plan is None:
-        arr, n_main, n_comb, n_part = build_tasks(ctx.h_starts, ctx.h_counts, group, window)
-        tasks = torch.from_numpy(arr).to(q.device, non_blocking=False)
-        plan = (tasks, n_main, n_comb, n_part)
-        ctx.scratch[key] = plan
-    tasks, n_main, n_comb, n_part = plan
+        # a caller without a step planner (a kernel test): plan here and now
+        key = ("attention_tasks_adhoc", group, window)
+        plan = ctx.scratch.get(key)
+        if plan is None:
+            arr, meta = build_tasks(ctx.h_starts, ctx.h_counts, group, window)
+            plan = (torch.from_numpy(arr).to(q.device), meta)
+            ctx.scratch[key] = plan
+    tasks, (n_main, n_comb, n_part) = plan
     part_o = part_lse = None
     if n_part:
         ws_key = ("attention_partials", nkv, hd)

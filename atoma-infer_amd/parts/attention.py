@@ -62,6 +62,16 @@ class PagedAttention(Mixer):
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
 
+    def step_planner(self, page_size: int, cache_dtype: torch.dtype):
+        """(key, fn(starts, counts, bucket) -> (int32 array, meta)): the task list of the MFMA attention kernels,
+        built once per step on the host and shipped with the step's metadata."""
+        from ..kernels import attention_bf16
+        if cache_dtype is not torch.bfloat16 or page_size != attention_bf16.PAGE:
+            return None
+        group, window = self.nh // self.nkv, self.window or 0
+        return (attention_bf16.plan_key(group, window),
+                lambda starts, counts, bucket: attention_bf16.build_tasks(starts, counts, group, window, bucket))
+
     # -- execution ------------------------------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         nh, nkv, hd = self.nh, self.nkv, self.hd

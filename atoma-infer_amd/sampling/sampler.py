@@ -48,16 +48,19 @@ class Sampler:
                 uniq = set(contexts[i][-pl.repeat_last_n:])
                 pen_rows += [i] * len(uniq)
                 pen_toks += list(uniq)
-        meta = np.zeros((4, s), dtype=np.float32)
+        # one packed upload: temperature, top_p, uniform, penalty (float32) and top_k (int32 bits)
+        meta = np.zeros((5, s), dtype=np.float32)
+        top_k = meta[4].view(np.int32)
         for i, pl in enumerate(plans):
             meta[0, i] = 0.0 if pl.greedy else pl.temperature
             meta[1, i] = pl.top_p
-            meta[2, i] = uniform(pl.random_seed, steps[i])
+            meta[2, i] = uniform(pl.random_seed, steps[i]) if not pl.greedy else 0.0
             meta[3, i] = pl.repetition_penalty
+            top_k[i] = pl.top_k
         m = torch.from_numpy(meta).to(self.device)
-        top_k = torch.tensor([pl.top_k for pl in plans], dtype=torch.int32, device=self.device)
         if pen_rows:
-            ops.repeat_penalty(logits, torch.tensor(pen_rows, dtype=torch.int32, device=self.device),
-                               torch.tensor(pen_toks, dtype=torch.int32, device=self.device), m[3].contiguous())
-        tok, lg = ops.sample(logits, m[0].contiguous(), top_k, m[1].contiguous(), m[2].contiguous())
-        return tok.cpu().tolist(), lg.cpu().tolist()
+            pen = torch.tensor([pen_rows, pen_toks], dtype=torch.int32, device=self.device)
+            ops.repeat_penalty(logits, pen[0], pen[1], m[3])
+        tok, lg = ops.sample(logits, m[0], m[4].view(torch.int32), m[1], m[2])
+        both = torch.stack([tok.view(torch.float32), lg]).cpu()      # one download
+        return both[0].view(torch.int32).tolist(), both[1].tolist()

@@ -199,3 +199,52 @@ def test_first_tokens_and_long_decoding(model_dirs, dtype):
     from atoma_infer_amd.engine import StepEntry, StepError
     with pytest.raises(StepError):
         runner.step([StepEntry(0, [1], n, [0])])  # beyond max_position_embeddings
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_decode_graphs_replay_like_eager_steps(model_dirs, name, dtype):
+    """Decode steps are captured into HIP graphs.  Every replay is compared with the same step run eagerly, with
+    eager work (prompt portions of another request, frees, new requests) and synchronisations between replays."""
+    from atoma_infer_amd.engine import StepEntry
+    vocab = TINY[name]["vocab_size"]
+    toks = {r: random_tokens(n, vocab, 70 + i) for i, (r, n) in enumerate([("a", 90), ("b", 60), ("c", 50)])}
+    graphed = make_runner(model_dirs[name], dtype, PAGE[name], 32)
+    eager = make_runner(model_dirs[name], dtype, PAGE[name], 32)
+    eager.use_graphs = False
+    for rn in (graphed, eager):
+        for i in range(3):
+            rn.add_request(i)
+    ids = {"a": 0, "b": 1, "c": 2}
+
+    def both(entries):
+        outs = []
+        for rn in (graphed, eager):
+            batch = [StepEntry(ids[r], toks[r][rn.computed_len(ids[r]):rn.computed_len(ids[r]) + n],
+                               rn.computed_len(ids[r]), [n - 1]) for r, n in entries]
+            outs.append(rn.step(batch).cpu())
+        return outs
+
+    g, e = both([("a", 40), ("b", 20)])
+    assert torch.equal(g, e)
+    replays = 0
+    for step in range(25):
+        g, e = both([("a", 1), ("b", 1)])          # the same shape again and again: captured, then replayed
+        assert torch.equal(g, e), f"decode step {step}"
+        replays += 1
+        if step % 6 == 2:                          # eager work between replays
+            g, e = both([("c", 7)])
+            assert torch.equal(g, e)
+        if step == 12:
+            torch.cuda.synchronize()
+    assert (2, 1) in graphed._graphs and graphed._graphs[(2, 1)].graph is not None
+    assert not eager._graphs
+    # three decoding requests: another graph; then back to two
+    for step in range(4):
+        g, e = both([("a", 1), ("b", 1), ("c", 1)])
+        assert torch.equal(g, e)
+    g, e = both([("b", 1), ("a", 1)])
+    assert torch.equal(g, e)
+    # and all of it equals the plain model
+    got = {("a", graphed.computed_len(0) - 1): g[1], ("b", graphed.computed_len(1) - 1): g[0]}
+    check_against_plain(model_dirs[name], {k: v for k, v in toks.items() if k != "c"}, got, dtype)
