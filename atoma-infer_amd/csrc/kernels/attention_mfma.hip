@@ -7,9 +7,10 @@
 // kernels: csrc/src/lib.rs:69-100).  The four waves of a workgroup run four consecutive tasks; the host orders
 // tasks so that these read the same keys (the heads of one tile, or neighbouring key ranges of one request) and
 // meet in the L1 cache.  A task either covers all keys its rows may see and writes the output, or covers one
-// 256-key chunk and writes a partial result (normalised output and log-sum-exp) that the combine kernel merges:
+// chunk of 64 to 256 keys and writes a partial result (normalised output and log-sum-exp) that the combine kernel merges:
 // the split keeps the GPU busy when few rows face many keys (csrc/kernels/flash_fwd_kernel.h:1131-1310 is the
-// reference's combine).  The cut depends only on the request's own lengths, never on the rest of the batch.
+// reference's combine).  Chunk borders are multiples of the chunk size, so a partial result covers the same keys
+// whatever else the batch holds.
 //
 // Per block of 32 keys (two pages), with v_mfma_f32_32x32x16_bf16:
 //   S^T[key, row] = K[key, :] . Q[row, :]     K page rows are the A operand straight from global memory,
@@ -47,6 +48,10 @@ struct Task {
   int32_t k_end;
   int32_t dest;     // < 0: write the output; else index of the partial result
   int32_t n_parts;  // combine tasks: number of partial results starting at dest
+  int32_t tok_base; // row of the entry's first token in the step's batch
+  int32_t count;    // tokens of the entry in this step
+  int32_t pos0;     // absolute position of the entry's first token
+  int32_t pad;
 };
 
 __device__ __forceinline__ bf16x8 pack8(const float* v) {
@@ -60,8 +65,7 @@ __global__ void __launch_bounds__(256)
 attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
                       const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
                       float* __restrict__ part_o, float* __restrict__ part_lse, const Task* __restrict__ tasks,
-                      int n_tasks, const int32_t* __restrict__ block_tables, int max_blocks,
-                      const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions, float scale,
+                      int n_tasks, const int32_t* __restrict__ block_tables, int max_blocks, float scale,
                       int window, int nh, int nkv) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ti = blockIdx.x * 4 + wave;
@@ -75,11 +79,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   // this lane's row
   const int r = task.row0 + c;
   const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
-  const int tok_base = q_start[task.entry];
-  const int count = q_start[task.entry + 1] - tok_base;
-  const bool row_ok = hq < g && tok < count;
-  const int trow = tok_base + (row_ok ? tok : 0);
-  const int p_row = row_ok ? positions[trow] : -1;
+  const bool row_ok = hq < g && tok < task.count;
+  const int trow = task.tok_base + (row_ok ? tok : 0);
+  const int p_row = row_ok ? task.pos0 + tok : -1;
   const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
   const int head = kvh * g + (row_ok ? hq : 0);
 
@@ -103,32 +105,28 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const size_t kv_head_stride = (size_t)PAGE * HD;            // one (page, head) tile
   const size_t page_stride = (size_t)nkv * kv_head_stride;
 
-  for (int kb = task.k_begin; kb < task.k_end; kb += 32) {
+  // keys and values of a block are fetched one block ahead (while the previous block's softmax runs) when
+  // registers allow
+  constexpr bool PREFETCH = HD <= 128;
+  auto pages_of = [&](int kb, int& p0, int& p1) {
     int b0 = kb / PAGE, b1 = b0 + 1;
     if (b0 > max_blocks - 1) b0 = max_blocks - 1;
     if (b1 > max_blocks - 1) b1 = max_blocks - 1;
-    const int pg0 = table[b0], pg1 = table[b1];
-
-    // S^T = K Q^T
-    f32x16 s;
+    p0 = table[b0];
+    p1 = table[b1];
+  };
+  auto load_keys = [&](int p0, int p1, bf16x8* kf) {
+    const int pg = (c < 16) ? p0 : p1;
+    const uint16_t* kp = kcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride + (size_t)(c & 15) * HD +
+                         hg * 8;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    {
-      const int pg = (c < 16) ? pg0 : pg1;
-      const uint16_t* kp = kcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride + (size_t)(c & 15) * HD +
-                           hg * 8;
-#pragma unroll
-      for (int st = 0; st < KSTEPS; ++st) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + st * 16);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
-      }
-    }
-
-    // V^T fragments for both pages, issued before the softmax so that their latency hides behind it
-    bf16x8 vf[2][DTILES];
+    for (int st = 0; st < KSTEPS; ++st) kf[st] = *reinterpret_cast<const bf16x8*>(kp + st * 16);
+  };
+  // V^T fragments of both pages: lane (d = dt*32 + c, key slots hg*4..+4 and 8 + hg*4..+4 of each page)
+  auto load_vals = [&](int p0, int p1, bf16x8 (*vf)[DTILES]) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int pg = j ? pg1 : pg0;
+      const int pg = j ? p1 : p0;
 #pragma unroll
       for (int dt = 0; dt < DTILES; ++dt) {
         const int d = dt * 32 + c;
@@ -142,6 +140,31 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
 #pragma unroll
           for (int i = 0; i < 8; ++i) vf[j][dt][i] = (__bf16)0.f;
         }
+      }
+    }
+  };
+  int pg0 = 0, pg1 = 0;
+  bf16x8 kf[KSTEPS];
+  bf16x8 vf[2][DTILES], vn[2][DTILES];
+  if (task.k_begin < task.k_end) {
+    pages_of(task.k_begin, pg0, pg1);
+    load_keys(pg0, pg1, kf);
+    load_vals(pg0, pg1, vf);
+  }
+
+  for (int kb = task.k_begin; kb < task.k_end; kb += 32) {
+    // S^T = K Q^T
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[st], s, 0, 0, 0);
+    const bool has_next = kb + 32 < task.k_end;
+    if (has_next) {
+      pages_of(kb + 32, pg0, pg1);
+      if (PREFETCH) {
+        load_keys(pg0, pg1, kf);
+        load_vals(pg0, pg1, vn);
       }
     }
 
@@ -177,6 +200,17 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[0][dt], p0, o[dt], 0, 0, 0);
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[1][dt], p1, o[dt], 0, 0, 0);
+    }
+    if (has_next) {
+      if (PREFETCH) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int dt = 0; dt < DTILES; ++dt) vf[j][dt] = vn[j][dt];
+      } else {
+        load_keys(pg0, pg1, kf);
+        load_vals(pg0, pg1, vf);
+      }
     }
   }
 
@@ -217,39 +251,35 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
 }
 
 // Merge partial results: out = sum_s w_s O_s / sum_s w_s with w_s = exp2(lse_s - max lse).
-// One block per (combine task, KV head): 32 rows x 8 threads, each thread HD/8 values of its row.
+// One block per (combine task, KV head).  The valid rows of the task (group x tokens, at most 32) times HD
+// output values are spread over the 256 threads; the partial results of one value are added in order of their
+// index, with the loads of several parts in flight.
 __global__ void __launch_bounds__(256)
 attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
-                         uint16_t* __restrict__ out, int out_stride, const Task* __restrict__ tasks,
-                         const int32_t* __restrict__ q_start, int nh, int nkv) {
+                         uint16_t* __restrict__ out, int out_stride, const Task* __restrict__ tasks, int nh,
+                         int nkv) {
   const Task task = tasks[blockIdx.x];
   if (task.entry < 0) return;
   const int kvh = blockIdx.y, g = nh / nkv;
-  const int c = threadIdx.x >> 3, sub = threadIdx.x & 7;
-  const int r = task.row0 + c;
-  const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
-  const int tok_base = q_start[task.entry];
-  const int count = q_start[task.entry + 1] - tok_base;
-  if (hq >= g || tok >= count) return;
-  float mx = -INFINITY;
-  for (int s = 0; s < task.n_parts; ++s)
-    mx = fmaxf(mx, part_lse[((size_t)(task.dest + s) * nkv + kvh) * 32 + c]);
-  float acc[HD / 8];
-#pragma unroll
-  for (int i = 0; i < HD / 8; ++i) acc[i] = 0.f;
-  float wsum = 0.f;
-  for (int s = 0; s < task.n_parts; ++s) {
-    const size_t base = ((size_t)(task.dest + s) * nkv + kvh) * 32 + c;
-    const float w = __builtin_amdgcn_exp2f(part_lse[base] - mx);  // lse = -inf gives weight 0
-    wsum += w;
-    const float* po = part_o + base * HD;
-#pragma unroll
-    for (int i = 0; i < HD / 8; ++i) acc[i] += w * po[sub + i * 8];
+  const int tok_base = task.tok_base, count = task.count;
+  const size_t part_stride = (size_t)nkv * 32;   // rows between two partial results of the same (KV head, row)
+  for (int idx = threadIdx.x; idx < 32 * HD; idx += 256) {
+    const int c = idx / HD, d = idx % HD;
+    const int r = task.row0 + c;
+    const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
+    if (hq >= g || tok >= count) continue;
+    const size_t base = ((size_t)task.dest * nkv + kvh) * 32 + c;
+    float mx = -INFINITY;
+    for (int s = 0; s < task.n_parts; ++s) mx = fmaxf(mx, part_lse[base + s * part_stride]);
+    float acc = 0.f, wsum = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < task.n_parts; ++s) {
+      const float w = __builtin_amdgcn_exp2f(part_lse[base + s * part_stride] - mx);  // lse = -inf: weight 0
+      wsum += w;
+      acc += w * part_o[(base + s * part_stride) * HD + d];
+    }
+    out[(size_t)(tok_base + tok) * out_stride + (size_t)(kvh * g + hq) * HD + d] = f32_to_bf16_bits(acc / wsum);
   }
-  const float inv = 1.0f / wsum;
-  uint16_t* op = out + (size_t)(tok_base + tok) * out_stride + (size_t)(kvh * g + hq) * HD;
-#pragma unroll
-  for (int i = 0; i < HD / 8; ++i) op[sub + i * 8] = f32_to_bf16_bits(acc[i] * inv);
 }
 
 extern "C" int atoma_attention_mfma_head_size() { return HD; }
@@ -257,9 +287,8 @@ extern "C" int atoma_attention_mfma_head_size() { return HD; }
 // tasks: device array of n_tasks Task records (main kernel), followed by n_combine records for the combine kernel.
 extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kcache, const void* vcache, void* out,
                                     int out_stride, float* part_o, float* part_lse, const int32_t* tasks, int n_tasks,
-                                    int n_combine, const int32_t* block_tables, int max_blocks,
-                                    const int32_t* q_start, const int32_t* positions, float scale, int window,
-                                    int nh, int nkv, hipStream_t stream) {
+                                    int n_combine, const int32_t* block_tables, int max_blocks, float scale,
+                                    int window, int nh, int nkv, hipStream_t stream) {
   if (n_tasks <= 0) return 0;
   if (nkv <= 0 || nh % nkv || nkv > 65535 || max_blocks <= 0 || (q_stride & 7) || (out_stride & 3) ||
       ((uintptr_t)q & 15) || ((uintptr_t)out & 7))
@@ -267,11 +296,11 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
   const Task* t = reinterpret_cast<const Task*>(tasks);
   hipLaunchKernelGGL(attention_mfma_kernel, dim3((n_tasks + 3) / 4, nkv), dim3(256), 0, stream, (const uint16_t*)q,
                      q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride, part_o,
-                     part_lse, t, n_tasks, block_tables, max_blocks, q_start, positions, scale, window, nh, nkv);
+                     part_lse, t, n_tasks, block_tables, max_blocks, scale, window, nh, nkv);
   ATOMA_LAUNCH_CHECK();
   if (n_combine > 0) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(n_combine, nkv), dim3(256), 0, stream, part_o, part_lse,
-                       (uint16_t*)out, out_stride, t + n_tasks, q_start, nh, nkv);
+                       (uint16_t*)out, out_stride, t + n_tasks, nh, nkv);
     ATOMA_LAUNCH_CHECK();
   }
   return 0;

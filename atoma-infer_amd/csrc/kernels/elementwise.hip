@@ -63,19 +63,110 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   }
 }
 
+// The same for rows of at most 4096 columns, a multiple of 4, with 16-byte aligned rows: every thread keeps its
+// values in registers between the two passes and all loads of a pass are issued together.
+struct f4 { float v[4]; };
+__device__ __forceinline__ f4 load4(const float* p) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  return f4{{t.x, t.y, t.z, t.w}};
+}
+__device__ __forceinline__ f4 load4(const bf16_t* p) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  return f4{{bf16_bits_to_f32((uint16_t)(t.x & 0xffff)), bf16_bits_to_f32((uint16_t)(t.x >> 16)),
+             bf16_bits_to_f32((uint16_t)(t.y & 0xffff)), bf16_bits_to_f32((uint16_t)(t.y >> 16))}};
+}
+__device__ __forceinline__ void store4(float* p, const f4& a) {
+  *reinterpret_cast<float4*>(p) = make_float4(a.v[0], a.v[1], a.v[2], a.v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const f4& a) {
+  uint2 t;
+  t.x = (uint32_t)f32_to_bf16_bits(a.v[0]) | ((uint32_t)f32_to_bf16_bits(a.v[1]) << 16);
+  t.y = (uint32_t)f32_to_bf16_bits(a.v[2]) | ((uint32_t)f32_to_bf16_bits(a.v[3]) << 16);
+  *reinterpret_cast<uint2*>(p) = t;
+}
+
+template <typename TD, typename TW, typename TO>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_vec_kernel(float* __restrict__ resid, const TD* __restrict__ delta, const TW* __restrict__ w,
+                       TO* __restrict__ out, const int32_t* __restrict__ rows, int width, float eps, int planes,
+                       size_t plane_stride) {
+  constexpr int MAXJ = 4;
+  __shared__ float scratch[4];
+  const int r = blockIdx.x;
+  const size_t src = (size_t)(rows ? rows[r] : r) * width, dst = (size_t)r * width;
+  const int n4 = width >> 2;
+  f4 v[MAXJ];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) v[j] = load4(resid + src + 4 * c);
+  }
+  if (delta) {
+    for (int p = 0; p < planes; ++p) {
+      f4 d[MAXJ];
+#pragma unroll
+      for (int j = 0; j < MAXJ; ++j) {
+        const int c = threadIdx.x + j * 256;
+        if (c < n4) d[j] = load4(delta + p * plane_stride + src + 4 * c);
+      }
+#pragma unroll
+      for (int j = 0; j < MAXJ; ++j) {
+        const int c = threadIdx.x + j * 256;
+        if (c < n4)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[j].v[i] += d[j].v[i];
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) {
+      if (delta && !rows) store4(resid + src + 4 * c, v[j]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss += v[j].v[i] * v[j].v[i];
+    }
+  }
+  ss = block_sum<4>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) {
+      const f4 wv = load4(w + 4 * c);
+      f4 o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o.v[i] = v[j].v[i] * inv * wv.v[i];
+      store4(out + dst + 4 * c, o);
+    }
+  }
+}
+
 template <typename TD, typename TW>
 static int add_rmsnorm_out(float* resid, const TD* delta, const TW* w, void* out, int out_dtype, const int32_t* rows,
                            int n_rows, int width, float eps, int planes, size_t plane_stride,
                            hipStream_t stream) {
   dim3 grid(n_rows), block(256);
-  if (out_dtype == kF32)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, float>), grid, block, 0, stream, resid, delta, w, (float*)out,
-                       rows, width, eps, planes, plane_stride);
-  else if (out_dtype == kBF16)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, bf16_t>), grid, block, 0, stream, resid, delta, w,
-                       (bf16_t*)out, rows, width, eps, planes, plane_stride);
-  else
+  const bool vec = width % 4 == 0 && width <= 4096 && ((uintptr_t)resid & 15) == 0 && ((uintptr_t)delta & 15) == 0 &&
+                   ((uintptr_t)w & 15) == 0 && ((uintptr_t)out & 15) == 0 && plane_stride % 4 == 0;
+  if (out_dtype == kF32) {
+    if (vec)
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, float>), grid, block, 0, stream, resid, delta, w,
+                         (float*)out, rows, width, eps, planes, plane_stride);
+    else
+      hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, float>), grid, block, 0, stream, resid, delta, w, (float*)out,
+                         rows, width, eps, planes, plane_stride);
+  } else if (out_dtype == kBF16) {
+    if (vec)
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, bf16_t>), grid, block, 0, stream, resid, delta, w,
+                         (bf16_t*)out, rows, width, eps, planes, plane_stride);
+    else
+      hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, bf16_t>), grid, block, 0, stream, resid, delta, w,
+                         (bf16_t*)out, rows, width, eps, planes, plane_stride);
+  } else {
     return ATOMA_ERR_DTYPE;
+  }
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
@@ -114,52 +205,47 @@ extern "C" int atoma_add_rmsnorm(float* resid, const void* delta, int delta_dtyp
 // csrc/kernels/cache_manager.cu:151-155).  cos/sin may be null: then nothing is rotated.
 // Pairing and signs: csrc/kernels/rotary.h:116-131; rotation applies to q and k only: models/src/llama.rs:298-299.
 template <typename TA, typename TC>
-__global__ void rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __restrict__ positions,
-                                        const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-                                        int rotary_dim, TC* __restrict__ kcache, TC* __restrict__ vcache,
-                                        const int32_t* __restrict__ slot_mapping, int page_size, int nh, int nkv,
-                                        int hd) {
-  const int t = blockIdx.x;
-  TA* row = qkv + (size_t)t * row_stride;
-  const int half = rotary_dim / 2;
+__global__ void __launch_bounds__(64)
+rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __restrict__ positions,
+                        const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim,
+                        TC* __restrict__ kcache, TC* __restrict__ vcache, const int32_t* __restrict__ slot_mapping,
+                        int page_size, int nh, int nkv, int hd) {
+  // one block of 64 threads per (token, head): q heads, then k heads, then v heads
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  TA* x = qkv + (size_t)t * row_stride + (size_t)head * hd;
   const int slot = (kcache && slot_mapping) ? slot_mapping[t] : -1;
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
-  const float* cs = cos_t ? cos_t + (size_t)positions[t] * half : nullptr;
-  const float* sn = sin_t ? sin_t + (size_t)positions[t] * half : nullptr;
-
-  // rotated pairs of q and k
-  const int n_rot = cs ? (nh + nkv) * half : 0;
-  for (int it = threadIdx.x; it < n_rot; it += blockDim.x) {
-    const int head = it / half, i = it % half;
-    TA* x = row + (size_t)head * hd;
-    const float x1 = to_f32(x[i]), x2 = to_f32(x[i + half]);
-    const float c = cs[i], s = sn[i];
-    const float o1 = x1 * c - x2 * s, o2 = x2 * c + x1 * s;
-    if (head < nh) {
-      x[i] = from_f32<TA>(o1);
-      x[i + half] = from_f32<TA>(o2);
-    } else if (slot >= 0) {
-      const int kvh = head - nh;
-      TC* dst = kcache + (((size_t)page * nkv + kvh) * page_size + off) * hd;
-      dst[i] = from_f32<TC>(o1);
-      dst[i + half] = from_f32<TC>(o2);
+  if (head >= nh + nkv) {
+    // v: stored transposed inside the page
+    if (slot < 0) return;
+    const int kvh = head - nh - nkv;
+    TC* dst = vcache + ((size_t)page * nkv + kvh) * hd * page_size + off;
+    for (int i = lane; i < hd; i += 64) dst[(size_t)i * page_size] = from_f32<TC>(to_f32(x[i]));
+    return;
+  }
+  const bool is_k = head >= nh;
+  if (is_k && slot < 0) return;
+  TC* kdst = is_k ? kcache + (((size_t)page * nkv + (head - nh)) * page_size + off) * hd : nullptr;
+  const int half = cos_t ? rotary_dim / 2 : 0;
+  if (half) {
+    const float* cs = cos_t + (size_t)positions[t] * half;
+    const float* sn = sin_t + (size_t)positions[t] * half;
+    for (int i = lane; i < half; i += 64) {
+      const float x1 = to_f32(x[i]), x2 = to_f32(x[i + half]);
+      const float c = cs[i], sv = sn[i];
+      const float o1 = x1 * c - x2 * sv, o2 = x2 * c + x1 * sv;
+      if (is_k) {
+        kdst[i] = from_f32<TC>(o1);
+        kdst[i + half] = from_f32<TC>(o2);
+      } else {
+        x[i] = from_f32<TA>(o1);
+        x[i + half] = from_f32<TA>(o2);
+      }
     }
   }
-  if (slot < 0) return;
   // the part of k that is not rotated (all of it without tables)
-  const int rd = cs ? rotary_dim : 0;
-  const int tail = hd - rd;
-  for (int it = threadIdx.x; it < nkv * tail; it += blockDim.x) {
-    const int kvh = it / tail, i = rd + it % tail;
-    kcache[(((size_t)page * nkv + kvh) * page_size + off) * hd + i] =
-        from_f32<TC>(to_f32(row[(size_t)(nh + kvh) * hd + i]));
-  }
-  // v, transposed inside the page
-  for (int it = threadIdx.x; it < nkv * hd; it += blockDim.x) {
-    const int kvh = it / hd, i = it % hd;
-    vcache[(((size_t)page * nkv + kvh) * hd + i) * page_size + off] =
-        from_f32<TC>(to_f32(row[(size_t)(nh + nkv + kvh) * hd + i]));
-  }
+  if (is_k)
+    for (int i = 2 * half + lane; i < hd; i += 64) kdst[i] = from_f32<TC>(to_f32(x[i]));
 }
 
 extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, const int32_t* positions,
@@ -169,7 +255,9 @@ extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, 
   if (n_tokens <= 0) return 0;
   if (rotary_dim < 0 || rotary_dim > hd || (rotary_dim & 1) || row_stride < (nh + 2 * nkv) * hd || page_size <= 0)
     return ATOMA_ERR_SHAPE;
-  dim3 grid(n_tokens), block(256);
+  if (nh + 2 * nkv > 65535) return ATOMA_ERR_SHAPE;
+  // without caches only q (and, for a caller that rotates k in place of q, all nh heads) is touched
+  dim3 grid(n_tokens, kcache ? nh + 2 * nkv : nh), block(64);
 #define ATOMA_ROPE(TA, TC)                                                                                        \
   hipLaunchKernelGGL((rope_cache_write_kernel<TA, TC>), grid, block, 0, stream, (TA*)qkv, row_stride, positions, \
                      cos_t, sin_t, rotary_dim, (TC*)kcache, (TC*)vcache, slot_mapping, page_size, nh, nkv, hd)
@@ -196,9 +284,41 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
   }
 }
 
+// four values per thread; needs inter % 4 == 0 and 16-byte aligned rows
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int n_tokens) {
+  const int quads = inter >> 2;
+  const size_t total = (size_t)n_tokens * quads;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
+    const size_t t = idx / quads;
+    const int i = (int)(idx % quads) * 4;
+    const f4 g = load4(gu + t * 2 * inter + i), u = load4(gu + t * 2 * inter + inter + i);
+    f4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o.v[e] = g.v[e] / (1.0f + expf(-g.v[e])) * u.v[e];
+    store4(out + t * inter + i, o);
+  }
+}
+
 extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   const size_t total = (size_t)n_tokens * inter;
+  if (inter % 4 == 0 && ((uintptr_t)gu & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    size_t quads = total / 4;
+    int vb = (int)((quads + 255) / 256);
+    if (vb > 16384) vb = 16384;
+    if (dtype == kF32)
+      hipLaunchKernelGGL(swiglu_vec_kernel<float>, dim3(vb), dim3(256), 0, stream, (const float*)gu, (float*)out, inter,
+                         n_tokens);
+    else if (dtype == kBF16)
+      hipLaunchKernelGGL(swiglu_vec_kernel<bf16_t>, dim3(vb), dim3(256), 0, stream, (const bf16_t*)gu, (bf16_t*)out,
+                         inter, n_tokens);
+    else
+      return ATOMA_ERR_DTYPE;
+    ATOMA_LAUNCH_CHECK();
+    return 0;
+  }
   int blocks = (int)((total + 255) / 256);
   if (blocks > 65536) blocks = 65536;
   if (dtype == kF32)

@@ -5,8 +5,8 @@
 // MT tiles of 16 rows of A with v_mfma_f32_16x16x32_bf16: the W tile is the MFMA's A operand (lane l: row l%16,
 // eight consecutive k at (l/16)*8), the activations its B operand (lane l: row of A l%16, the same eight k), so
 // both are 16-byte loads straight from global memory and nothing passes through LDS on the way in.
-// The four waves of a workgroup either take different rows of W (WK = 1) or split K four ways for the same rows
-// and add their accumulators in LDS (WK = 4), which keeps enough workgroups in flight when N is small.
+// The waves of a workgroup either take different rows of W (WK = 1, four waves) or split K four or eight ways for
+// the same rows and add their accumulators in LDS (WK = 4, 8), which keeps enough loads in flight when N is small.
 // K can additionally be split across blockIdx.y; then each slice writes its own float32 plane
 // C[slice][M][N] and the consumer adds the planes (the fused residual-add + RMSNorm kernel does).
 // Each output's sum order depends only on (K, WK, slices), never on M or on the row's place in the batch.
@@ -19,11 +19,13 @@ using namespace atoma;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-template <int MT, int RT, int WK, typename TC>
-__global__ void __launch_bounds__(256)
+template <int MT, int RT, int WN, int WK, typename TC>
+__global__ void __launch_bounds__(64 * WN * WK)
 gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
                    int K, int lda, int ldw, int ldc, size_t plane) {
-  constexpr int WN = 4 / WK;  // waves along N
+  // loads of U steps of K are issued together before their MFMAs, so that a wave keeps U * (RT + MT) 16-byte
+  // loads per lane in flight: the product is bound by memory latency and bandwidth, not by arithmetic
+  constexpr int U = (RT + MT <= 2) ? 4 : (RT + MT <= 5) ? 2 : 1;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wn = wave % WN, wk = wave / WN;
   const int r16 = lane & 15, kg = lane >> 4;
@@ -54,22 +56,56 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[r][m] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-#pragma unroll 4
-  for (int k = 0; k < k_len; k += 32) {
-    bf16x8 wf[RT], af[MT];
+  // two buffers of U steps each: while the MFMAs of one run, the loads of the other are in flight
+  bf16x8 wf[2][U][RT], af[2][U][MT];
+  auto load = [&](int buf, int k0) {
 #pragma unroll
-    for (int r = 0; r < RT; ++r) wf[r] = *reinterpret_cast<const bf16x8*>(wp[r] + k);
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
-    for (int m = 0; m < MT; ++m) af[m] = *reinterpret_cast<const bf16x8*>(ap[m] + k);
+      for (int r = 0; r < RT; ++r) wf[buf][u][r] = *reinterpret_cast<const bf16x8*>(wp[r] + k0 + u * 32);
+#pragma unroll
+      for (int m = 0; m < MT; ++m) af[buf][u][m] = *reinterpret_cast<const bf16x8*>(ap[m] + k0 + u * 32);
+    }
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+          acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[buf][u][r], af[buf][u][m], acc[r][m], 0, 0, 0);
+  };
+  constexpr int STEP = 32 * U;
+  const int n_batches = k_len / STEP;
+  int k = 0;
+  if (n_batches > 0) {
+    load(0, 0);
+    int b = 0;
+    for (; b + 2 <= n_batches; b += 2) {
+      load(1, (b + 1) * STEP);
+      multiply(0);
+      if (b + 2 < n_batches) load(0, (b + 2) * STEP);
+      multiply(1);
+    }
+    if (b < n_batches) multiply(0);
+    k = n_batches * STEP;
+  }
+  for (; k < k_len; k += 32) {
+    bf16x8 wt[RT], at[MT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) wt[r] = *reinterpret_cast<const bf16x8*>(wp[r] + k);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) at[m] = *reinterpret_cast<const bf16x8*>(ap[m] + k);
 #pragma unroll
     for (int r = 0; r < RT; ++r)
 #pragma unroll
       for (int m = 0; m < MT; ++m)
-        acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[r], af[m], acc[r][m], 0, 0, 0);
+        acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt[r], at[m], acc[r][m], 0, 0, 0);
   }
 
   if constexpr (WK > 1) {
-    // add the WK partial accumulators of the same rows: wave wk > 0 writes, wave wk == 0 sums in fixed order
+    // add the WK partial accumulators of the same rows: waves wk > 0 write, wave wk == 0 sums in fixed order
     __shared__ float red[(WK - 1) * WN * RT * MT * 4 * 64];
     constexpr int per_wave = RT * MT * 4 * 64;
     if (wk > 0) {
@@ -123,17 +159,16 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   }
 }
 
-template <int MT, int RT, int WK>
+template <int MT, int RT, int WN, int WK>
 static int launch(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc,
                   int slices, hipStream_t stream) {
-  constexpr int WN = 4 / WK;
-  dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), slices), block(256);
+  dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), slices), block(64 * WN * WK);
   const size_t plane = (size_t)M * ldc;
   if (c_dtype == kF32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WK, float>), grid, block, 0, stream, (const uint16_t*)a,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, float>), grid, block, 0, stream, (const uint16_t*)a,
                        (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane);
   else if (c_dtype == kBF16)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WK, bf16_t>), grid, block, 0, stream, (const uint16_t*)a,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t>), grid, block, 0, stream, (const uint16_t*)a,
                        (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane);
   else
     return ATOMA_ERR_DTYPE;
@@ -144,19 +179,22 @@ static int launch(const void* a, const void* w, void* c, int c_dtype, int M, int
 template <int MT>
 static int launch_mt(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, int lda, int ldw,
                      int ldc, int rt, int wk, int slices, hipStream_t stream) {
-#define ATOMA_CASE(R, W_)                                                                                   \
-  if (rt == R && wk == W_) return launch<MT, R, W_>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, slices, stream)
-  ATOMA_CASE(1, 1);
-  ATOMA_CASE(2, 1);
-  ATOMA_CASE(4, 1);
-  ATOMA_CASE(1, 4);
-  ATOMA_CASE(2, 4);
+#define ATOMA_CASE(R, WN_, WK_)                                                                                   \
+  if (rt == R && wk == WK_) return launch<MT, R, WN_, WK_>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, slices, stream)
+  ATOMA_CASE(1, 4, 1);
+  ATOMA_CASE(2, 4, 1);
+  ATOMA_CASE(4, 4, 1);
+  ATOMA_CASE(1, 1, 4);
+  ATOMA_CASE(2, 1, 4);
+  ATOMA_CASE(1, 1, 8);
+  ATOMA_CASE(2, 1, 8);
 #undef ATOMA_CASE
   return ATOMA_ERR_SHAPE;
 }
 
 // a [M <= 64, K] bf16, w [N, K] bf16 -> c [slices][M, N] (bf16 only with slices == 1, or float32).
-// rt: tiles of 16 rows of W per wave (1, 2, 4); wk: 1 or 4 (waves split K); slices: K split across the grid.
+// rt: tiles of 16 rows of W per wave (1, 2, 4); wk: 1 (four waves on different rows), 4 or 8 (that many waves
+// split K for the same rows); slices: K split across the grid.
 extern "C" int atoma_gemm_bf16_skinny(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
                                       int lda, int ldw, int ldc, int rt, int wk, int slices, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;

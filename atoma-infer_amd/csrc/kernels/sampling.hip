@@ -79,7 +79,21 @@ sample_kernel(const float* __restrict__ logits, int ld, int vocab, const float* 
   float* w = weights + (size_t)row * vocab;
 
   ArgMax a = {-INFINITY, 0x7fffffff};
-  for (int i = tid; i < vocab; i += kSampThreads) a = better(a, ArgMax{lr[i], i});
+  if ((vocab & 3) == 0 && (((uintptr_t)lr) & 15) == 0) {
+    // four values per load, several loads in flight
+    const float4* l4 = reinterpret_cast<const float4*>(lr);
+    const int n4 = vocab >> 2;
+#pragma unroll 4
+    for (int i = tid; i < n4; i += kSampThreads) {
+      const float4 v = l4[i];
+      a = better(a, ArgMax{v.x, 4 * i});
+      a = better(a, ArgMax{v.y, 4 * i + 1});
+      a = better(a, ArgMax{v.z, 4 * i + 2});
+      a = better(a, ArgMax{v.w, 4 * i + 3});
+    }
+  } else {
+    for (int i = tid; i < vocab; i += kSampThreads) a = better(a, ArgMax{lr[i], i});
+  }
   a = block_argmax(a, am);
   const float temp = temperature[row];
   if (!(temp > 0.f)) {

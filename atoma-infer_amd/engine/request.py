@@ -38,7 +38,7 @@ class RequestMetrics:
     num_preemptions: int = 0
 
 
-@dataclasses.dataclass
+@dataclasses.dataclass(eq=False)
 class Request:
     uid: int                      # engine-wide unique number, the cache manager's key
     request_id: str               # the caller's name

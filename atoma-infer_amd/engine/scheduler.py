@@ -147,8 +147,20 @@ class Scheduler:
 
         # 1 and 2: running requests, decodes before portions of prompts
         order = [r for r in self.running if not r.in_prefill] + [r for r in self.running if r.in_prefill]
+        if len(order) <= cfg.max_num_sequences and len(order) <= cfg.max_num_batched_tokens and \
+                all(r.num_uncomputed == 1 for r in order):
+            # the common step: everything running decodes one token and fits both budgets; pages are taken
+            # request by request, and the general path below takes over at the first that finds none
+            done = 0
+            for r in order:
+                if not self.cache.can_reserve(r.uid, r.num_computed + 1):
+                    break
+                self.cache.reserve(r.uid, r.num_computed + 1)
+                out.entries.append(ScheduledEntry(r, 1, r.num_computed, True))
+                done += 1
+            order = order[done:]
         for r in order:
-            if r not in self.running:
+            if r.status is not Status.RUNNING:
                 continue  # preempted while serving an earlier request
             if len(out.entries) >= cfg.max_num_sequences:
                 break
@@ -167,7 +179,7 @@ class Scheduler:
                 self._preempt(victim, out)
                 if victim is r:
                     break
-            if r not in self.running:
+            if r.status is not Status.RUNNING:
                 continue
             self.cache.reserve(r.uid, r.num_computed + n)
             out.entries.append(ScheduledEntry(r, n, r.num_computed, r.num_computed + n == r.length))

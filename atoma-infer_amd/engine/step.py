@@ -227,7 +227,11 @@ class ModelRunner:
         max_seq = int((starts + counts).max())
         page = self.pool.page_size
         max_blocks = -(-max_seq // page) if bucket is None else -(-bucket * DECODE_BUCKET // page)
-        extras = [(key, *fn(starts, counts, bucket)) for key, fn in self._planners.items()]
+        # a step that only decodes is planned the same way whether it is captured or run eagerly
+        plan_bucket = bucket
+        if plan_bucket is None and int(counts.max()) == 1:
+            plan_bucket = -(-max_seq // DECODE_BUCKET)
+        extras = [(key, *fn(starts, counts, plan_bucket)) for key, fn in self._planners.items()]
         # layout of the one staging buffer
         o_tok, o_pos, o_seq = 0, t, 2 * t
         o_qs, o_len, o_slot = 3 * t, 3 * t + s + 1, 3 * t + 2 * s + 1

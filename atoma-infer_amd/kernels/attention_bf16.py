@@ -21,7 +21,8 @@ from .library import load_hip_module
 from .ops import _check, _p, _stream
 
 PAGE = 16
-CHUNK = 256          # keys per partial task
+CHUNK = 256          # keys per partial task, at most; fewer when few requests are split (see chunk_for)
+MAX_SPLIT_TASKS = 1024
 SPLIT_MAX_TOKENS = 16  # entries with at most this many tokens may be split along the keys
 SPLIT_MIN_KEYS = 2 * CHUNK
 _libs: Dict[int, ctypes.CDLL] = {}
@@ -39,43 +40,71 @@ def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
     return _libs[hd]
 
 
+def chunk_for(n_split: int, max_keys: int) -> int:
+    """Keys per partial task: 64, 128 or 256, the smallest that keeps the step's partial tasks under a bound.
+
+    A wave walks its keys one 32-key block after another, so short chunks shorten the chain when few requests
+    decode, and long ones save partial results when many do.  ``max_keys`` is rounded up to 256.
+    """
+    buckets = -(-max_keys // CHUNK)
+    for chunk in (64, 128):
+        if n_split * buckets * (CHUNK // chunk) <= MAX_SPLIT_TASKS:
+            return chunk
+    return CHUNK
+
+
 def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket: Optional[int] = None,
-                ) -> Tuple[np.ndarray, Tuple[int, int, int]]:
-    """Task records [n, 8] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials).
+                vectorized: bool = True) -> Tuple[np.ndarray, Tuple[int, int, int]]:
+    """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials).
 
     Main tasks are padded to a multiple of 4 (one workgroup runs 4) and ordered so that tasks sharing keys are
     neighbours and long tasks come first.  With ``bucket`` (decode graphs: one token per entry) every entry is
     split and owns ``bucket`` chunk slots, used or not, so all counts depend on (entries, bucket) alone.
     """
+    if vectorized and bucket is not None and len(counts) and int(counts.max()) == 1:
+        return _build_decode_tasks(starts, group, window, bucket)
     qt_max = max(1, 128 // group)
-    null = (-1, 0, 1, 0, 0, 0, -1, 0)
+    null = (-1, 0, 1, 0, 0, 0, -1, 0, 0, 0, 0, 0)
+    tok_bases = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
     direct, split, combine = [], [], []
     n_part = 0
+
+    def splits(e):
+        first_key = max(0, int(starts[e]) - window + 1) if window > 0 else 0
+        return bucket is not None or (int(counts[e]) <= SPLIT_MAX_TOKENS
+                                      and int(starts[e]) + int(counts[e]) - first_key >= SPLIT_MIN_KEYS)
+
+    split_entries = [e for e in range(len(starts)) if splits(e)]
+    chunk = CHUNK
+    if split_entries:
+        chunk = chunk_for(len(split_entries), max(int(starts[e]) + int(counts[e]) for e in split_entries))
     for e in range(len(starts)):
         start, count = int(starts[e]), int(counts[e])
-        k_end_all = start + count
         qt = min(qt_max, count)
         rows = qt * group
-        first_key = max(0, start - window + 1) if window > 0 else 0
-        do_split = bucket is not None or (count <= SPLIT_MAX_TOKENS and (k_end_all - first_key) >= SPLIT_MIN_KEYS)
+        do_split = splits(e)
+        tail = (int(tok_bases[e]), count, start, 0)
         for tok0 in range(0, count, qt):
             last = min(tok0 + qt, count)
             k_end = start + last
             lo = max(0, start + tok0 - window + 1) if window > 0 else 0
+            # 32-row pieces of the tile that hold at least one live row (the last tile of an entry may be short)
+            live = [row0 for row0 in range(0, rows, 32)
+                    if any(tok0 + r % qt < count for r in range(row0, min(row0 + 32, rows)))]
             if do_split:
-                c_first, c_last = lo // CHUNK, (k_end - 1) // CHUNK
-                slots = bucket if bucket is not None else c_last + 1
-                for row0 in range(0, rows, 32):
-                    combine.append((e, tok0, qt, row0, 0, 0, n_part + c_first, c_last - c_first + 1))
+                c_first, c_last = lo // chunk, (k_end - 1) // chunk
+                slots = bucket * (CHUNK // chunk) if bucket is not None else c_last + 1
+                for row0 in live:
+                    combine.append((e, tok0, qt, row0, 0, 0, n_part + c_first, c_last - c_first + 1) + tail)
                     for c in range(slots):
                         if c_first <= c <= c_last:
-                            split.append((e, tok0, qt, row0, c * CHUNK, min((c + 1) * CHUNK, k_end), n_part + c, 0))
+                            split.append((e, tok0, qt, row0, c * chunk, min((c + 1) * chunk, k_end), n_part + c, 0) + tail)
                         elif bucket is not None:
                             split.append(null)
                     n_part += slots
             else:
                 kb = (lo // 32) * 32
-                wave_tasks = [(e, tok0, qt, row0, kb, k_end, -1, 0) for row0 in range(0, rows, 32)]
+                wave_tasks = [(e, tok0, qt, row0, kb, k_end, -1, 0) + tail for row0 in live]
                 while len(wave_tasks) % 4:
                     wave_tasks.append(null)
                 direct.append((k_end - kb, wave_tasks))
@@ -83,8 +112,53 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     main = [t for _, ws in direct for t in ws] + split
     while len(main) % 4:
         main.append(null)
-    arr = np.asarray(main + combine, dtype=np.int32).reshape(-1, 8)
+    arr = np.asarray(main + combine, dtype=np.int32).reshape(-1, 12)
     return arr, (len(main), len(combine), n_part)
+
+
+def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int):
+    """``build_tasks`` for a step in which every entry brings one token, without a Python loop over entries."""
+    s = len(starts)
+    starts = starts.astype(np.int64)
+    k_end = starts + 1
+    lo = np.maximum(0, starts - window + 1) if window > 0 else np.zeros(s, dtype=np.int64)
+    chunk = chunk_for(s, int(k_end.max()))
+    slots = bucket * (CHUNK // chunk)
+    row_chunks = -(-group // 32)
+    c = np.arange(slots, dtype=np.int64)
+    c_first, c_last = lo // chunk, (k_end - 1) // chunk
+    valid = (c[None, :] >= c_first[:, None]) & (c[None, :] <= c_last[:, None])          # [s, slots]
+    main = np.zeros((s, row_chunks, slots, 12), dtype=np.int32)
+    e = np.arange(s, dtype=np.int64)
+    rc = np.arange(row_chunks, dtype=np.int64)
+    v = np.broadcast_to(valid[:, None, :], (s, row_chunks, slots))
+    main[..., 0] = np.where(v, e[:, None, None], -1)
+    main[..., 2] = 1
+    main[..., 3] = np.where(v, 32 * rc[None, :, None], 0)
+    main[..., 4] = np.where(v, (c * chunk)[None, None, :], 0)
+    main[..., 5] = np.where(v, np.minimum((c + 1) * chunk, k_end[:, None])[:, None, :], 0)
+    part = (e[:, None, None] * row_chunks + rc[None, :, None]) * slots + c[None, None, :]
+    main[..., 6] = np.where(v, part, -1)
+    main[..., 8] = np.where(v, e[:, None, None], 0)
+    main[..., 9] = np.where(v, 1, 0)
+    main[..., 10] = np.where(v, starts[:, None, None], 0)
+    main = main.reshape(-1, 12)
+    pad = (-len(main)) % 4
+    if pad:
+        filler = np.zeros((pad, 12), dtype=np.int32)
+        filler[:, 0], filler[:, 2], filler[:, 6] = -1, 1, -1
+        main = np.concatenate([main, filler])
+    comb = np.zeros((s, row_chunks, 12), dtype=np.int32)
+    comb[..., 0] = e[:, None]
+    comb[..., 2] = 1
+    comb[..., 3] = 32 * rc[None, :]
+    comb[..., 6] = (e[:, None] * row_chunks + rc[None, :]) * slots + c_first[:, None]
+    comb[..., 7] = (c_last - c_first + 1)[:, None]
+    comb[..., 8] = e[:, None]
+    comb[..., 9] = 1
+    comb[..., 10] = starts[:, None]
+    arr = np.concatenate([main, comb.reshape(-1, 12)])
+    return arr, (len(main), s * row_chunks, s * row_chunks * slots)
 
 
 def plan_key(group: int, window: int):
@@ -120,6 +194,5 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
     bt = cache.block_tables
     _check(lib(hd).atoma_attention_mfma(_p(q), q.stride(0), _p(k_cache), _p(v_cache), _p(out), out.stride(0),
                                         _p(part_o), _p(part_lse), _p(tasks), n_main, n_comb, _p(bt), bt.shape[1],
-                                        _p(ctx.q_start), _p(ctx.positions), ctypes.c_float(scale), int(window), nh,
-                                        nkv, _stream()), "attention_mfma")
+                                        ctypes.c_float(scale), int(window), nh, nkv, _stream()), "attention_mfma")
     return True

@@ -33,25 +33,31 @@ def _aligned(t: torch.Tensor) -> bool:
     return t.data_ptr() % 16 == 0 and (t.shape[0] == 1 or t.stride(0) % 8 == 0) and t.stride(1) == 1
 
 
-def _plan(n: int, k: int, allow_slices: bool):
-    """(rows-of-16 per wave, waves splitting K, K slices over the grid) for a product with N outputs."""
+def _plan(m: int, n: int, k: int, allow_slices: bool):
+    """(rows-of-16 per wave, waves splitting K, K slices over the grid) for x [m, k] @ w [n, k]^T.
+
+    Chosen from measurements on MI355X at the sizes of Llama-3.2-1B: few rows of x want many waves that split K
+    (every wave's loads are in flight at once); many rows want waves that own several row tiles of W, so that
+    each fragment of x feeds several MFMAs.
+    """
     tiles = -(-n // 16)
+    small_m = m <= 16
     if tiles >= 4096:
-        rt, wk = 4, 1
-    elif tiles >= 2048:
-        rt, wk = 2, 1
+        rt, wk = (2, 8) if small_m else (4, 1)
     elif tiles >= 512:
         rt, wk = 2, 4
     else:
-        rt, wk = 1, 4
-    if k % (32 * wk):
+        rt, wk = (1, 4) if small_m or not allow_slices else (2, 4)
+    while wk > 1 and k % (32 * wk):
+        wk //= 2
+    if wk == 2:
         wk = 1
     slices = 1
     if allow_slices:
-        groups = -(-tiles // ((4 // wk) * rt))
-        slices = max(1, min(8, 256 // max(groups, 1)))
-        while slices > 1 and (k % (32 * wk * slices) or k // (wk * slices) < 256):
-            slices -= 1
+        groups = -(-tiles // ((4 if wk == 1 else 1) * rt))
+        slices = 8
+        while slices > 1 and (k % (32 * wk * slices) or k // (wk * slices) < 128 or groups * slices > 1024):
+            slices //= 2
     return rt, wk, slices
 
 
@@ -65,7 +71,7 @@ def skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, slices: int = 1,
     m, k = x.shape
     n = w.shape[0]
     if not rt:
-        rt, wk, _ = _plan(n, k, False)
+        rt, wk, _ = _plan(m, n, k, False)
         if k % (32 * wk * slices):
             wk = 1
     ldc = out.stride(-2) if m > 1 else n
@@ -100,7 +106,7 @@ def linear_planes(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
     n = w.shape[0]
     if m > SKINNY_MAX_M or not skinny_ok(x, w):
         return None
-    rt, wk, slices = _plan(n, k, True)
+    rt, wk, slices = _plan(m, n, k, True)
     out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
     skinny(x, w, out, slices, rt, wk)
     return out

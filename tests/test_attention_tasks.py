@@ -1,0 +1,82 @@
+"""The host-side task lists of the MFMA attention kernels: every (row, key) a request may see is covered exactly
+once, partial results are merged from the right slots, and the vectorised decode builder equals the general one."""
+import numpy as np
+import pytest
+
+from atoma_infer_amd.kernels import attention_bf16 as A
+
+
+def coverage(arr, meta, starts, counts, group, window):
+    n_main, n_comb, n_part = meta
+    main, comb = arr[:n_main], arr[n_main:]
+    assert len(comb) == n_comb and n_main % 4 == 0
+    seen = {}          # (entry, token, head) -> list of key ranges, direct
+    parts = {}         # partial index -> (entry, token/head rows, key range)
+    for t in main:
+        e, tok0, qt, row0, kb, ke, dest, _, tok_base, count, pos0, _ = (int(x) for x in t)
+        if e < 0:
+            continue
+        assert tok_base == int(np.sum(counts[:e])) and count == counts[e] and pos0 == starts[e]
+        assert kb % 32 == 0 and kb < ke
+        rows = [(tok0 + r % qt, r // qt) for r in range(row0, row0 + 32) if r // qt < group and tok0 + r % qt < count]
+        assert rows
+        if dest < 0:
+            for row in rows:
+                seen.setdefault((e,) + row, []).append((kb, ke))
+        else:
+            assert 0 <= dest < n_part and dest not in parts
+            parts[dest] = (e, rows, (kb, ke))
+    for t in comb:
+        e, tok0, qt, row0, _, _, dest, n_parts, *_ = (int(x) for x in t)
+        rows = [(tok0 + r % qt, r // qt) for r in range(row0, row0 + 32) if r // qt < group and tok0 + r % qt < counts[e]]
+        for p in range(dest, dest + n_parts):
+            pe, prows, rng = parts.pop(p)
+            assert pe == e and prows == rows
+            for row in rows:
+                seen.setdefault((e,) + row, []).append(rng)
+    assert not parts, "a partial result that nobody merges"
+    for e in range(len(starts)):
+        for tok in range(counts[e]):
+            p = starts[e] + tok
+            lo = max(0, p - window + 1) if window else 0
+            for h in range(group):
+                ranges = sorted(seen[(e, tok, h)])
+                # ranges tile a span that holds every visible key, without overlap
+                assert ranges[0][0] <= lo and ranges[-1][1] >= p + 1
+                for (a, b), (c, d) in zip(ranges, ranges[1:]):
+                    assert b == c
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_tasks_cover_every_visible_key_once(seed):
+    rng = np.random.default_rng(seed)
+    s = int(rng.integers(1, 9))
+    group = int(rng.choice([1, 3, 4, 8, 40]))
+    window = int(rng.choice([0, 0, 50, 700]))
+    counts = rng.choice([1, 1, 2, 7, 33, 150], size=s).astype(np.int32)
+    starts = rng.integers(0, 2500, size=s).astype(np.int32)
+    arr, meta = A.build_tasks(starts, counts, group, window)
+    coverage(arr, meta, starts, counts, group, window)
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_decode_builder_equals_the_general_one(seed):
+    rng = np.random.default_rng(100 + seed)
+    s = int(rng.integers(1, 80))
+    group = int(rng.choice([1, 3, 4, 8, 40]))
+    window = int(rng.choice([0, 0, 100, 700]))
+    starts = rng.integers(0, 3000, size=s).astype(np.int32)
+    counts = np.ones(s, dtype=np.int32)
+    bucket = -(-int(starts.max() + 1) // 256)
+    fast, mf = A.build_tasks(starts, counts, group, window, bucket)
+    slow, ms = A.build_tasks(starts, counts, group, window, bucket, vectorized=False)
+    assert mf == ms
+    # null tasks may differ in their unused fields; compare what the kernels read
+    live = fast[:, 0] >= 0
+    assert np.array_equal(live, slow[:, 0] >= 0)
+    assert np.array_equal(fast[live], slow[live])
+    coverage(fast, mf, starts, counts, group, window)
+    # sizes depend on (entries, bucket) alone
+    other = rng.integers(0, bucket * 256, size=s).astype(np.int32)
+    assert A.build_tasks(other, counts, group, window, bucket)[1] == mf or \
+        A.chunk_for(s, int(other.max()) + 1) != A.chunk_for(s, int(starts.max()) + 1)
