@@ -143,13 +143,21 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       }
     }
   };
+  // Two blocks are always in flight: (kf, vf) hold the block being worked on, (kn, vn) the next one, and the
+  // loads of the one after that are issued as soon as (kn, vn) have moved up.
+  constexpr bool DEEP = false;      // measured on MI355X: the second buffer costs occupancy and gains nothing
   int pg0 = 0, pg1 = 0;
-  bf16x8 kf[KSTEPS];
+  bf16x8 kf[KSTEPS], kn[DEEP ? KSTEPS : 1];
   bf16x8 vf[2][DTILES], vn[2][DTILES];
   if (task.k_begin < task.k_end) {
     pages_of(task.k_begin, pg0, pg1);
     load_keys(pg0, pg1, kf);
     load_vals(pg0, pg1, vf);
+    if (DEEP && task.k_begin + 32 < task.k_end) {
+      pages_of(task.k_begin + 32, pg0, pg1);
+      load_keys(pg0, pg1, kn);
+      load_vals(pg0, pg1, vn);
+    }
   }
 
   for (int kb = task.k_begin; kb < task.k_end; kb += 32) {
@@ -160,11 +168,34 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[st], s, 0, 0, 0);
     const bool has_next = kb + 32 < task.k_end;
-    if (has_next) {
-      pages_of(kb + 32, pg0, pg1);
-      if (PREFETCH) {
-        load_keys(pg0, pg1, kf);
+    bf16x8 vc[2][DTILES];
+    if (DEEP) {
+      // this block's values move aside, the next block moves up, the block after it is requested
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) {
+          vc[j][dt] = vf[j][dt];
+          vf[j][dt] = vn[j][dt];
+        }
+#pragma unroll
+      for (int st = 0; st < KSTEPS; ++st) kf[st] = kn[st];
+      if (kb + 64 < task.k_end) {
+        pages_of(kb + 64, pg0, pg1);
+        load_keys(pg0, pg1, kn);
         load_vals(pg0, pg1, vn);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) vc[j][dt] = vf[j][dt];
+      if (has_next) {
+        pages_of(kb + 32, pg0, pg1);
+        if (PREFETCH) {
+          load_keys(pg0, pg1, kf);
+          load_vals(pg0, pg1, vf);
+        }
       }
     }
 
@@ -198,19 +229,12 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     for (int dt = 0; dt < DTILES; ++dt) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[0][dt], p0, o[dt], 0, 0, 0);
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[1][dt], p1, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[0][dt], p0, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[1][dt], p1, o[dt], 0, 0, 0);
     }
-    if (has_next) {
-      if (PREFETCH) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int dt = 0; dt < DTILES; ++dt) vf[j][dt] = vn[j][dt];
-      } else {
-        load_keys(pg0, pg1, kf);
-        load_vals(pg0, pg1, vf);
-      }
+    if (!DEEP && !PREFETCH && has_next) {
+      load_keys(pg0, pg1, kf);
+      load_vals(pg0, pg1, vf);
     }
   }
 
@@ -251,34 +275,89 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
 }
 
 // Merge partial results: out = sum_s w_s O_s / sum_s w_s with w_s = exp2(lse_s - max lse).
-// One block per (combine task, KV head).  The valid rows of the task (group x tokens, at most 32) times HD
-// output values are spread over the 256 threads; the partial results of one value are added in order of their
-// index, with the loads of several parts in flight.
+// One block per (combine task, KV head).  The log-sum-exps of all parts are first brought into LDS by all
+// threads at once and turned into weights there; then the valid rows of the task (group x tokens, at most 32)
+// times HD output values are spread over the 256 threads, and each adds its parts in order of their index with
+// eight loads in flight.
+constexpr int kCombineParts = 128;   // parts whose weights fit in LDS at once; more are merged in rounds
+
 __global__ void __launch_bounds__(256)
 attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
                          uint16_t* __restrict__ out, int out_stride, const Task* __restrict__ tasks, int nh,
                          int nkv) {
+  __shared__ float wts[kCombineParts][32];
+  __shared__ float row_max[32];
   const Task task = tasks[blockIdx.x];
   if (task.entry < 0) return;
   const int kvh = blockIdx.y, g = nh / nkv;
   const int tok_base = task.tok_base, count = task.count;
   const size_t part_stride = (size_t)nkv * 32;   // rows between two partial results of the same (KV head, row)
-  for (int idx = threadIdx.x; idx < 32 * HD; idx += 256) {
+  const size_t base0 = ((size_t)task.dest * nkv + kvh) * 32;
+  const int tid = threadIdx.x;
+
+  // the largest log-sum-exp of every row, over all parts
+  {
+    const int c = tid & 31, lane_part = tid >> 5;   // 8 parts at a time per row
+    float mx = -INFINITY;
+    for (int s = lane_part; s < task.n_parts; s += 8) mx = fmaxf(mx, part_lse[base0 + s * part_stride + c]);
+    wts[lane_part][c] = mx;
+    __syncthreads();
+    if (tid < 32) {
+      float m2 = wts[0][tid];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) m2 = fmaxf(m2, wts[i][tid]);
+      row_max[tid] = m2;
+    }
+    __syncthreads();
+  }
+
+  float acc[(32 * HD + 255) / 256];
+  float wsum[(32 * HD + 255) / 256];
+#pragma unroll
+  for (int i = 0; i < (32 * HD + 255) / 256; ++i) acc[i] = wsum[i] = 0.f;
+
+  for (int p0 = 0; p0 < task.n_parts; p0 += kCombineParts) {
+    const int np = task.n_parts - p0 < kCombineParts ? task.n_parts - p0 : kCombineParts;
+    __syncthreads();
+    for (int i = tid; i < np * 32; i += 256) {
+      const int s = i >> 5, c = i & 31;
+      wts[s][c] = __builtin_amdgcn_exp2f(part_lse[base0 + (size_t)(p0 + s) * part_stride + c] - row_max[c]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < (32 * HD + 255) / 256; ++it) {
+      const int idx = tid + it * 256;
+      const int c = idx / HD, d = idx % HD;
+      const int r = task.row0 + c;
+      const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
+      if (idx >= 32 * HD || hq >= g || tok >= count) continue;
+      const float* po = part_o + (base0 + (size_t)p0 * part_stride + c) * HD + d;
+      int s = 0;
+      for (; s + 8 <= np; s += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = po[(size_t)(s + u) * part_stride * HD];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          acc[it] += wts[s + u][c] * v[u];
+          wsum[it] += wts[s + u][c];
+        }
+      }
+      for (; s < np; ++s) {
+        acc[it] += wts[s][c] * po[(size_t)s * part_stride * HD];
+        wsum[it] += wts[s][c];
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < (32 * HD + 255) / 256; ++it) {
+    const int idx = tid + it * 256;
     const int c = idx / HD, d = idx % HD;
     const int r = task.row0 + c;
     const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
-    if (hq >= g || tok >= count) continue;
-    const size_t base = ((size_t)task.dest * nkv + kvh) * 32 + c;
-    float mx = -INFINITY;
-    for (int s = 0; s < task.n_parts; ++s) mx = fmaxf(mx, part_lse[base + s * part_stride]);
-    float acc = 0.f, wsum = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < task.n_parts; ++s) {
-      const float w = __builtin_amdgcn_exp2f(part_lse[base + s * part_stride] - mx);  // lse = -inf: weight 0
-      wsum += w;
-      acc += w * part_o[(base + s * part_stride) * HD + d];
-    }
-    out[(size_t)(tok_base + tok) * out_stride + (size_t)(kvh * g + hq) * HD + d] = f32_to_bf16_bits(acc / wsum);
+    if (idx >= 32 * HD || hq >= g || tok >= count) continue;
+    out[(size_t)(tok_base + tok) * out_stride + (size_t)(kvh * g + hq) * HD + d] =
+        f32_to_bf16_bits(acc[it] / wsum[it]);
   }
 }
 
