@@ -205,47 +205,50 @@ extern "C" int atoma_add_rmsnorm(float* resid, const void* delta, int delta_dtyp
 // csrc/kernels/cache_manager.cu:151-155).  cos/sin may be null: then nothing is rotated.
 // Pairing and signs: csrc/kernels/rotary.h:116-131; rotation applies to q and k only: models/src/llama.rs:298-299.
 template <typename TA, typename TC>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __restrict__ positions,
                         const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim,
                         TC* __restrict__ kcache, TC* __restrict__ vcache, const int32_t* __restrict__ slot_mapping,
-                        int page_size, int nh, int nkv, int hd) {
-  // one block of 64 threads per (token, head): q heads, then k heads, then v heads
-  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+                        int page_size, int nh, int nkv, int hd, int heads) {
+  // One thread per item of a token: a rotated pair (or, beyond the rotary dimension, a pair of plain columns)
+  // of a q or k head, or two columns of a v head.  `heads` is how many heads of the row are touched.
+  const int t = blockIdx.x;
+  const int hp = hd >> 1;                       // items per head
+  const int item = blockIdx.y * 256 + threadIdx.x;
+  if (item >= heads * hp) return;
+  const int head = item / hp, i = item % hp;
   TA* x = qkv + (size_t)t * row_stride + (size_t)head * hd;
   const int slot = (kcache && slot_mapping) ? slot_mapping[t] : -1;
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
   if (head >= nh + nkv) {
     // v: stored transposed inside the page
     if (slot < 0) return;
-    const int kvh = head - nh - nkv;
-    TC* dst = vcache + ((size_t)page * nkv + kvh) * hd * page_size + off;
-    for (int i = lane; i < hd; i += 64) dst[(size_t)i * page_size] = from_f32<TC>(to_f32(x[i]));
+    TC* dst = vcache + ((size_t)page * nkv + (head - nh - nkv)) * hd * page_size + off;
+    dst[(size_t)(2 * i) * page_size] = from_f32<TC>(to_f32(x[2 * i]));
+    dst[(size_t)(2 * i + 1) * page_size] = from_f32<TC>(to_f32(x[2 * i + 1]));
     return;
   }
   const bool is_k = head >= nh;
   if (is_k && slot < 0) return;
   TC* kdst = is_k ? kcache + (((size_t)page * nkv + (head - nh)) * page_size + off) * hd : nullptr;
   const int half = cos_t ? rotary_dim / 2 : 0;
-  if (half) {
-    const float* cs = cos_t + (size_t)positions[t] * half;
-    const float* sn = sin_t + (size_t)positions[t] * half;
-    for (int i = lane; i < half; i += 64) {
-      const float x1 = to_f32(x[i]), x2 = to_f32(x[i + half]);
-      const float c = cs[i], sv = sn[i];
-      const float o1 = x1 * c - x2 * sv, o2 = x2 * c + x1 * sv;
-      if (is_k) {
-        kdst[i] = from_f32<TC>(o1);
-        kdst[i + half] = from_f32<TC>(o2);
-      } else {
-        x[i] = from_f32<TA>(o1);
-        x[i + half] = from_f32<TA>(o2);
-      }
+  if (i < half) {
+    const float c = cos_t[(size_t)positions[t] * half + i], sv = sin_t[(size_t)positions[t] * half + i];
+    const float x1 = to_f32(x[i]), x2 = to_f32(x[i + half]);
+    const float o1 = x1 * c - x2 * sv, o2 = x2 * c + x1 * sv;
+    if (is_k) {
+      kdst[i] = from_f32<TC>(o1);
+      kdst[i + half] = from_f32<TC>(o2);
+    } else {
+      x[i] = from_f32<TA>(o1);
+      x[i + half] = from_f32<TA>(o2);
     }
+  } else if (is_k) {
+    // columns beyond the rotary dimension are copied as they are (all of them without tables)
+    const int a = 2 * half + 2 * (i - half);
+    kdst[a] = from_f32<TC>(to_f32(x[a]));
+    kdst[a + 1] = from_f32<TC>(to_f32(x[a + 1]));
   }
-  // the part of k that is not rotated (all of it without tables)
-  if (is_k)
-    for (int i = 2 * half + lane; i < hd; i += 64) kdst[i] = from_f32<TC>(to_f32(x[i]));
 }
 
 extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, const int32_t* positions,
@@ -257,10 +260,13 @@ extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, 
     return ATOMA_ERR_SHAPE;
   if (nh + 2 * nkv > 65535) return ATOMA_ERR_SHAPE;
   // without caches only q (and, for a caller that rotates k in place of q, all nh heads) is touched
-  dim3 grid(n_tokens, kcache ? nh + 2 * nkv : nh), block(64);
+  const int heads = kcache ? nh + 2 * nkv : nh;
+  const int items = heads * (hd / 2);
+  if (hd & 1) return ATOMA_ERR_SHAPE;
+  dim3 grid(n_tokens, (items + 255) / 256), block(256);
 #define ATOMA_ROPE(TA, TC)                                                                                        \
   hipLaunchKernelGGL((rope_cache_write_kernel<TA, TC>), grid, block, 0, stream, (TA*)qkv, row_stride, positions, \
-                     cos_t, sin_t, rotary_dim, (TC*)kcache, (TC*)vcache, slot_mapping, page_size, nh, nkv, hd)
+                     cos_t, sin_t, rotary_dim, (TC*)kcache, (TC*)vcache, slot_mapping, page_size, nh, nkv, hd, heads)
   if (act_dtype == kF32 && cache_dtype == kF32) ATOMA_ROPE(float, float);
   else if (act_dtype == kBF16 && cache_dtype == kBF16) ATOMA_ROPE(bf16_t, bf16_t);
   else if (act_dtype == kF32 && cache_dtype == kBF16) ATOMA_ROPE(float, bf16_t);
