@@ -3,9 +3,9 @@
 Every layer call that owns a cache entry is put into the group of its ``CacheSpec`` (KV heads, head size,
 window); a group has one pool of pages, and a page holds ``page_size`` tokens of every entry of its group, so
 one page number serves all those layers (the reference does the same for its single group:
-backends/vllm/src/worker.rs:570-598).  Keys of an entry are [pages, kv_heads, page_size, head] and values
-[pages, kv_heads, head, page_size]: a (page, head) tile is contiguous, keys along the head axis and values
-along the token axis, which is how the attention kernels read them.
+backends/vllm/src/worker.rs:570-598).  Keys and values of an entry are [pages, kv_heads, page_size * head]:
+a (page, head) tile is contiguous, and the order of its elements is the one in which the MFMA attention kernel's
+lanes read them (``cache/layout.py`` and csrc/kernels/cache_layout.h state it).
 
 Mixers that declare a ``StateSpec`` get a float32 tensor [slots, *shape] per layer call, indexed by the
 request's state slot.
@@ -96,10 +96,9 @@ class CachePool:
         for g, n in zip(plan.groups, num_pages):
             cs = g.spec
             # zero-filled, so that pages never written hold finite numbers
-            self.k.append(torch.zeros((len(g.calls), n, cs.kv_heads, page_size, cs.head_size), dtype=dtype,
-                                      device=device))
-            self.v.append(torch.zeros((len(g.calls), n, cs.kv_heads, cs.head_size, page_size), dtype=dtype,
-                                      device=device))
+            tile = page_size * cs.head_size
+            self.k.append(torch.zeros((len(g.calls), n, cs.kv_heads, tile), dtype=dtype, device=device))
+            self.v.append(torch.zeros((len(g.calls), n, cs.kv_heads, tile), dtype=dtype, device=device))
             geometry.append(GroupGeometry(page_size, n, cs.window))
         self.states = {pos: torch.zeros((num_state_slots, *shape), dtype=torch.float32, device=device)
                        for pos, shape in plan.states.items()}

@@ -10,6 +10,7 @@
 // Online softmax in float32 (csrc/kernels/softmax.h:128-186 of the reference); query head h reads KV head
 // h / (nh / nkv) (csrc/kernels/flash_fwd_kernel.h:593).
 #include "common.h"
+#include "cache_layout.h"
 
 using namespace atoma;
 
@@ -47,9 +48,14 @@ paged_attention_generic_kernel(const TQ* __restrict__ q, int q_stride, const TC*
     if (valid) {
       page = table[j / page_size];
       off = j % page_size;
-      const TC* kr = kcache + (((size_t)page * nkv + kvh) * page_size + off) * hd;
+      // the token's columns lie in runs of 8 inside the tile (cache_layout.h)
+      const TC* kt = kcache + ((size_t)page * nkv + kvh) * page_size * hd;
       float dot = 0.f;
-      for (int d = 0; d < hd; ++d) dot += qs[d] * to_f32(kr[d]);
+      for (int d0 = 0; d0 < hd; d0 += 8) {
+        const TC* kr = kt + key_offset(off, d0, page_size);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dot += qs[d0 + e] * to_f32(kr[e]);
+      }
       sc = dot * scale;
     }
     const float m_new = fmaxf(m, wave_max(sc));
@@ -69,7 +75,8 @@ paged_attention_generic_kernel(const TQ* __restrict__ q, int q_stride, const TC*
       if (d < hd) {
         float a = acc[i] * corr;
         for (int jj = 0; jj < n; ++jj)
-          a += ps[jj] * to_f32(vcache[(((size_t)pg[jj] * nkv + kvh) * hd + d) * page_size + of[jj]]);
+          a += ps[jj] * to_f32(vcache[((size_t)pg[jj] * nkv + kvh) * hd * page_size +
+                                      value_offset(d, of[jj], hd, page_size)]);
         acc[i] = a;
       }
     }

@@ -93,6 +93,15 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     for (int s = 0; s < KSTEPS; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
   }
 
+  // the lowest own position and the highest window start among this wave's live rows: blocks wholly between
+  // them need no mask
+  int p_lo = row_ok ? p_row : 0x7fffffff, lo_hi = row_ok ? lo_row : 0;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    p_lo = min(p_lo, __shfl_xor(p_lo, off, 64));
+    lo_hi = max(lo_hi, __shfl_xor(lo_hi, off, 64));
+  }
+
   const int32_t* table = block_tables + (size_t)task.entry * max_blocks;
   const float sc2 = scale * kLog2e;
   float m = -INFINITY, l = 0.f;
@@ -117,10 +126,11 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   };
   auto load_keys = [&](int p0, int p1, bf16x8* kf) {
     const int pg = (c < 16) ? p0 : p1;
-    const uint16_t* kp = kcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride + (size_t)(c & 15) * HD +
-                         hg * 8;
+    // tile order (cache_layout.h): for each 16 columns, the 8-column pieces of all 16 tokens side by side
+    const uint16_t* kp = kcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride +
+                         (size_t)(hg * PAGE + (c & 15)) * 8;
 #pragma unroll
-    for (int st = 0; st < KSTEPS; ++st) kf[st] = *reinterpret_cast<const bf16x8*>(kp + st * 16);
+    for (int st = 0; st < KSTEPS; ++st) kf[st] = *reinterpret_cast<const bf16x8*>(kp + st * (2 * PAGE * 8));
   };
   // V^T fragments of both pages: lane (d = dt*32 + c, key slots hg*4..+4 and 8 + hg*4..+4 of each page)
   auto load_vals = [&](int p0, int p1, bf16x8 (*vf)[DTILES]) {
@@ -131,11 +141,12 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       for (int dt = 0; dt < DTILES; ++dt) {
         const int d = dt * 32 + c;
         if (HD % 32 == 0 || d < HD) {
-          const uint16_t* vp = vcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride + (size_t)d * PAGE +
-                               hg * 4;
-          const bf16x4 a = *reinterpret_cast<const bf16x4*>(vp);
-          const bf16x4 b = *reinterpret_cast<const bf16x4*>(vp + 8);
-          vf[j][dt] = bf16x8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+          // tile order (cache_layout.h): this lane's eight key slots of column d are one 16-byte piece
+          constexpr int last_rows = HD % 32 == 0 ? 32 : HD % 32;
+          const int rows = (HD % 32 == 0 || dt < DTILES - 1) ? 32 : last_rows;
+          const uint16_t* vp = vcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride + dt * 512 +
+                               (size_t)(hg * rows + c) * 8;
+          vf[j][dt] = *reinterpret_cast<const bf16x8*>(vp);
         } else {
 #pragma unroll
           for (int i = 0; i < 8; ++i) vf[j][dt][i] = (__bf16)0.f;
@@ -199,36 +210,54 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       }
     }
 
-    // mask and online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4
-    float bmax = -INFINITY;
+    // Online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4.  The running maximum is kept in
+    // units of the scaled score (score * scale * log2 e), so one fused multiply-add feeds exp2.  Only blocks
+    // that touch a row's own position, the window's edge or the end of the key range need the mask.
+    const bool edge = kb + 31 > p_lo || kb < lo_hi || kb + 32 > task.k_end;
     float sv[16];
+    float bmax = -INFINITY;
+    if (edge) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
-      const bool ok = key <= p_row && key >= lo_row && key < task.k_end;
-      sv[i] = ok ? s[i] * sc2 : -INFINITY;
-      bmax = fmaxf(bmax, sv[i]);
+      for (int i = 0; i < 16; ++i) {
+        const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
+        const bool ok = key <= p_row && key >= lo_row && key < task.k_end;
+        sv[i] = ok ? s[i] : -INFINITY;
+        bmax = fmaxf(bmax, sv[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        sv[i] = s[i];
+        bmax = fmaxf(bmax, sv[i]);
+      }
     }
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64)) * sc2;
     const float m_new = fmaxf(m, bmax);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float corr = __builtin_amdgcn_exp2f(m - m_use);
     float psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      sv[i] = __builtin_amdgcn_exp2f(sv[i] - m_use);
+      sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
       psum += sv[i];
     }
     psum += __shfl_xor(psum, 32, 64);
-    l = l * corr + psum;
-    m = m_new;
+    // the accumulators are rescaled only when some row's maximum has grown (a wave-uniform decision)
+    const bool grew = __ballot(m_new > m) != 0;
+    if (grew) {
+      const float corr = __builtin_amdgcn_exp2f(m - m_use);
+      l *= corr;
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
+      m = m_new;
+    }
+    l += psum;
 
-    // O^T = O^T * corr + V^T P^T
+    // O^T += V^T P^T
     const bf16x8 p0 = pack8(sv), p1 = pack8(sv + 8);
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[0][dt], p0, o[dt], 0, 0, 0);
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[1][dt], p1, o[dt], 0, 0, 0);
     }

@@ -2,6 +2,7 @@
 // write of keys and values into the paged cache, SiLU(gate)*up.  All arithmetic is float32; element
 // types only decide how values are read and stored.
 #include "common.h"
+#include "cache_layout.h"
 
 using namespace atoma;
 
@@ -199,8 +200,8 @@ extern "C" int atoma_add_rmsnorm(float* resid, const void* delta, int delta_dtyp
 // ---------------------------------------------------------------------------------------------
 // Rotary encoding of q and k in half-split pairs (i, i + rd/2), and the write of k (rotated) and v into the
 // paged cache.  qkv is [T, row_stride]: q heads, then k heads, then v heads, each head hd wide.
-// q is rotated in place.  K pages are [page][kv_head][slot][hd]; V pages are [page][kv_head][hd][slot], so that
-// the attention kernels read keys along hd and values along the slot axis contiguously.
+// q is rotated in place.  Keys and values go into (page, kv_head) tiles of page_size * hd elements whose inner
+// order is that of cache_layout.h (the order in which the MFMA attention kernel reads them).
 // A negative slot, or null caches, skip the cache write (the reference skips negative slots:
 // csrc/kernels/cache_manager.cu:151-155).  cos/sin may be null: then nothing is rotated.
 // Pairing and signs: csrc/kernels/rotary.h:116-131; rotation applies to q and k only: models/src/llama.rs:298-299.
@@ -223,22 +224,22 @@ rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __r
   if (head >= nh + nkv) {
     // v: stored transposed inside the page
     if (slot < 0) return;
-    TC* dst = vcache + ((size_t)page * nkv + (head - nh - nkv)) * hd * page_size + off;
-    dst[(size_t)(2 * i) * page_size] = from_f32<TC>(to_f32(x[2 * i]));
-    dst[(size_t)(2 * i + 1) * page_size] = from_f32<TC>(to_f32(x[2 * i + 1]));
+    TC* tile = vcache + ((size_t)page * nkv + (head - nh - nkv)) * hd * page_size;
+    tile[value_offset(2 * i, off, hd, page_size)] = from_f32<TC>(to_f32(x[2 * i]));
+    tile[value_offset(2 * i + 1, off, hd, page_size)] = from_f32<TC>(to_f32(x[2 * i + 1]));
     return;
   }
   const bool is_k = head >= nh;
   if (is_k && slot < 0) return;
-  TC* kdst = is_k ? kcache + (((size_t)page * nkv + (head - nh)) * page_size + off) * hd : nullptr;
+  TC* ktile = is_k ? kcache + ((size_t)page * nkv + (head - nh)) * page_size * hd : nullptr;
   const int half = cos_t ? rotary_dim / 2 : 0;
   if (i < half) {
     const float c = cos_t[(size_t)positions[t] * half + i], sv = sin_t[(size_t)positions[t] * half + i];
     const float x1 = to_f32(x[i]), x2 = to_f32(x[i + half]);
     const float o1 = x1 * c - x2 * sv, o2 = x2 * c + x1 * sv;
     if (is_k) {
-      kdst[i] = from_f32<TC>(o1);
-      kdst[i + half] = from_f32<TC>(o2);
+      ktile[key_offset(off, i, page_size)] = from_f32<TC>(o1);
+      ktile[key_offset(off, i + half, page_size)] = from_f32<TC>(o2);
     } else {
       x[i] = from_f32<TA>(o1);
       x[i + half] = from_f32<TA>(o2);
@@ -246,8 +247,8 @@ rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __r
   } else if (is_k) {
     // columns beyond the rotary dimension are copied as they are (all of them without tables)
     const int a = 2 * half + 2 * (i - half);
-    kdst[a] = from_f32<TC>(to_f32(x[a]));
-    kdst[a + 1] = from_f32<TC>(to_f32(x[a + 1]));
+    ktile[key_offset(off, a, page_size)] = from_f32<TC>(to_f32(x[a]));
+    ktile[key_offset(off, a + 1, page_size)] = from_f32<TC>(to_f32(x[a + 1]));
   }
 }
 

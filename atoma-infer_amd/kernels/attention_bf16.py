@@ -171,6 +171,8 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
         return False
     if q.stride(0) % 8 or q.data_ptr() % 16 or out.stride(0) % 4:
         return False
+    if tuple(k_cache.shape[1:]) != (nkv, PAGE * hd) or tuple(v_cache.shape[1:]) != (nkv, PAGE * hd):
+        raise ValueError("cache tensors must be [pages, nkv, page_size * hd] tiles")
     group = nh // nkv
     plan = getattr(ctx, "plans", {}).get(plan_key(group, window))
     if plan is None:

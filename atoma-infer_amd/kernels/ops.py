@@ -129,7 +129,7 @@ def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[t
                      nkv: int, hd: int) -> None:
     """Rotate q and k of ``qkv`` [T, (nh + 2 nkv) hd] (q in place), store rotated k and v at ``slot_mapping``.
 
-    kcache is [pages, nkv, page_size, hd], vcache [pages, nkv, hd, page_size].  Null caches: rotate q only.
+    kcache and vcache are [pages, nkv, page_size * hd] tiles (order: cache/layout.py).  Null caches: rotate q only.
     """
     _dev(qkv, positions, cos, sin, kcache, vcache, slot_mapping)
     t = qkv.shape[0]
@@ -144,9 +144,9 @@ def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[t
         _need(vcache is not None and slot_mapping is not None, "cache write needs k, v and slots")
         _i32(slot_mapping, "slot_mapping", t)
         pages = kcache.shape[0]
-        _need(kcache.is_contiguous() and vcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size, hd)
-              and tuple(vcache.shape) == (pages, nkv, hd, page_size) and kcache.dtype is vcache.dtype,
-              "cache tensors must be [pages, nkv, page, hd] and [pages, nkv, hd, page]")
+        _need(kcache.is_contiguous() and vcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size * hd)
+              and tuple(vcache.shape) == (pages, nkv, page_size * hd) and kcache.dtype is vcache.dtype,
+              "cache tensors must be [pages, nkv, page_size * hd] tiles")
         cache_code = _code(kcache, "cache")
     _check(core().atoma_rope_cache_write(_p(qkv), _code(qkv, "qkv"), qkv.stride(0), _p(positions), _p(cos), _p(sin),
                                          rotary_dim, _p(kcache), _p(vcache), cache_code, _p(slot_mapping), page_size,
@@ -167,9 +167,9 @@ def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch
     _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == t and out.shape[1] >= nh * hd
           and out.dtype is q.dtype, "out: bad shape")
     pages = kcache.shape[0]
-    _need(kcache.is_contiguous() and vcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size, hd)
-          and tuple(vcache.shape) == (pages, nkv, hd, page_size) and kcache.dtype is vcache.dtype,
-          "cache tensors must be [pages, nkv, page, hd] and [pages, nkv, hd, page]")
+    _need(kcache.is_contiguous() and vcache.is_contiguous() and tuple(kcache.shape) == (pages, nkv, page_size * hd)
+          and tuple(vcache.shape) == (pages, nkv, page_size * hd) and kcache.dtype is vcache.dtype,
+          "cache tensors must be [pages, nkv, page_size * hd] tiles")
     _need(block_tables.dim() == 2 and block_tables.dtype is torch.int32 and block_tables.is_contiguous(),
           "block_tables must be contiguous int32 [requests, blocks]")
     _i32(token_seq, "token_seq", t)

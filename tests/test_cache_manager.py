@@ -177,3 +177,25 @@ def test_plan_cache_groups_layers_by_their_needs():
     with pytest.raises(ValueError):
         spec.run_order = [LayerCall(0), LayerCall(2, kv_from=0)]   # needs differ
         spec.__post_init__()
+
+
+@pytest.mark.parametrize("page,head", [(16, 64), (16, 48), (16, 16), (4, 16), (16, 256), (16, 80), (8, 32), (1, 32)])
+def test_tile_layout_is_a_permutation_and_serves_the_mfma_lanes(page, head):
+    import torch
+    from atoma_infer_amd.cache.layout import (key_index, pack_keys, pack_values, unpack_keys, unpack_values,
+                                               value_index)
+    ki, vi = key_index(page, head), value_index(page, head)
+    assert sorted(ki.reshape(-1).tolist()) == list(range(page * head))
+    assert sorted(vi.reshape(-1).tolist()) == list(range(page * head))
+    k, v = torch.randn(3, page, head), torch.randn(3, head, page)
+    assert torch.equal(unpack_keys(pack_keys(k), page, head), k)
+    assert torch.equal(unpack_values(pack_values(v), page, head), v)
+    # a lane's 8 columns of a key are contiguous; with 16-token pages a lane's 8 key slots of a value column too
+    for t in range(page):
+        for d0 in range(0, head, 8):
+            assert ki[t, d0:d0 + 8].tolist() == list(range(int(ki[t, d0]), int(ki[t, d0]) + 8))
+    if page == 16:
+        for d in range(head):
+            for hg in (0, 1):
+                slots = [int(vi[d, hg * 4 + i]) for i in range(4)] + [int(vi[d, 8 + hg * 4 + i]) for i in range(4)]
+                assert slots == list(range(slots[0], slots[0] + 8)) and slots[0] % 8 == 0

@@ -175,6 +175,7 @@ def paged_setup(lens, nkv, hd, page, dtype, seed=0):
     blocks = [-(-n // page) for n in lens]
     total = sum(blocks) + 3
     perm = torch.randperm(total, generator=g).tolist()
+    from atoma_infer_amd.cache.layout import pack_keys, pack_values
     kc = torch.randn(total, nkv, page, hd, generator=g).to(dtype)    # unused slots hold noise, not zeros
     vc = torch.randn(total, nkv, hd, page, generator=g).to(dtype)
     bt = torch.zeros(len(lens), max(blocks), dtype=torch.int32)
@@ -187,7 +188,7 @@ def paged_setup(lens, nkv, hd, page, dtype, seed=0):
             lo, hi = b * page, min((b + 1) * page, n)
             kc[pg, :, : hi - lo, :] = ks[e][lo:hi].permute(1, 0, 2)
             vc[pg, :, :, : hi - lo] = vs[e][lo:hi].permute(1, 2, 0)
-    return ks, vs, kc.to(DEV), vc.to(DEV), bt.to(DEV)
+    return ks, vs, pack_keys(kc).to(DEV), pack_values(vc).to(DEV), bt.to(DEV)
 
 
 def plain_attention(q, k, v, start, scale, window, group):
@@ -272,6 +273,8 @@ def test_attention_reference_vectors():
     vc = torch.zeros(1, nh, hd, page)
     kc[0, :, :2, :8] = k
     vc[0, :, :8, :2] = v.permute(0, 2, 1)
+    from atoma_infer_amd.cache.layout import pack_keys, pack_values
+    kc, vc = pack_keys(kc), pack_values(vc)
     out = torch.empty(2, nh * hd, device=DEV)
     bt = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
     ctx = FakeCtx([0], [2])
@@ -296,8 +299,10 @@ def test_rope_cache_write(dtype):
     slots = torch.tensor([8, 9, 10, 11, 0, 1, -1, 30, 31], dtype=torch.int32)
     kc = torch.zeros(8, nkv, page, hd, dtype=dtype)
     vc = torch.zeros(8, nkv, hd, page, dtype=dtype)
-    d_qkv, d_kc, d_vc = qkv.to(DEV), kc.to(DEV), vc.to(DEV)
+    from atoma_infer_amd.cache.layout import pack_keys, pack_values, unpack_keys, unpack_values
+    d_qkv, d_kc, d_vc = qkv.to(DEV), pack_keys(kc).to(DEV), pack_values(vc).to(DEV)
     ops.rope_cache_write(d_qkv, pos.to(DEV), cos.to(DEV), sin.to(DEV), hd, d_kc, d_vc, slots.to(DEV), page, nh, nkv, hd)
+    d_kc, d_vc = unpack_keys(d_kc, page, hd), unpack_values(d_vc, page, hd)
     x = qkv.float().view(t, nh + 2 * nkv, hd)
     c, s = cos[pos.long()][:, None, :], sin[pos.long()][:, None, :]
     x1, x2 = x[..., : hd // 2], x[..., hd // 2:]
