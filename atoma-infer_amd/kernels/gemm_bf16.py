@@ -56,7 +56,9 @@ def _plan(m: int, n: int, k: int, allow_slices: bool):
     slices = 1
     if allow_slices:
         groups = -(-tiles // ((4 if wk == 1 else 1) * rt))
-        slices = 8
+        # two planes already put enough workgroups in flight (more measured no faster) and keep the consumer,
+        # which adds the planes, cheap
+        slices = 2
         while slices > 1 and (k % (32 * wk * slices) or k // (wk * slices) < 128 or groups * slices > 1024):
             slices //= 2
     return rt, wk, slices
