@@ -339,3 +339,19 @@ extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, 
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// dst[dst_idx[i]] = src[src_idx[i]]: puts tokens sampled by the previous step, which the host has not seen yet,
+// into the next step's token list on the device.  pairs = [n][2] (dst index, src index).
+__global__ void feed_tokens_kernel(int32_t* __restrict__ dst, const int32_t* __restrict__ src,
+                                   const int32_t* __restrict__ pairs, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[pairs[2 * i]] = src[pairs[2 * i + 1]];
+}
+
+extern "C" int atoma_feed_tokens(int32_t* dst, const int32_t* src, const int32_t* pairs, int n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(feed_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, dst, src, pairs, n);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}

@@ -8,6 +8,7 @@ thread and one process.  The cache pool is sized after the weights are on the de
 """
 from __future__ import annotations
 
+import dataclasses
 import os
 import time
 from typing import Dict, List, Optional, Sequence, Union
@@ -18,12 +19,21 @@ from ..cache.pool import CachePool, pages_for_memory, plan_cache
 from ..config.engine import CacheConfig, EngineConfig, SchedulerConfig, ValidationConfig, parse_dtype
 from ..models.model import Model, load_model
 from ..sampling.params import GenerateParameters, ValidationError, validate
-from ..sampling.sampler import Sampler
+from ..sampling.sampler import Pending, Sampler
 from .request import GenerateRequestOutput, Request, RequestMetrics, Status
 from .scheduler import ScheduleOutput, Scheduler
 from .step import ModelRunner, RunnerCache, StepEntry
 
 Inputs = Union[str, Sequence[int]]
+
+
+@dataclasses.dataclass
+class _InFlight:
+    """A launched step whose sampled tokens the host has not read yet."""
+    sampled: List[Request]
+    pending: Optional[Pending]
+    rows: Dict[int, int]          # request uid -> row of the sampled tokens
+    sync: bool                    # the tokens are needed before the next step can be planned
 
 
 class LlmEngine:
@@ -63,6 +73,7 @@ class LlmEngine:
         self._next_uid = 0
         self._requests: Dict[str, Request] = {}
         self.tokenizer = None
+        self._in_flight: Optional[_InFlight] = None
         self.stats = {"steps": 0, "tokens": 0, "sampled": 0, "preemptions": 0}
 
     # -- construction from the reference's TOML ----------------------------------------------------------
@@ -122,49 +133,102 @@ class LlmEngine:
         return rid
 
     def abort(self, request_id: str) -> Optional[GenerateRequestOutput]:
+        self.drain()
         r = self.scheduler.abort(request_id)
         if r is None:
             return None
         return self._output(r)
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_unfinished()
+        return self.scheduler.has_unfinished() or self._in_flight is not None
 
     # -- one step ------------------------------------------------------------------------------------------
     def step(self) -> List[GenerateRequestOutput]:
-        """Plan, run and sample one step; returns the requests that finished in it."""
+        """Plan and launch one step, then read the tokens of the step before it; returns the requests that finished.
+
+        The engine runs one step ahead of the host's knowledge of the sampled tokens: the tokens a step samples
+        stay on the device, where the next step reads them, and reach the host while that next step runs.  So the
+        GPU does not wait for scheduling and bookkeeping.  A request that ends on a token (EOS, a stop string) is
+        seen one step late; the token it sampled meanwhile is dropped.  Requests whose sampling needs the host to
+        know every earlier token (a repeat penalty, stop strings) are read at once instead.
+        """
         plan: ScheduleOutput = self.scheduler.schedule()
         finished: List[Request] = list(plan.ignored) + list(plan.capped)
         self.stats["preemptions"] += len(plan.preempted)
+        launched = None
         if not plan.empty:
-            entries, sampled = [], []
-            for e in plan.entries:
-                r = e.request
-                entries.append(StepEntry(r.uid, r.next_tokens(e.num_tokens), e.start,
-                                         [e.num_tokens - 1] if e.do_sample else []))
-                if e.do_sample:
-                    sampled.append(r)
-            logits = self.runner.step(entries)
-            now = time.monotonic()
-            for e in plan.entries:
-                e.request.num_computed += e.num_tokens
-            self.stats["steps"] += 1
-            self.stats["tokens"] += plan.num_tokens
-            if sampled:
-                toks, lgs = self.sampler.sample(logits, [r.plan for r in sampled],
-                                                [len(r.output_ids) for r in sampled],
-                                                [r.all_ids() if r.plan.repetition_penalty != 1.0 else ()
-                                                 for r in sampled])
-                self.stats["sampled"] += len(sampled)
-                for r, tok, lg in zip(sampled, toks, lgs):
-                    status = self._append(r, tok, lg, now)
-                    if status is not None:
-                        self.scheduler.finish(r, status)
-                        finished.append(r)
+            launched = self._launch(plan)
+        if self._in_flight is not None:
+            finished += self._resolve(self._in_flight)
+        self._in_flight = launched
+        if launched is not None and launched.sync:
+            finished += self._resolve(launched)
+            self._in_flight = None
         outs = []
         for r in finished:
             r.metrics.finished_time = time.monotonic()
             outs.append(self._output(r))
+        return outs
+
+    def _launch(self, plan: ScheduleOutput) -> "_InFlight":
+        prev = self._in_flight
+        entries, sampled = [], []
+        for e in plan.entries:
+            r = e.request
+            feed = -1
+            if e.num_tokens == 1 and r.num_computed == len(r.prompt_ids) + len(r.output_ids):
+                # its last token is still on the device: row of the previous step's sampled tokens
+                feed = prev.rows[r.uid]
+            entries.append(StepEntry(r.uid, r.next_tokens(e.num_tokens), e.start,
+                                     [e.num_tokens - 1] if e.do_sample else [], feed))
+            if e.do_sample:
+                sampled.append(r)
+        logits = self.runner.step(entries, prev.pending.tokens if prev is not None and prev.pending else None)
+        for e in plan.entries:
+            e.request.num_computed += e.num_tokens
+        self.stats["steps"] += 1
+        self.stats["tokens"] += plan.num_tokens
+        flight = _InFlight(sampled, None, {r.uid: i for i, r in enumerate(sampled)}, False)
+        if sampled:
+            flight.pending = self.sampler.launch(
+                logits, [r.plan for r in sampled], [r.num_sampled for r in sampled],
+                [r.all_ids() if r.plan.repetition_penalty != 1.0 else () for r in sampled])
+            self.stats["sampled"] += len(sampled)
+            limit = self.scheduler_config.max_model_len
+            for r in sampled:
+                r.pending += 1
+                # by count alone this may be the request's last token: then nothing more is scheduled for it
+                if r.num_sampled >= r.plan.max_new_tokens or r.length > limit:
+                    r.frozen = True
+                if r.plan.repetition_penalty != 1.0 or r.plan.stop:
+                    flight.sync = True
+        return flight
+
+    def _resolve(self, flight: "_InFlight") -> List[Request]:
+        """Read the tokens of a launched step and apply them; returns the requests that ended."""
+        done: List[Request] = []
+        if flight.pending is None:
+            return done
+        toks, lgs = flight.pending.result()
+        now = time.monotonic()
+        for r, tok, lg in zip(flight.sampled, toks, lgs):
+            r.pending -= 1
+            if r.status.finished:
+                continue      # it ended on an earlier token; this one was sampled in vain
+            status = self._append(r, tok, lg, now)
+            if status is not None:
+                self.scheduler.finish(r, status)
+                done.append(r)
+        return done
+
+    def drain(self) -> List[GenerateRequestOutput]:
+        """Read what is still in flight (call before reading clocks or state from outside)."""
+        outs = []
+        if self._in_flight is not None:
+            for r in self._resolve(self._in_flight):
+                r.metrics.finished_time = time.monotonic()
+                outs.append(self._output(r))
+            self._in_flight = None
         return outs
 
     def _append(self, r: Request, tok: int, logit: float, now: float) -> Optional[Status]:
@@ -182,7 +246,7 @@ class LlmEngine:
         if tok in self.eos_ids and not r.plan.ignore_eos_token:
             r.stop_reason = tok
             return Status.FINISHED_STOPPED
-        if r.length > self.scheduler_config.max_model_len:
+        if len(r.prompt_ids) + len(r.output_ids) > self.scheduler_config.max_model_len:
             return Status.FINISHED_LENGTH_CAPPED
         if len(r.output_ids) >= r.plan.max_new_tokens:
             return Status.FINISHED_LENGTH_CAPPED

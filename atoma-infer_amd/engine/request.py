@@ -51,10 +51,18 @@ class Request:
     num_computed: int = 0         # tokens whose keys and values are in the cache
     status: Status = Status.WAITING
     stop_reason: Optional[object] = None
+    #: tokens sampled on the device that the host has not read yet (the engine runs one step ahead of them)
+    pending: int = 0
+    #: the token that ends this request by count is on its way: nothing more is scheduled for it
+    frozen: bool = False
 
     @property
     def length(self) -> int:
-        return len(self.prompt_ids) + len(self.output_ids)
+        return len(self.prompt_ids) + len(self.output_ids) + self.pending
+
+    @property
+    def num_sampled(self) -> int:
+        return len(self.output_ids) + self.pending
 
     @property
     def num_uncomputed(self) -> int:
@@ -64,12 +72,17 @@ class Request:
 
     @property
     def in_prefill(self) -> bool:
-        return self.num_uncomputed > 1 or not self.output_ids
+        return self.num_uncomputed > 1 or self.num_sampled == 0
 
     def all_ids(self) -> List[int]:
         return self.prompt_ids + self.output_ids
 
     def next_tokens(self, n: int) -> List[int]:
+        """The next ``n`` tokens to run.  A token still pending on the device is given as 0; the caller feeds it."""
+        known = len(self.prompt_ids) + len(self.output_ids)
+        if self.num_computed + n > known:
+            assert n == 1 and self.num_computed == known and self.pending > 0
+            return [0]
         lo = self.num_computed
         p = len(self.prompt_ids)
         if lo + n <= p:

@@ -95,9 +95,13 @@ class Scheduler:
         return None
 
     def finish(self, request: Request, status: Status) -> None:
-        """A running request has produced its last token: give back what it holds."""
+        """A request has produced its last token: give back what it holds.  It is usually running; it waits if it
+        was preempted while that token was still on its way."""
         assert status.finished
-        self.running.remove(request)
+        if request.status is Status.RUNNING:
+            self.running.remove(request)
+        else:
+            self.waiting.remove(request)
         self._release(request)
         request.status = status
 
@@ -146,7 +150,8 @@ class Scheduler:
             return sum(e.num_tokens for e in out.entries)
 
         # 1 and 2: running requests, decodes before portions of prompts
-        order = [r for r in self.running if not r.in_prefill] + [r for r in self.running if r.in_prefill]
+        live = [r for r in self.running if not r.frozen]
+        order = [r for r in live if not r.in_prefill] + [r for r in live if r.in_prefill]
         if len(order) <= cfg.max_num_sequences and len(order) <= cfg.max_num_batched_tokens and \
                 all(r.num_uncomputed == 1 for r in order):
             # the common step: everything running decodes one token and fits both budgets; pages are taken
@@ -168,7 +173,8 @@ class Scheduler:
             if n <= 0:
                 continue
             while not self.cache.can_reserve(r.uid, r.num_computed + n):
-                victim = self.running[-1]
+                # the latest arrival that is not just waiting for its last token (that one frees its pages soon)
+                victim = next((v for v in reversed(self.running) if not v.frozen), r)
                 if victim is r and len(self.running) == 1:
                     # nothing else to give back: the pool cannot hold this request any longer
                     self.running.remove(r)

@@ -45,6 +45,9 @@ class StepEntry:
     tokens: Sequence[int]
     start: int
     want: Sequence[int] = ()
+    #: for an entry of one token that the host does not know yet: the row of the previous step's sampled tokens
+    #: (a device tensor given to ``step``) to take it from; ``tokens`` then holds any valid id as a stand-in
+    feed: int = -1
 
 
 @dataclasses.dataclass
@@ -209,8 +212,11 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= w < n:
                     raise StepError(f"request {e.request}: wanted place {w} outside its {n} tokens")
+            if e.feed >= 0 and n != 1:
+                raise StepError(f"request {e.request}: only an entry of one token can be fed from the device")
 
-    def _build(self, entries: Sequence[StepEntry], stage: _Staging, bucket: Optional[int]) -> StepContext:
+    def _build(self, entries: Sequence[StepEntry], stage: _Staging, bucket: Optional[int],
+               feed_src: Optional[torch.Tensor] = None) -> StepContext:
         """Fill ``stage`` with the step's metadata, start its copy to the device and describe it.
 
         With ``bucket`` (decode graphs) every size is a function of (entries, bucket) alone, so the layout, and
@@ -238,7 +244,8 @@ class ModelRunner:
         o_want = 3 * t + 3 * s + 1
         o_sm = o_want + n_want
         o_bt = o_sm + n_groups * t
-        total = o_bt + n_groups * s * max_blocks
+        o_feed = o_bt + n_groups * s * max_blocks          # pairs (token row, row of the fed tokens), 2 per entry
+        total = o_feed + 2 * s
         ex_off = []
         for _, arr, _ in extras:
             total += (-total) % 4                  # every extra starts on a 16-byte boundary
@@ -250,8 +257,13 @@ class ModelRunner:
         np.cumsum(counts, out=q_start[1:])
         row = 0
         wi = o_want
+        n_feed = 0
         for i, e in enumerate(entries):
             n = counts[i]
+            if e.feed >= 0:
+                buf[o_feed + 2 * n_feed] = row
+                buf[o_feed + 2 * n_feed + 1] = e.feed
+                n_feed += 1
             buf[o_tok + row: o_tok + row + n] = e.tokens
             buf[o_pos + row: o_pos + row + n] = np.arange(e.start, e.start + n, dtype=np.int32)
             buf[o_seq + row: o_seq + row + n] = i
@@ -271,6 +283,9 @@ class ModelRunner:
             buf[off: off + arr.size] = arr.reshape(-1)
         stage.upload(total)
         dev = stage.dev
+        if n_feed:
+            from ..kernels import ops
+            ops.feed_tokens(dev[o_tok: o_tok + t], feed_src, dev[o_feed: o_feed + 2 * n_feed].view(n_feed, 2))
         ctx = StepContext(
             n_tokens=t, n_entries=s, n_want=n_want,
             tokens=dev[o_tok: o_tok + t], positions=dev[o_pos: o_pos + t], token_seq=dev[o_seq: o_seq + t],
@@ -298,8 +313,10 @@ class ModelRunner:
             self._computed[e.request] = done
             self.manager.release_behind(e.request, done)
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], feed_src: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run one batch; returns float32 logits [wanted places, vocab] (order: entries, then ``want``) or None.
+
+        ``feed_src`` (int32 device tensor) supplies the token of every entry with ``feed >= 0``.
 
         The tensor returned by a decode step belongs to that step's graph and is overwritten by the next step of
         the same shape: use it (sample, copy) before stepping again.
@@ -309,14 +326,14 @@ class ModelRunner:
             self.manager.reserve(e.request, e.start + len(e.tokens))
         logits = None
         if self.use_graphs and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries):
-            logits = self._decode_with_graph(entries)
+            logits = self._decode_with_graph(entries, feed_src)
         if logits is None:
-            ctx = self._build(entries, self._stage, None)
+            ctx = self._build(entries, self._stage, None, feed_src)
             logits = self.model.forward(ctx)
         self._finish(entries)
         return logits
 
-    def _decode_with_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _decode_with_graph(self, entries: Sequence[StepEntry], feed_src=None) -> Optional[torch.Tensor]:
         s = len(entries)
         max_seq = max(e.start for e in entries) + 1
         key = (s, -(-max_seq // DECODE_BUCKET))
@@ -328,7 +345,7 @@ class ModelRunner:
                 self._graphs.popitem(last=False)
             return None
         self._graphs.move_to_end(key)
-        ctx = self._build(entries, g.stage, key[1])
+        ctx = self._build(entries, g.stage, key[1], feed_src)
         if g.graph is None:
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()

@@ -243,3 +243,13 @@ def repeat_penalty(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tenso
     _need(penalty.dtype is torch.float32 and penalty.numel() == logits.shape[0], "penalty must be float32 [S]")
     _check(core().atoma_repeat_penalty(_p(logits), logits.stride(0), _p(rows), _p(tokens), _p(penalty), n, _stream()),
            "repeat_penalty")
+
+
+def feed_tokens(dst: torch.Tensor, src: torch.Tensor, pairs: torch.Tensor) -> None:
+    """dst[pairs[i, 0]] = src[pairs[i, 1]] for int32 device tensors; the caller guarantees the indices' ranges."""
+    _dev(dst, src, pairs)
+    _i32(dst, "dst")
+    _i32(src, "src")
+    _need(pairs.dtype is torch.int32 and pairs.is_contiguous() and pairs.dim() == 2 and pairs.shape[1] == 2,
+          "pairs must be contiguous int32 [n, 2]")
+    _check(core().atoma_feed_tokens(_p(dst), _p(src), _p(pairs), pairs.shape[0], _stream()), "feed_tokens")

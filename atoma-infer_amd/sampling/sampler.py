@@ -28,17 +28,30 @@ def uniform(seed: int, counter: int) -> float:
     return (z >> 40) / float(1 << 24)
 
 
+class Pending:
+    """A sampling launched on the device whose tokens the host has not read yet."""
+
+    def __init__(self, tokens: torch.Tensor, logits: torch.Tensor, host: torch.Tensor, event: torch.cuda.Event):
+        self.tokens, self.logits, self._host, self._event = tokens, logits, host, event
+
+    def result(self) -> Tuple[List[int], List[float]]:
+        """Wait for the copy and return (tokens, logits of the chosen tokens)."""
+        self._event.synchronize()
+        n = self.tokens.numel()
+        return self._host[0, :n].view(torch.int32).tolist(), self._host[1, :n].tolist()
+
+
 class Sampler:
     def __init__(self, device: torch.device):
         self.device = device
 
-    def sample(self, logits: torch.Tensor, plans: Sequence[SamplingPlan], steps: Sequence[int],
-               contexts: Sequence[Sequence[int]]) -> Tuple[List[int], List[float]]:
-        """One token per row of ``logits`` [S, V].
+    def launch(self, logits: torch.Tensor, plans: Sequence[SamplingPlan], steps: Sequence[int],
+               contexts: Sequence[Sequence[int]]) -> Pending:
+        """Start sampling one token per row of ``logits`` [S, V]; nothing waits for the GPU.
 
         ``steps[i]`` is how many tokens request i has sampled before (the generator's counter); ``contexts[i]``
-        the token ids (prompt and output) the repeat penalty looks back over.
-        Returns the tokens and the (penalised) logits of the chosen tokens.
+        the token ids (prompt and output) the repeat penalty looks back over.  The sampled tokens stay on the
+        device (``Pending.tokens``, int32 [S]) for the next step to read, and travel to the host in the background.
         """
         s = logits.shape[0]
         assert len(plans) == s and len(steps) == s
@@ -49,18 +62,30 @@ class Sampler:
                 pen_rows += [i] * len(uniq)
                 pen_toks += list(uniq)
         # one packed upload: temperature, top_p, uniform, penalty (float32) and top_k (int32 bits)
-        meta = np.zeros((5, s), dtype=np.float32)
-        top_k = meta[4].view(np.int32)
+        meta = torch.empty((5, s), dtype=torch.float32, pin_memory=True)
+        mn = meta.numpy()
+        top_k = mn[4].view(np.int32)
         for i, pl in enumerate(plans):
-            meta[0, i] = 0.0 if pl.greedy else pl.temperature
-            meta[1, i] = pl.top_p
-            meta[2, i] = uniform(pl.random_seed, steps[i]) if not pl.greedy else 0.0
-            meta[3, i] = pl.repetition_penalty
+            mn[0, i] = 0.0 if pl.greedy else pl.temperature
+            mn[1, i] = pl.top_p
+            mn[2, i] = uniform(pl.random_seed, steps[i]) if not pl.greedy else 0.0
+            mn[3, i] = pl.repetition_penalty
             top_k[i] = pl.top_k
-        m = torch.from_numpy(meta).to(self.device)
+        m = meta.to(self.device, non_blocking=True)
         if pen_rows:
-            pen = torch.tensor([pen_rows, pen_toks], dtype=torch.int32, device=self.device)
+            pen = torch.tensor([pen_rows, pen_toks], dtype=torch.int32).to(self.device)
             ops.repeat_penalty(logits, pen[0], pen[1], m[3])
         tok, lg = ops.sample(logits, m[0], m[4].view(torch.int32), m[1], m[2])
-        both = torch.stack([tok.view(torch.float32), lg]).cpu()      # one download
-        return both[0].view(torch.int32).tolist(), both[1].tolist()
+        host = torch.empty((2, s), dtype=torch.float32, pin_memory=True)
+        host[0].copy_(tok.view(torch.float32), non_blocking=True)
+        host[1].copy_(lg, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        pending = Pending(tok, lg, host, ev)
+        pending._meta = meta          # pinned memory must outlive the copy that reads it
+        return pending
+
+    def sample(self, logits: torch.Tensor, plans: Sequence[SamplingPlan], steps: Sequence[int],
+               contexts: Sequence[Sequence[int]]) -> Tuple[List[int], List[float]]:
+        """``launch`` and wait: the tokens and the (penalised) logits of the chosen tokens."""
+        return self.launch(logits, plans, steps, contexts).result()

@@ -60,11 +60,13 @@ def decode_run(model, batch, prompt_len, steps, warmup, context, seed=0):
         eng.step()
     for _ in range(warmup):
         eng.step()
+    eng.drain()
     ctx0 = sum(r.length for r in eng.scheduler.running)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         eng.step()
+    eng.drain()             # the engine runs one step ahead of the sampled tokens: read the last ones too
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ctx1 = sum(r.length for r in eng.scheduler.running)
