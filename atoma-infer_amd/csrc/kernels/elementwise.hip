@@ -279,14 +279,22 @@ extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(z) = z * sigmoid(z).
+// out[t, i] = silu(gate[t, i]) * up[t, i], silu(z) = z * sigmoid(z); gate and up come in one row of 2 * inter.
 // Reference: models/src/llama.rs:364.
+// Where gate and up of output i lie in a row of 2 * inter values: in two halves (block == 0), or interleaved in
+// blocks of 16 gate values followed by their 16 up values (block == 16), the layout of the fused gate-up product.
+__device__ __forceinline__ int gate_index(int i, int block) { return block ? ((i >> 4) << 5) + (i & 15) : i; }
+__device__ __forceinline__ int up_index(int i, int inter, int block) {
+  return block ? ((i >> 4) << 5) + 16 + (i & 15) : inter + i;
+}
+
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total, int block) {
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / inter;
     const int i = (int)(idx % inter);
-    const float g = to_f32(gu[t * 2 * inter + i]), u = to_f32(gu[t * 2 * inter + inter + i]);
+    const float g = to_f32(gu[t * 2 * inter + gate_index(i, block)]);
+    const float u = to_f32(gu[t * 2 * inter + up_index(i, inter, block)]);
     out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
   }
 }
@@ -294,13 +302,14 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
 // four values per thread; needs inter % 4 == 0 and 16-byte aligned rows
 template <typename T>
 __global__ void __launch_bounds__(256)
-swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int n_tokens) {
+swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int n_tokens, int block) {
   const int quads = inter >> 2;
   const size_t total = (size_t)n_tokens * quads;
   for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
     const size_t t = idx / quads;
     const int i = (int)(idx % quads) * 4;
-    const f4 g = load4(gu + t * 2 * inter + i), u = load4(gu + t * 2 * inter + inter + i);
+    const f4 g = load4(gu + t * 2 * inter + gate_index(i, block));
+    const f4 u = load4(gu + t * 2 * inter + up_index(i, inter, block));
     f4 o;
 #pragma unroll
     for (int e = 0; e < 4; ++e) o.v[e] = g.v[e] / (1.0f + expf(-g.v[e])) * u.v[e];
@@ -308,8 +317,10 @@ swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int 
   }
 }
 
-extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, hipStream_t stream) {
+extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, int block,
+                            hipStream_t stream) {
   if (n_tokens <= 0) return 0;
+  if (block != 0 && (block != 16 || inter % 16)) return ATOMA_ERR_SHAPE;
   const size_t total = (size_t)n_tokens * inter;
   if (inter % 4 == 0 && ((uintptr_t)gu & 15) == 0 && ((uintptr_t)out & 15) == 0) {
     size_t quads = total / 4;
@@ -317,10 +328,10 @@ extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, 
     if (vb > 16384) vb = 16384;
     if (dtype == kF32)
       hipLaunchKernelGGL(swiglu_vec_kernel<float>, dim3(vb), dim3(256), 0, stream, (const float*)gu, (float*)out, inter,
-                         n_tokens);
+                         n_tokens, block);
     else if (dtype == kBF16)
       hipLaunchKernelGGL(swiglu_vec_kernel<bf16_t>, dim3(vb), dim3(256), 0, stream, (const bf16_t*)gu, (bf16_t*)out,
-                         inter, n_tokens);
+                         inter, n_tokens, block);
     else
       return ATOMA_ERR_DTYPE;
     ATOMA_LAUNCH_CHECK();
@@ -330,10 +341,10 @@ extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, 
   if (blocks > 65536) blocks = 65536;
   if (dtype == kF32)
     hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)gu, (float*)out, inter,
-                       total);
+                       total, block);
   else if (dtype == kBF16)
     hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)gu, (bf16_t*)out,
-                       inter, total);
+                       inter, total, block);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();

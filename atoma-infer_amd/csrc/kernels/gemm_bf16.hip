@@ -19,7 +19,7 @@ using namespace atoma;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-template <int MT, int RT, int WN, int WK, typename TC>
+template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false>
 __global__ void __launch_bounds__(64 * WN * WK)
 gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
                    int K, int lda, int ldw, int ldc, size_t plane) {
@@ -131,6 +131,33 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
     }
   }
 
+  if constexpr (SWIGLU) {
+    // W holds, for every 16 outputs, 16 gate rows followed by 16 up rows: row tile r is a gate tile, r + 1 its
+    // up tile, and the lane that holds gate value (n, row) holds up value (n, row) too.
+    // C[row][n] = silu(gate) * up, with N / 2 columns (the reference: models/src/llama.rs:364).
+    static_assert(!SWIGLU || (RT % 2 == 0 && sizeof(TC) == 2), "swiglu epilogue needs pairs of tiles, bf16 out");
+#pragma unroll
+    for (int r = 0; r < RT; r += 2) {
+      const int n0 = (n_base + r * 16) / 2 + kg * 4;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const int row = m * 16 + r16;
+        if (row >= M || n0 + 3 >= N / 2) continue;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float g = acc[r][m][i];
+          v[i] = g / (1.0f + expf(-g)) * acc[r + 1][m][i];
+        }
+        uint2 o;
+        o.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+        o.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(c) + (size_t)row * ldc + n0) = o;
+      }
+    }
+    return;
+  }
+
   // D[n = kg*4 + i][row of A = r16]: four consecutive columns of C per lane
   TC* cp = c + (size_t)blockIdx.y * plane;
 #pragma unroll
@@ -207,5 +234,41 @@ extern "C" int atoma_gemm_bf16_skinny(const void* a, const void* w, void* c, int
     case 2: return launch_mt<2>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
     case 3: return launch_mt<3>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
     default: return launch_mt<4>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
+  }
+}
+
+template <int MT, int RT, int WN, int WK>
+static int launch_swiglu(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
+                         hipStream_t stream) {
+  dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, true>), grid, block, 0, stream, (const uint16_t*)a,
+                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int MT>
+static int launch_swiglu_mt(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
+                            int rt, int wk, hipStream_t stream) {
+  if (rt == 2 && wk == 1) return launch_swiglu<MT, 2, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+  if (rt == 4 && wk == 1) return launch_swiglu<MT, 4, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+  if (rt == 2 && wk == 4) return launch_swiglu<MT, 2, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+  if (rt == 2 && wk == 8) return launch_swiglu<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+  return ATOMA_ERR_SHAPE;
+}
+
+// The gate-up product with SiLU(gate) * up in its epilogue.  w [N, K] holds gate and up rows interleaved in blocks
+// of 16 (16 gate rows, then the 16 up rows of the same outputs); c is [M, N / 2] bfloat16.  N % 32 == 0.
+extern "C" int atoma_gemm_bf16_skinny_swiglu(const void* a, const void* w, void* c, int M, int N, int K, int lda,
+                                             int ldw, int ldc, int rt, int wk, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % (32 * wk) || (N & 31) || (lda & 7) || (ldw & 7) || lda < K || ldw < K || ldc < N / 2 ||
+      (ldc & 3) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)c & 7))
+    return ATOMA_ERR_SHAPE;
+  switch ((M + 15) / 16) {
+    case 1: return launch_swiglu_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
+    case 2: return launch_swiglu_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
+    case 3: return launch_swiglu_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
+    default: return launch_swiglu_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
   }
 }

@@ -41,13 +41,14 @@ def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
 
 
 def chunk_for(n_split: int, max_keys: int) -> int:
-    """Keys per partial task: 64, 128 or 256, the smallest that keeps the step's partial tasks under a bound.
+    """Keys per partial task: 128 or 256, the smaller if that keeps the step's partial tasks under a bound.
 
     A wave walks its keys one 32-key block after another, so short chunks shorten the chain when few requests
-    decode, and long ones save partial results when many do.  ``max_keys`` is rounded up to 256.
+    decode, and long ones save partial results (and time in the combine kernel) when many do; measured on
+    MI355X, 128 wins up to about 8 requests of 2,000 tokens and 256 beyond.  ``max_keys`` is rounded up to 256.
     """
     buckets = -(-max_keys // CHUNK)
-    for chunk in (64, 128):
+    for chunk in (128,):
         if n_split * buckets * (CHUNK // chunk) <= MAX_SPLIT_TASKS:
             return chunk
     return CHUNK

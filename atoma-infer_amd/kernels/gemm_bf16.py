@@ -116,3 +116,23 @@ def linear_planes(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
     out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
     skinny(x, w, out, slices, rt, wk)
     return out
+
+
+def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
+    """silu(gate) * up of x @ w^T in one kernel, for few rows of x; w [2 I, K] is interleaved in blocks of 16.
+
+    None when the shape is not taken (the caller then runs the product and the activation separately).
+    """
+    m, k = x.shape
+    n = w.shape[0]
+    if m > LIBRARY_MIN_M_WIDE or n % 32 or not skinny_ok(x, w):
+        return None
+    rt, wk, _ = _plan(m, n, k, False)
+    if rt % 2:
+        rt = 2
+    if (rt, wk) not in ((2, 1), (4, 1), (2, 4), (2, 8)):
+        return None
+    out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    _check(lib().atoma_gemm_bf16_skinny_swiglu(_p(x), _p(w), _p(out), m, n, k, x.stride(0) if m > 1 else k,
+                                               w.stride(0), n // 2, rt, wk, _stream()), "gemm_bf16_skinny_swiglu")
+    return out

@@ -180,15 +180,19 @@ def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch
         page_size, t, nh, nkv, hd, _stream()), "paged_attention_generic")
 
 
-def swiglu(gu: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t, i] = silu(gu[t, i]) * gu[t, I + i] for gu [T, 2 I]."""
+def swiglu(gu: torch.Tensor, out: Optional[torch.Tensor] = None, block: int = 0) -> torch.Tensor:
+    """out[t, i] = silu(gate[t, i]) * up[t, i] for gu [T, 2 I].
+
+    ``block`` 0: gate is the first half of a row and up the second; 16: blocks of 16 gate values followed by
+    their 16 up values (the order of the fused gate-up product's weight rows).
+    """
     _dev(gu)
     _need(gu.dim() == 2 and gu.is_contiguous() and gu.shape[1] % 2 == 0, "swiglu input must be contiguous [T, 2 I]")
     t, inter = gu.shape[0], gu.shape[1] // 2
     if out is None:
         out = torch.empty((t, inter), dtype=gu.dtype, device=gu.device)
     _need(out.is_contiguous() and tuple(out.shape) == (t, inter) and out.dtype is gu.dtype, "swiglu: bad out")
-    _check(core().atoma_swiglu(_p(gu), _p(out), _code(gu, "swiglu input"), t, inter, _stream()), "swiglu")
+    _check(core().atoma_swiglu(_p(gu), _p(out), _code(gu, "swiglu input"), t, inter, int(block), _stream()), "swiglu")
     return out
 
 

@@ -1,6 +1,9 @@
 """Dense SwiGLU feed-forward: ``down(silu(gate(x)) * up(x))``, no biases (models/src/llama.rs:362-366, 372-374).
 
 gate and up are fused into one [2 I, width] matrix at load time, so one product feeds the SiLU-multiply kernel.
+When I is a multiple of 16 the rows are interleaved in blocks of 16 (16 gate rows, then the 16 up rows of the
+same outputs): a lane of the weight-streaming MFMA product then holds a gate value and its up value, and the
+activation runs in that product's epilogue for few rows of x.
 """
 from __future__ import annotations
 
@@ -16,6 +19,7 @@ from .linear import linear, linear_delta
 class SwiGLU(FeedForward):
     def __init__(self, width: int, intermediate: int):
         self.width, self.inter = int(width), int(intermediate)
+        self.block = 0
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
@@ -27,14 +31,26 @@ class SwiGLU(FeedForward):
     def load(self, get, device, act_dtype) -> None:
         g, u = get("gate_proj.weight"), get("up_proj.weight")
         dt = g.dtype if g.dtype is u.dtype else torch.float32
-        self.w_gate_up = torch.cat([g.to(device=device, dtype=dt), u.to(device=device, dtype=dt)], dim=0).contiguous()
+        g, u = g.to(device=device, dtype=dt), u.to(device=device, dtype=dt)
+        self.block = 16 if self.inter % 16 == 0 else 0
+        if self.block:
+            gu = torch.stack([g.view(self.inter // 16, 16, self.width), u.view(self.inter // 16, 16, self.width)], dim=1)
+            self.w_gate_up = gu.reshape(2 * self.inter, self.width).contiguous()
+        else:
+            self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = get("down_proj.weight").to(device).contiguous()
 
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        return linear_delta(ops.swiglu(linear(x, self.w_gate_up)), self.w_down)
+        h = None
+        if self.block and x.dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            h = gemm_bf16.try_linear_swiglu(x, self.w_gate_up)
+        if h is None:
+            h = ops.swiglu(linear(x, self.w_gate_up), block=self.block)
+        return linear_delta(h, self.w_down)
 
 
 register_feed_forward("swiglu", SwiGLU)

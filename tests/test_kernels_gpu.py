@@ -321,3 +321,35 @@ def test_rope_cache_write(dtype):
     assert torch.count_nonzero(d_kc[3:7]) == 0 and torch.count_nonzero(d_vc[3:7]) == 0
     # position 0 is the identity
     assert torch.allclose(got[0, :nh], x[0, :nh], atol=tol)
+
+
+def interleave16(g, u):
+    """Rows of gate and up in blocks of 16: 16 gate rows, then the 16 up rows of the same outputs."""
+    i, w = g.shape
+    return torch.stack([g.view(i // 16, 16, w), u.view(i // 16, 16, w)], dim=1).reshape(2 * i, w).contiguous()
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_swiglu_interleaved_layout(dt):
+    from atoma_infer_amd.kernels import ops
+    inter = 48
+    g, u = rnd(5, inter, dtype=dt, seed=1, scale=2.0), rnd(5, inter, dtype=dt, seed=2, scale=2.0)
+    gu = interleave16(g.t().contiguous(), u.t().contiguous()).t().contiguous()      # columns interleaved
+    out = ops.swiglu(gu, block=16)
+    want = torch.nn.functional.silu(g.float()) * u.float()
+    tol = 1e-6 if dt is torch.float32 else 2e-2
+    assert torch.allclose(out.float(), want, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("m", [1, 8, 17, 32])
+@pytest.mark.parametrize("inter,k", [(16, 32), (160, 64), (8192, 2048), (1024, 96)])
+def test_gemm_with_swiglu_epilogue(m, inter, k):
+    from atoma_infer_amd.kernels import gemm_bf16
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    wg, wu = rnd(inter, k, dtype=torch.bfloat16, seed=2, scale=0.1), rnd(inter, k, dtype=torch.bfloat16, seed=3, scale=0.1)
+    out = gemm_bf16.try_linear_swiglu(x, interleave16(wg, wu))
+    assert out is not None and tuple(out.shape) == (m, inter)
+    g, u = x.double().cpu() @ wg.double().cpu().T, x.double().cpu() @ wu.double().cpu().T
+    want = torch.nn.functional.silu(g) * u
+    assert (out.double().cpu() - want).abs().max() <= 1e-2 * want.abs().max()
+    assert gemm_bf16.try_linear_swiglu(rnd(40, k, dtype=torch.bfloat16), interleave16(wg, wu)) is None   # too many rows
