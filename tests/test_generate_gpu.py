@@ -242,3 +242,95 @@ def test_trace_run_program(model_dirs, tmp_path, dtype):
             assert rel_err(got, ref) < TOL_F32
         else:
             assert frob_err(got, ref) < TOL_BF16
+
+
+# ----------------------------------------------------------------------------------------------------------
+# the engine runs one step ahead of the sampled tokens
+
+
+def test_running_ahead_changes_no_token(model_dirs):
+    """EOS is seen one step late and the token sampled meanwhile is dropped; a repeat penalty makes the engine
+    read tokens at once.  Either way the tokens are those of the plain model."""
+    from atoma_infer_amd.sampling import GenerateParameters
+    d = model_dirs["B"]
+    w, cfg = plain_weights(d), plain_config(d)
+    prompts = [random_tokens(9, 1000, 11), random_tokens(4, 1000, 12), random_tokens(15, 1000, 13)]
+    free = [plain_llama.greedy_generate(p, 12, w, cfg) for p in prompts]
+    eng = engine(d, "float32", 16, 16)
+    eng.eos_ids = {free[0][5], free[2][2]}
+    outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=12))
+    for o, f in zip(outs, free):
+        cut = next((i for i, t in enumerate(f) if t in eng.eos_ids), None)
+        want = f if cut is None else f[:cut + 1]
+        assert o.inference_outputs[0].token_ids == want
+        assert o.inference_outputs[0].finish_reason == ("length_capped" if cut is None else "stopped")
+    assert eng.runner.manager.num_requests() == 0 and eng.runner.manager.num_free_pages() == 16
+    assert not eng.has_unfinished()
+    # with a repeat penalty: greedy over penalised logits, token by token, as the plain functions give it
+    eng2 = engine(d, "float32", 16, 16)
+    params = GenerateParameters(do_sample=False, max_new_tokens=8, repetition_penalty=1.3, repeat_last_n=6,
+                                ignore_eos_token=True)
+    got = eng2.generate(prompts[:2], params)
+    for p, o in zip(prompts, got):
+        seq = list(p)
+        for tok in o.inference_outputs[0].token_ids:
+            logits = plain_llama.repeat_penalty(plain_llama.forward(seq, w, cfg)[-1], 1.3, seq[-6:])
+            top2 = torch.topk(logits, 2).values
+            if float(top2[0] - top2[1]) > 1e-4:       # a near tie may fall either way in float32
+                assert tok == int(torch.argmax(logits))
+            seq.append(tok)
+    # step by step from outside: outputs arrive when requests finish, and drain() leaves nothing in flight
+    eng3 = engine(d, "float32", 16, 16)
+    rid = eng3.add_request(prompts[1], GenerateParameters(do_sample=False, max_new_tokens=3, ignore_eos_token=True))
+    seen = []
+    for _ in range(10):
+        seen += eng3.step()
+        if not eng3.has_unfinished():
+            break
+    assert [o.request_id for o in seen] == [rid] and seen[0].inference_outputs[0].token_ids == free[1][:3]
+    assert eng3.drain() == []
+
+
+def test_command_line_generates(model_dirs, tmp_path):
+    d = model_dirs["A"]
+    w, cfg = plain_weights(d), plain_config(d)
+    prompt = random_tokens(7, 512, 5)
+    want = plain_llama.greedy_generate(prompt, 5, w, cfg)
+    toml = tmp_path / "engine.toml"
+    toml.write_text(f'''
+[inference]
+model_name = "{d}"
+dtype = "f32"
+device_ids = [0]
+[cache]
+block_size = 4
+num_gpu_blocks_override = 16
+[scheduler]
+max_num_batched_tokens = 32
+max_num_sequences = 4
+max_model_len = 64
+enable_chunked_prefill = true
+[validation]
+max_input_length = 32
+max_total_tokens = 64
+''')
+    reqs = tmp_path / "requests.jsonl"
+    reqs.write_text(json.dumps({"request_id": "one", "inputs": prompt,
+                                "parameters": {"do_sample": False, "max_new_tokens": 5, "ignore_eos_token": True}}) + "\n")
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    proc = subprocess.run([sys.executable, "-m", "atoma_infer_amd", "generate", "--config-path", str(toml),
+                           "--requests", str(reqs)], capture_output=True, text=True, env=env, timeout=300, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert out["request_id"] == "one" and out["is_finished"]
+    assert out["inference_outputs"][0]["token_ids"] == want
+    assert out["inference_outputs"][0]["finish_reason"] == "length_capped"
+    # the same through flags instead of files
+    proc = subprocess.run([sys.executable, "-m", "atoma_infer_amd", "generate", "--model", d, "--dtype", "f32",
+                           "--block-size", "4", "--num-gpu-blocks-override", "16", "--max-model-len", "64",
+                           "--max-num-batched-tokens", "64", "--max-num-sequences", "4", "--greedy",
+                           "--max-new-tokens", "5", "--ignore-eos-token", "--prompt-ids",
+                           ",".join(str(t) for t in prompt)], capture_output=True, text=True, env=env, timeout=300,
+                          cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert json.loads(proc.stdout.strip().splitlines()[-1])["inference_outputs"][0]["token_ids"] == want
