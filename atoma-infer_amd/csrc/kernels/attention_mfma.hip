@@ -61,6 +61,10 @@ __device__ __forceinline__ bf16x8 pack8(const float* v) {
   return r;
 }
 
+// DEPTH blocks of keys and values are in flight per wave.  Measured on MI355X, more than one gains nothing at any
+// batch size (a decode step of few requests is bound by the start of the kernel and of the memory system, one of
+// many requests by bandwidth) and costs registers, so one is what is launched.
+template <int DEPTH>
 __global__ void __launch_bounds__(256)
 attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
                       const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
@@ -75,6 +79,10 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const int kvh = blockIdx.y;
   const int g = nh / nkv;
   const int c = lane & 31, hg = lane >> 5;
+  // the same in every lane; saying so keeps loop control and page arithmetic in scalar registers
+  const int k_begin = __builtin_amdgcn_readfirstlane(task.k_begin);
+  const int k_end = __builtin_amdgcn_readfirstlane(task.k_end);
+  const int entry = __builtin_amdgcn_readfirstlane(task.entry);
 
   // this lane's row
   const int r = task.row0 + c;
@@ -84,6 +92,17 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const int p_row = row_ok ? task.pos0 + tok : -1;
   const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
   const int head = kvh * g + (row_ok ? hq : 0);
+
+  // page numbers of the task's keys: lane i holds the page of block first_block + i, fetched by one load for 64
+  // blocks (1024 keys) at a time, so that no load of keys waits for a load of its page number
+  const int32_t* table = block_tables + (size_t)entry * max_blocks;
+  int first_block = k_begin / PAGE;
+  auto fetch_pages = [&](int base) {
+    int b = base + lane;
+    if (b > max_blocks - 1) b = max_blocks - 1;
+    return table[b];
+  };
+  int my_page = fetch_pages(first_block);
 
   // Q fragments: B operand, lane (row c, k half hg) holds 8 consecutive d per step
   bf16x8 qf[KSTEPS];
@@ -102,7 +121,6 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     lo_hi = max(lo_hi, __shfl_xor(lo_hi, off, 64));
   }
 
-  const int32_t* table = block_tables + (size_t)task.entry * max_blocks;
   const float sc2 = scale * kLog2e;
   float m = -INFINITY, l = 0.f;
   f32x16 o[DTILES];
@@ -114,15 +132,16 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const size_t kv_head_stride = (size_t)PAGE * HD;            // one (page, head) tile
   const size_t page_stride = (size_t)nkv * kv_head_stride;
 
-  // keys and values of a block are fetched one block ahead (while the previous block's softmax runs) when
-  // registers allow
-  constexpr bool PREFETCH = HD <= 128;
+  // the two pages of the block of 32 keys at kb (a multiple of 32, asked for in rising order)
   auto pages_of = [&](int kb, int& p0, int& p1) {
-    int b0 = kb / PAGE, b1 = b0 + 1;
-    if (b0 > max_blocks - 1) b0 = max_blocks - 1;
-    if (b1 > max_blocks - 1) b1 = max_blocks - 1;
-    p0 = table[b0];
-    p1 = table[b1];
+    int b0 = kb / PAGE - first_block;
+    if (b0 >= 64) {
+      first_block += 64;
+      my_page = fetch_pages(first_block);
+      b0 -= 64;
+    }
+    p0 = __builtin_amdgcn_readlane(my_page, b0);
+    p1 = __builtin_amdgcn_readlane(my_page, b0 + 1);
   };
   auto load_keys = [&](int p0, int p1, bf16x8* kf) {
     const int pg = (c < 16) ? p0 : p1;
@@ -154,116 +173,104 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       }
     }
   };
-  // Two blocks are always in flight: (kf, vf) hold the block being worked on, (kn, vn) the next one, and the
-  // loads of the one after that are issued as soon as (kn, vn) have moved up.
-  constexpr bool DEEP = false;      // measured on MI355X: the second buffer costs occupancy and gains nothing
-  int pg0 = 0, pg1 = 0;
-  bf16x8 kf[KSTEPS], kn[DEEP ? KSTEPS : 1];
-  bf16x8 vf[2][DTILES], vn[2][DTILES];
-  if (task.k_begin < task.k_end) {
-    pages_of(task.k_begin, pg0, pg1);
-    load_keys(pg0, pg1, kf);
-    load_vals(pg0, pg1, vf);
-    if (DEEP && task.k_begin + 32 < task.k_end) {
-      pages_of(task.k_begin + 32, pg0, pg1);
-      load_keys(pg0, pg1, kn);
-      load_vals(pg0, pg1, vn);
-    }
+
+  // With one block in flight, the next block's loads are issued right after S^T (the values move aside first)
+  // when registers allow; with more, buffer j is refilled for block + DEPTH once block's products are issued.
+  constexpr bool EARLY = DEPTH == 1 && HD <= 128;
+  bf16x8 kf[DEPTH][KSTEPS];
+  bf16x8 vf[DEPTH][2][DTILES];
+  {
+    int p0, p1;
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j)
+      if (k_begin + 32 * j < k_end) {
+        pages_of(k_begin + 32 * j, p0, p1);
+        load_keys(p0, p1, kf[j]);
+        load_vals(p0, p1, vf[j]);
+      }
   }
 
-  for (int kb = task.k_begin; kb < task.k_end; kb += 32) {
-    // S^T = K Q^T
-    f32x16 s;
+  for (int kb0 = k_begin; kb0 < k_end; kb0 += 32 * DEPTH) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    for (int j = 0; j < DEPTH; ++j) {
+      const int kb = kb0 + 32 * j;
+      if (kb >= k_end) break;
+      // S^T = K Q^T
+      f32x16 s;
 #pragma unroll
-    for (int st = 0; st < KSTEPS; ++st) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[st], s, 0, 0, 0);
-    const bool has_next = kb + 32 < task.k_end;
-    bf16x8 vc[2][DTILES];
-    if (DEEP) {
-      // this block's values move aside, the next block moves up, the block after it is requested
+      for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int st = 0; st < KSTEPS; ++st) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[j][st], qf[st], s, 0, 0, 0);
+      const int kb_next = kb + 32 * DEPTH;
+      bf16x8 vc[2][DTILES];
 #pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt) {
-          vc[j][dt] = vf[j][dt];
-          vf[j][dt] = vn[j][dt];
-        }
+      for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-      for (int st = 0; st < KSTEPS; ++st) kf[st] = kn[st];
-      if (kb + 64 < task.k_end) {
-        pages_of(kb + 64, pg0, pg1);
-        load_keys(pg0, pg1, kn);
-        load_vals(pg0, pg1, vn);
+        for (int dt = 0; dt < DTILES; ++dt) vc[jj][dt] = vf[j][jj][dt];
+      if (EARLY && kb_next < k_end) {
+        int p0, p1;
+        pages_of(kb_next, p0, p1);
+        load_keys(p0, p1, kf[j]);
+        load_vals(p0, p1, vf[j]);
       }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt) vc[j][dt] = vf[j][dt];
-      if (has_next) {
-        pages_of(kb + 32, pg0, pg1);
-        if (PREFETCH) {
-          load_keys(pg0, pg1, kf);
-          load_vals(pg0, pg1, vf);
-        }
-      }
-    }
 
-    // Online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4.  The running maximum is kept in
-    // units of the scaled score (score * scale * log2 e), so one fused multiply-add feeds exp2.  Only blocks
-    // that touch a row's own position, the window's edge or the end of the key range need the mask.
-    const bool edge = kb + 31 > p_lo || kb < lo_hi || kb + 32 > task.k_end;
-    float sv[16];
-    float bmax = -INFINITY;
-    if (edge) {
+      // Online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4.  The running maximum is kept in
+      // units of the scaled score (score * scale * log2 e), so one fused multiply-add feeds exp2.  Only blocks
+      // that touch a row's own position, the window's edge or the end of the key range need the mask.
+      const bool edge = kb + 31 > p_lo || kb < lo_hi || kb + 32 > k_end;
+      float sv[16];
+      float bmax = -INFINITY;
+      if (edge) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
+          const bool ok = key <= p_row && key >= lo_row && key < k_end;
+          sv[i] = ok ? s[i] : -INFINITY;
+          bmax = fmaxf(bmax, sv[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          sv[i] = s[i];
+          bmax = fmaxf(bmax, sv[i]);
+        }
+      }
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64)) * sc2;
+      const float m_new = fmaxf(m, bmax);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      float psum = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
-        const bool ok = key <= p_row && key >= lo_row && key < task.k_end;
-        sv[i] = ok ? s[i] : -INFINITY;
-        bmax = fmaxf(bmax, sv[i]);
+        sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
+        psum += sv[i];
       }
-    } else {
+      psum += __shfl_xor(psum, 32, 64);
+      // the accumulators are rescaled only when some row's maximum has grown (a wave-uniform decision)
+      const bool grew = __ballot(m_new > m) != 0;
+      if (grew) {
+        const float corr = __builtin_amdgcn_exp2f(m - m_use);
+        l *= corr;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        sv[i] = s[i];
-        bmax = fmaxf(bmax, sv[i]);
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
+        m = m_new;
       }
-    }
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64)) * sc2;
-    const float m_new = fmaxf(m, bmax);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
-      psum += sv[i];
-    }
-    psum += __shfl_xor(psum, 32, 64);
-    // the accumulators are rescaled only when some row's maximum has grown (a wave-uniform decision)
-    const bool grew = __ballot(m_new > m) != 0;
-    if (grew) {
-      const float corr = __builtin_amdgcn_exp2f(m - m_use);
-      l *= corr;
-#pragma unroll
-      for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
-      m = m_new;
-    }
-    l += psum;
+      l += psum;
 
-    // O^T += V^T P^T
-    const bf16x8 p0 = pack8(sv), p1 = pack8(sv + 8);
+      // O^T += V^T P^T
+      const bf16x8 pf0 = pack8(sv), pf1 = pack8(sv + 8);
 #pragma unroll
-    for (int dt = 0; dt < DTILES; ++dt) {
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[0][dt], p0, o[dt], 0, 0, 0);
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[1][dt], p1, o[dt], 0, 0, 0);
-    }
-    if (!DEEP && !PREFETCH && has_next) {
-      load_keys(pg0, pg1, kf);
-      load_vals(pg0, pg1, vf);
+      for (int dt = 0; dt < DTILES; ++dt) {
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[0][dt], pf0, o[dt], 0, 0, 0);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[1][dt], pf1, o[dt], 0, 0, 0);
+      }
+      if (!EARLY && kb_next < k_end) {
+        int p0, p1;
+        pages_of(kb_next, p0, p1);
+        load_keys(p0, p1, kf[j]);
+        load_vals(p0, p1, vf[j]);
+      }
     }
   }
 
@@ -287,13 +294,14 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
         }
       }
   } else {
+    // rows that are not live are never read by the combine kernel (their log-sum-exp is, and says -inf)
     float* po = part_o + (((size_t)task.dest * nkv + kvh) * 32 + c) * HD;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         const int d = dt * 32 + q4 * 8 + hg * 4;
-        if (HD % 32 == 0 || d < HD) {
+        if (row_ok && (HD % 32 == 0 || d < HD)) {
           float4 v = make_float4(o[dt][q4 * 4 + 0] * inv, o[dt][q4 * 4 + 1] * inv, o[dt][q4 * 4 + 2] * inv,
                                  o[dt][q4 * 4 + 3] * inv);
           *reinterpret_cast<float4*>(po + d) = v;
@@ -402,9 +410,9 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
       ((uintptr_t)q & 15) || ((uintptr_t)out & 7))
     return ATOMA_ERR_SHAPE;
   const Task* t = reinterpret_cast<const Task*>(tasks);
-  hipLaunchKernelGGL(attention_mfma_kernel, dim3((n_tasks + 3) / 4, nkv), dim3(256), 0, stream, (const uint16_t*)q,
-                     q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride, part_o,
-                     part_lse, t, n_tasks, block_tables, max_blocks, scale, window, nh, nkv);
+  hipLaunchKernelGGL(attention_mfma_kernel<1>, dim3((n_tasks + 3) / 4, nkv), dim3(256), 0, stream,
+                     (const uint16_t*)q, q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out,
+                     out_stride, part_o, part_lse, t, n_tasks, block_tables, max_blocks, scale, window, nh, nkv);
   ATOMA_LAUNCH_CHECK();
   if (n_combine > 0) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(n_combine, nkv), dim3(256), 0, stream, part_o, part_lse,
