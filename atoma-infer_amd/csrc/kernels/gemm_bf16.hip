@@ -11,17 +11,6 @@
 // C[slice][M][N] and the consumer adds the planes (the fused residual-add + RMSNorm kernel does).
 // Each output's sum order depends only on (K, WK, slices), never on M or on the row's place in the batch.
 //
-//
-// Fused around the product, to spare decode steps whole kernels:
-//  * NORM: the activations are rows of the float32 residual stream and the product is that of their RMSNorm.
-//    Since norm(x)[k] = x[k] * g[k] * rsqrt(mean(x^2) + eps) and the last factor is one number per row, the MFMA
-//    operand is bfloat16(x[k] * g[k]), the sum of x^2 is gathered from the same loads, and the accumulators are
-//    scaled by the row's factor at the end (the reference's norm: models/src/llama.rs:226-241 through candle's
-//    rms_norm; statistics in float32).  Rows may be picked through an index (the final norm of the wanted rows).
-//  * SWIGLU: SiLU(gate) * up on pairs of tiles (see the epilogue).
-//  * ACCUM: C is the float32 residual stream and the product is added to it (one slice only, so that every
-//    element has one owner and a fixed order of sums).
-//
 // Needs K % (32 * WK * slices) == 0 and 16-byte aligned rows; the host wrapper checks and otherwise refuses.
 #include "common.h"
 
@@ -30,27 +19,10 @@ using namespace atoma;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-__device__ __forceinline__ bf16x8 scaled_fragment(const f32x4& x0, const f32x4& x1, const f32x4& g0, const f32x4& g1,
-                                                  float& ssq) {
-  bf16x8 r;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    r[i] = (__bf16)(x0[i] * g0[i]);
-    r[4 + i] = (__bf16)(x1[i] * g1[i]);
-    ssq += x0[i] * x0[i];
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) ssq += x1[i] * x1[i];
-  return r;
-}
-
-template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false, bool NORM = false, bool ACCUM = false>
+template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false>
 __global__ void __launch_bounds__(64 * WN * WK)
-gemm_skinny_kernel(const void* __restrict__ a_, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
-                   int K, int lda, int ldw, int ldc, size_t plane, const float* __restrict__ gain,
-                   const int32_t* __restrict__ rows, float eps) {
-  static_assert(!ACCUM || sizeof(TC) == 4, "the residual stream is float32");
-  const uint16_t* a = reinterpret_cast<const uint16_t*>(a_);
+gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
+                   int K, int lda, int ldw, int ldc, size_t plane) {
   // loads of U steps of K are issued together before their MFMAs, so that a wave keeps U * (RT + MT) 16-byte
   // loads per lane in flight: the product is bound by memory latency and bandwidth, not by arithmetic
   constexpr int U = (RT + MT <= 2) ? 4 : (RT + MT <= 5) ? 2 : 1;
@@ -71,19 +43,11 @@ gemm_skinny_kernel(const void* __restrict__ a_, const uint16_t* __restrict__ w, 
     wp[r] = w + (size_t)n * ldw + k_begin + kg * 8;
   }
   const uint16_t* ap[MT];
-  const float* xp[MT];   // NORM: the row of the residual stream
-  const float* gp = NORM ? gain + k_begin + kg * 8 : nullptr;
-  float ssq[MT];
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
     int row = m * 16 + r16;
     if (row > M - 1) row = M - 1;
     ap[m] = a + (size_t)row * lda + k_begin + kg * 8;
-    if constexpr (NORM) {
-      const int src = rows ? rows[row] : row;
-      xp[m] = reinterpret_cast<const float*>(a_) + (size_t)src * lda + k_begin + kg * 8;
-    }
-    ssq[m] = 0.f;
   }
 
   f32x4 acc[RT][MT];
@@ -93,41 +57,24 @@ gemm_skinny_kernel(const void* __restrict__ a_, const uint16_t* __restrict__ w, 
     for (int m = 0; m < MT; ++m) acc[r][m] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // two buffers of U steps each: while the MFMAs of one run, the loads of the other are in flight
-  bf16x8 wf[2][U][RT], af[2][U][NORM ? 1 : MT];
-  f32x4 xf[2][U][NORM ? MT : 1][2], gf[2][U][2];
+  bf16x8 wf[2][U][RT], af[2][U][MT];
   auto load = [&](int buf, int k0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int r = 0; r < RT; ++r) wf[buf][u][r] = *reinterpret_cast<const bf16x8*>(wp[r] + k0 + u * 32);
-      if constexpr (NORM) {
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-          xf[buf][u][m][0] = *reinterpret_cast<const f32x4*>(xp[m] + k0 + u * 32);
-          xf[buf][u][m][1] = *reinterpret_cast<const f32x4*>(xp[m] + k0 + u * 32 + 4);
-        }
-        gf[buf][u][0] = *reinterpret_cast<const f32x4*>(gp + k0 + u * 32);
-        gf[buf][u][1] = *reinterpret_cast<const f32x4*>(gp + k0 + u * 32 + 4);
-      } else {
-#pragma unroll
-        for (int m = 0; m < MT; ++m) af[buf][u][m] = *reinterpret_cast<const bf16x8*>(ap[m] + k0 + u * 32);
-      }
+      for (int m = 0; m < MT; ++m) af[buf][u][m] = *reinterpret_cast<const bf16x8*>(ap[m] + k0 + u * 32);
     }
   };
   auto multiply = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        bf16x8 frag;
-        if constexpr (NORM)
-          frag = scaled_fragment(xf[buf][u][m][0], xf[buf][u][m][1], gf[buf][u][0], gf[buf][u][1], ssq[m]);
-        else
-          frag = af[buf][u][m];
+      for (int r = 0; r < RT; ++r)
 #pragma unroll
-        for (int r = 0; r < RT; ++r)
-          acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[buf][u][r], frag, acc[r][m], 0, 0, 0);
-      }
+        for (int m = 0; m < MT; ++m)
+          acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[buf][u][r], af[buf][u][m], acc[r][m], 0, 0, 0);
   };
   constexpr int STEP = 32 * U;
   const int n_batches = k_len / STEP;
@@ -149,14 +96,7 @@ gemm_skinny_kernel(const void* __restrict__ a_, const uint16_t* __restrict__ w, 
 #pragma unroll
     for (int r = 0; r < RT; ++r) wt[r] = *reinterpret_cast<const bf16x8*>(wp[r] + k);
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-      if constexpr (NORM)
-        at[m] = scaled_fragment(*reinterpret_cast<const f32x4*>(xp[m] + k), *reinterpret_cast<const f32x4*>(xp[m] + k + 4),
-                                *reinterpret_cast<const f32x4*>(gp + k), *reinterpret_cast<const f32x4*>(gp + k + 4),
-                                ssq[m]);
-      else
-        at[m] = *reinterpret_cast<const bf16x8*>(ap[m] + k);
-    }
+    for (int m = 0; m < MT; ++m) at[m] = *reinterpret_cast<const bf16x8*>(ap[m] + k);
 #pragma unroll
     for (int r = 0; r < RT; ++r)
 #pragma unroll
@@ -164,26 +104,11 @@ gemm_skinny_kernel(const void* __restrict__ a_, const uint16_t* __restrict__ w, 
         acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt[r], at[m], acc[r][m], 0, 0, 0);
   }
 
-  if constexpr (NORM) {
-    // the four lanes that share a row hold the sums of their own k; afterwards each holds the wave's sum
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-      ssq[m] += __shfl_xor(ssq[m], 16, 64);
-      ssq[m] += __shfl_xor(ssq[m], 32, 64);
-    }
-  }
-
   if constexpr (WK > 1) {
     // add the WK partial accumulators of the same rows: waves wk > 0 write, wave wk == 0 sums in fixed order
     __shared__ float red[(WK - 1) * WN * RT * MT * 4 * 64];
-    __shared__ float red_ssq[NORM ? (WK - 1) * WN * MT * 16 : 1];
     constexpr int per_wave = RT * MT * 4 * 64;
     if (wk > 0) {
-      if constexpr (NORM) {
-        if (kg == 0)
-#pragma unroll
-          for (int m = 0; m < MT; ++m) red_ssq[(((wk - 1) * WN + wn) * MT + m) * 16 + r16] = ssq[m];
-      }
       float* dst = red + ((wk - 1) * WN + wn) * per_wave;
 #pragma unroll
       for (int r = 0; r < RT; ++r)
@@ -203,22 +128,6 @@ gemm_skinny_kernel(const void* __restrict__ a_, const uint16_t* __restrict__ w, 
         for (int m = 0; m < MT; ++m)
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[r][m][i] += src[((r * MT + m) * 4 + i) * 64 + lane];
-      if constexpr (NORM) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m) ssq[m] += red_ssq[((s * WN + wn) * MT + m) * 16 + r16];
-      }
-    }
-  }
-
-  if constexpr (NORM) {
-    // every accumulator of a lane belongs to activation row m * 16 + r16
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-      const float inv = 1.0f / sqrtf(ssq[m] / (float)K + eps);
-#pragma unroll
-      for (int r = 0; r < RT; ++r)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[r][m][i] *= inv;
     }
   }
 
@@ -260,10 +169,7 @@ gemm_skinny_kernel(const void* __restrict__ a_, const uint16_t* __restrict__ w, 
       if (row >= M) continue;
       TC* dst = cp + (size_t)row * ldc + n0;
       if (n0 + 3 < N && (ldc & 3) == 0) {
-        if constexpr (ACCUM) {
-          const f32x4 old = *reinterpret_cast<const f32x4*>(dst);
-          *reinterpret_cast<f32x4*>(dst) = old + acc[r][m];
-        } else if (sizeof(TC) == 4) {
+        if (sizeof(TC) == 4) {
           *reinterpret_cast<f32x4*>(dst) = acc[r][m];
         } else {
           uint2 v;
@@ -274,10 +180,7 @@ gemm_skinny_kernel(const void* __restrict__ a_, const uint16_t* __restrict__ w, 
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (n0 + i < N) {
-            if constexpr (ACCUM) dst[i] = from_f32<TC>(to_f32(dst[i]) + acc[r][m][i]);
-            else dst[i] = from_f32<TC>(acc[r][m][i]);
-          }
+          if (n0 + i < N) dst[i] = from_f32<TC>(acc[r][m][i]);
       }
     }
   }
@@ -289,13 +192,11 @@ static int launch(const void* a, const void* w, void* c, int c_dtype, int M, int
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), slices), block(64 * WN * WK);
   const size_t plane = (size_t)M * ldc;
   if (c_dtype == kF32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, float>), grid, block, 0, stream, (const void*)a,
-                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane, (const float*)nullptr,
-                       (const int32_t*)nullptr, 0.f);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, float>), grid, block, 0, stream, (const uint16_t*)a,
+                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane);
   else if (c_dtype == kBF16)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t>), grid, block, 0, stream, (const void*)a,
-                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane, (const float*)nullptr,
-                       (const int32_t*)nullptr, 0.f);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t>), grid, block, 0, stream, (const uint16_t*)a,
+                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();
@@ -340,9 +241,8 @@ template <int MT, int RT, int WN, int WK>
 static int launch_swiglu(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
                          hipStream_t stream) {
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, true>), grid, block, 0, stream, (const void*)a,
-                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, (const float*)nullptr,
-                     (const int32_t*)nullptr, 0.f);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, true>), grid, block, 0, stream, (const uint16_t*)a,
+                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
@@ -370,75 +270,5 @@ extern "C" int atoma_gemm_bf16_skinny_swiglu(const void* a, const void* w, void*
     case 2: return launch_swiglu_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
     case 3: return launch_swiglu_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
     default: return launch_swiglu_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
-  }
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// fused forms: RMSNorm of float32 residual rows on the way in, SiLU-multiply or accumulation on the way out
-
-enum { kModeSwiglu = 1, kModeNorm = 2, kModeAccum = 4 };
-
-template <int MT, int RT, int WN, int WK, typename TC, bool SW, bool NO, bool AC>
-static int launch_fused(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
-                        const float* gain, const int32_t* rows, float eps, hipStream_t stream) {
-  dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, TC, SW, NO, AC>), grid, block, 0, stream, a,
-                     (const uint16_t*)w, (TC*)c, M, N, K, lda, ldw, ldc, (size_t)0, gain, rows, eps);
-  ATOMA_LAUNCH_CHECK();
-  return 0;
-}
-
-template <int MT>
-static int launch_fused_mt(const void* a, const void* w, void* c, int c_dtype, int mode, int M, int N, int K, int lda,
-                           int ldw, int ldc, int rt, int wk, const float* gain, const int32_t* rows, float eps,
-                           hipStream_t stream) {
-#define ATOMA_FUSED(R, WN_, WK_, TC, SW, NO, AC)                                                       \
-  if (rt == R && wk == WK_)                                                                            \
-    return launch_fused<MT, R, WN_, WK_, TC, SW, NO, AC>(a, w, c, M, N, K, lda, ldw, ldc, gain, rows, eps, stream)
-  if (mode == kModeNorm && c_dtype == kBF16) {
-    ATOMA_FUSED(1, 1, 4, bf16_t, false, true, false);
-    ATOMA_FUSED(2, 1, 4, bf16_t, false, true, false);
-    ATOMA_FUSED(1, 1, 8, bf16_t, false, true, false);
-    ATOMA_FUSED(2, 1, 8, bf16_t, false, true, false);
-  } else if (mode == kModeNorm && c_dtype == kF32) {
-    ATOMA_FUSED(1, 1, 4, float, false, true, false);
-    ATOMA_FUSED(2, 1, 4, float, false, true, false);
-    ATOMA_FUSED(1, 1, 8, float, false, true, false);
-    ATOMA_FUSED(2, 1, 8, float, false, true, false);
-  } else if (mode == (kModeNorm | kModeSwiglu) && c_dtype == kBF16) {
-    ATOMA_FUSED(2, 1, 4, bf16_t, true, true, false);
-    ATOMA_FUSED(2, 1, 8, bf16_t, true, true, false);
-  } else if (mode == kModeAccum && c_dtype == kF32) {
-    ATOMA_FUSED(1, 1, 4, float, false, false, true);
-    ATOMA_FUSED(2, 1, 4, float, false, false, true);
-    ATOMA_FUSED(1, 1, 8, float, false, false, true);
-    ATOMA_FUSED(2, 1, 8, float, false, false, true);
-    ATOMA_FUSED(1, 1, 16, float, false, false, true);
-  }
-#undef ATOMA_FUSED
-  return ATOMA_ERR_SHAPE;
-}
-
-// mode: bit 0 SiLU-multiply epilogue (w interleaved as for atoma_gemm_bf16_skinny_swiglu, c [M, N / 2] bfloat16),
-// bit 1 RMSNorm on the way in (a is float32 [*, lda], gain float32 [K], rows an optional index of M source rows),
-// bit 2 add into c (float32).  M <= 32 with the norm (every group of waves reads the float32 rows), else <= 64.
-extern "C" int atoma_gemm_bf16_skinny_fused(const void* a, const void* w, void* c, int c_dtype, int mode, int M, int N,
-                                            int K, int lda, int ldw, int ldc, int rt, int wk, const float* gain,
-                                            const int32_t* rows, float eps, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  const bool norm = mode & kModeNorm, swiglu = mode & kModeSwiglu;
-  if (M > (norm ? 32 : 64) || K <= 0 || wk <= 0 || K % (32 * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K ||
-      ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || (norm && (gain == nullptr || ((uintptr_t)gain & 15))))
-    return ATOMA_ERR_SHAPE;
-  if (swiglu ? ((N & 31) || ldc < N / 2 || (ldc & 3) || ((uintptr_t)c & 7)) : (ldc < N)) return ATOMA_ERR_SHAPE;
-  switch ((M + 15) / 16) {
-    case 1: return launch_fused_mt<1>(a, w, c, c_dtype, mode, M, N, K, lda, ldw, ldc, rt, wk, gain, rows, eps, stream);
-    case 2: return launch_fused_mt<2>(a, w, c, c_dtype, mode, M, N, K, lda, ldw, ldc, rt, wk, gain, rows, eps, stream);
-    case 3:
-      if (norm) return ATOMA_ERR_SHAPE;
-      return launch_fused_mt<3>(a, w, c, c_dtype, mode, M, N, K, lda, ldw, ldc, rt, wk, gain, rows, eps, stream);
-    default:
-      if (norm) return ATOMA_ERR_SHAPE;
-      return launch_fused_mt<4>(a, w, c, c_dtype, mode, M, N, K, lda, ldw, ldc, rt, wk, gain, rows, eps, stream);
   }
 }

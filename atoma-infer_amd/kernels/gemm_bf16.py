@@ -136,39 +136,3 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
     _check(lib().atoma_gemm_bf16_skinny_swiglu(_p(x), _p(w), _p(out), m, n, k, x.stride(0) if m > 1 else k,
                                                w.stride(0), n // 2, rt, wk, _stream()), "gemm_bf16_skinny_swiglu")
     return out
-
-
-MODE_SWIGLU, MODE_NORM, MODE_ACCUM = 1, 2, 4
-NORM_MAX_M = 32
-
-
-def skinny_fused(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, mode: int, rt: int, wk: int,
-                 gain: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None, eps: float = 0.0) -> None:
-    """The streaming product with work fused around it (csrc/kernels/gemm_bf16.hip says what each mode does).
-
-    With MODE_NORM ``a`` is the float32 residual stream, ``gain`` the norm's float32 weight and ``rows`` an optional
-    int32 index of the rows to take; with MODE_ACCUM ``out`` is the float32 residual stream, added to in place.
-    """
-    n, k = w.shape
-    norm = bool(mode & MODE_NORM)
-    m = int(rows.shape[0]) if rows is not None else a.shape[0]
-    if norm:
-        if a.dtype is not torch.float32 or gain is None or gain.dtype is not torch.float32 or gain.numel() != k:
-            raise KernelError("fused norm: float32 rows and a float32 weight of K numbers are needed")
-        if rows is not None and (rows.dtype is not torch.int32 or not norm):
-            raise KernelError("fused norm: rows must be int32")
-    elif a.dtype is not torch.bfloat16 or rows is not None:
-        raise KernelError("gemm_bf16_skinny_fused: bfloat16 activations, no row index without the norm")
-    if w.dtype is not torch.bfloat16 or a.shape[1] != k or a.stride(1) != 1 or w.stride(1) != 1:
-        raise KernelError("gemm_bf16_skinny_fused: operand shapes do not match")
-    cols = n // 2 if mode & MODE_SWIGLU else n
-    if out.shape[-2] != m or out.shape[-1] != cols or out.stride(-1) != 1:
-        raise KernelError(f"gemm_bf16_skinny_fused: out must be [{m}, {cols}]")
-    if mode & MODE_ACCUM and out.dtype is not torch.float32:
-        raise KernelError("gemm_bf16_skinny_fused: accumulation needs float32")
-    code = {torch.float32: F32, torch.bfloat16: BF16}[out.dtype]
-    lda = a.stride(0) if a.shape[0] > 1 else k
-    _check(lib().atoma_gemm_bf16_skinny_fused(_p(a), _p(w), _p(out), code, mode, m, n, k, lda,
-                                              w.stride(0) if n > 1 else k, out.stride(-2) if m > 1 else cols, rt, wk,
-                                              _p(gain), _p(rows), ctypes.c_float(eps), _stream()),
-           "gemm_bf16_skinny_fused")
