@@ -217,6 +217,10 @@ ATTN_CASES = [
     (2, 1, 256, 16, 0, [(0, 35), (520, 2)]),
     (8, 2, 64, 16, 48, [(0, 130), (600, 1), (1030, 3), (40, 20)]),
     (4, 2, 32, 16, 600, [(0, 100), (900, 1), (640, 5)]),
+    # prompt tiles with so many keys that they are cut along the keys and merged
+    (8, 2, 64, 16, 0, [(0, 1100), (900, 150), (2047, 1)]),
+    (4, 2, 32, 16, 800, [(0, 1300), (1200, 40)]),
+    (4, 1, 128, 16, 0, [(4000, 70)]),
 ]
 
 
