@@ -252,6 +252,64 @@ rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __r
   }
 }
 
+// The same for bfloat16 rows and caches with hd % 16 == 0, the whole head rotated and 16-byte aligned rows: a
+// thread takes eight neighbouring pairs of a q or k head (two 16-byte loads, and since eight columns of a key are
+// one piece of its cache tile, two 16-byte stores) or eight columns of a v head.  One block per token.
+__global__ void __launch_bounds__(256)
+rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const int32_t* __restrict__ positions,
+                            const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                            uint16_t* __restrict__ kcache, uint16_t* __restrict__ vcache,
+                            const int32_t* __restrict__ slot_mapping, int page_size, int nh, int nkv, int hd) {
+  const int t = blockIdx.x;
+  const int half = hd >> 1;
+  const int per_qk = hd >> 4, per_v = hd >> 3;             // items per head
+  const int n_qk = (nh + nkv) * per_qk;
+  const int n_items = n_qk + (kcache ? nkv * per_v : 0);
+  const int slot = (kcache && slot_mapping) ? slot_mapping[t] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+  uint16_t* row = qkv + (size_t)t * row_stride;
+  const size_t pos = (size_t)positions[t];
+  for (int item = threadIdx.x; item < n_items; item += 256) {
+    if (item >= n_qk) {
+      if (slot < 0) continue;
+      const int head = (item - n_qk) / per_v, d0 = ((item - n_qk) % per_v) * 8;
+      const uint4 raw = *reinterpret_cast<const uint4*>(row + (size_t)(nh + nkv + head) * hd + d0);
+      const uint16_t* v = reinterpret_cast<const uint16_t*>(&raw);
+      uint16_t* tile = vcache + ((size_t)page * nkv + head) * hd * page_size;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tile[value_offset(d0 + e, off, hd, page_size)] = v[e];
+      continue;
+    }
+    const int head = item / per_qk, i0 = (item % per_qk) * 8;
+    const bool is_k = head >= nh;
+    if (is_k && (!kcache || slot < 0)) continue;
+    uint16_t* x = row + (size_t)head * hd;
+    const uint4 r1 = *reinterpret_cast<const uint4*>(x + i0), r2 = *reinterpret_cast<const uint4*>(x + i0 + half);
+    const f4 c0 = load4(cos_t + pos * half + i0), c1 = load4(cos_t + pos * half + i0 + 4);
+    const f4 s0 = load4(sin_t + pos * half + i0), s1 = load4(sin_t + pos * half + i0 + 4);
+    const uint16_t* a = reinterpret_cast<const uint16_t*>(&r1);
+    const uint16_t* b = reinterpret_cast<const uint16_t*>(&r2);
+    uint4 w1, w2;
+    uint16_t* o1 = reinterpret_cast<uint16_t*>(&w1);
+    uint16_t* o2 = reinterpret_cast<uint16_t*>(&w2);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float c = e < 4 ? c0.v[e] : c1.v[e - 4], sn = e < 4 ? s0.v[e] : s1.v[e - 4];
+      const float x1 = bf16_bits_to_f32(a[e]), x2 = bf16_bits_to_f32(b[e]);
+      o1[e] = f32_to_bf16_bits(x1 * c - x2 * sn);
+      o2[e] = f32_to_bf16_bits(x2 * c + x1 * sn);
+    }
+    if (is_k) {
+      uint16_t* ktile = kcache + ((size_t)page * nkv + (head - nh)) * page_size * hd;
+      *reinterpret_cast<uint4*>(ktile + key_offset(off, i0, page_size)) = w1;
+      *reinterpret_cast<uint4*>(ktile + key_offset(off, i0 + half, page_size)) = w2;
+    } else {
+      *reinterpret_cast<uint4*>(x + i0) = w1;
+      *reinterpret_cast<uint4*>(x + i0 + half) = w2;
+    }
+  }
+}
+
 extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, const int32_t* positions,
                                       const float* cos_t, const float* sin_t, int rotary_dim, void* kcache,
                                       void* vcache, int cache_dtype, const int32_t* slot_mapping, int page_size,
@@ -264,6 +322,16 @@ extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, 
   const int heads = kcache ? nh + 2 * nkv : nh;
   const int items = heads * (hd / 2);
   if (hd & 1) return ATOMA_ERR_SHAPE;
+  // few tokens (decode steps) are quicker with many small blocks; measured on MI355X
+  if (n_tokens >= 32 && act_dtype == kBF16 && cache_dtype == kBF16 && cos_t && sin_t && rotary_dim == hd && hd % 16 == 0 &&
+      row_stride % 8 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)kcache & 15) == 0 &&
+      ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0) {
+    hipLaunchKernelGGL(rope_cache_write_vec_kernel, dim3(n_tokens), dim3(256), 0, stream, (uint16_t*)qkv, row_stride,
+                       positions, cos_t, sin_t, (uint16_t*)kcache, (uint16_t*)vcache, slot_mapping, page_size, nh,
+                       nkv, hd);
+    ATOMA_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid(n_tokens, (items + 255) / 256), block(256);
 #define ATOMA_ROPE(TA, TC)                                                                                        \
   hipLaunchKernelGGL((rope_cache_write_kernel<TA, TC>), grid, block, 0, stream, (TA*)qkv, row_stride, positions, \

@@ -54,6 +54,64 @@ def chunk_for(n_split: int, max_keys: int) -> int:
     return CHUNK
 
 
+def _live_pieces(rows: int, qt: int, live_tokens: int):
+    """First rows of the 32-row pieces of a tile that hold a live row.  Row r is token r % qt of head r // qt, and
+    the tile's first ``live_tokens`` tokens exist (fewer than qt only in the last tile of an entry)."""
+    if live_tokens >= qt:
+        return list(range(0, rows, 32))
+    out = []
+    for row0 in range(0, rows, 32):
+        n = min(32, rows - row0)
+        first = row0 % qt
+        # rows row0 .. row0 + n - 1 hold tokens first, first + 1, ... modulo qt: live if the run starts below
+        # live_tokens or wraps around to token 0
+        if first < live_tokens or first + n > qt:
+            out.append(row0)
+    return out
+
+
+_NULL_TASK = np.asarray((-1, 0, 1, 0, 0, 0, -1, 0, 0, 0, 0, 0), dtype=np.int32)
+
+
+def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, window: int, qt: int):
+    """The tasks of an entry that is not split along its keys, without a loop over its tiles: (keys per group of
+    four tasks, tasks [groups, 4, 12]).  A tile is ``qt`` tokens times ``group`` heads, cut into pieces of 32 rows;
+    pieces are padded to fours with empty tasks."""
+    rows = qt * group
+    pieces = -(-rows // 32)
+    fours = -(-pieces // 4)
+    tok0 = np.arange(0, count, qt, dtype=np.int64)                           # [tiles]
+    last = np.minimum(tok0 + qt, count)
+    k_end = start + last
+    lo = np.maximum(0, start + tok0 - window + 1) if window > 0 else np.zeros_like(tok0)
+    kb = (lo // 32) * 32
+    tiles = len(tok0)
+    t = np.empty((tiles, fours * 4, 12), dtype=np.int32)
+    t[:] = _NULL_TASK
+    row0 = 32 * np.arange(pieces, dtype=np.int64)
+    live = np.ones((tiles, pieces), dtype=bool)
+    if int(last[-1] - tok0[-1]) < qt:                                        # the short last tile
+        live[-1] = False
+        live[-1, [r // 32 for r in _live_pieces(rows, qt, int(last[-1] - tok0[-1]))]] = True
+    body = t[:, :pieces]
+    vals = np.empty((tiles, pieces, 12), dtype=np.int32)
+    vals[..., 0] = e
+    vals[..., 1] = tok0[:, None]
+    vals[..., 2] = qt
+    vals[..., 3] = row0[None, :]
+    vals[..., 4] = kb[:, None]
+    vals[..., 5] = k_end[:, None]
+    vals[..., 6] = -1
+    vals[..., 7] = 0
+    vals[..., 8] = tok_base
+    vals[..., 9] = count
+    vals[..., 10] = start
+    vals[..., 11] = 0
+    body[live] = vals[live]
+    lengths = np.repeat(k_end - kb, fours)
+    return lengths, t.reshape(tiles * fours, 4, 12)
+
+
 def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket: Optional[int] = None,
                 vectorized: bool = True) -> Tuple[np.ndarray, Tuple[int, int, int]]:
     """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials).
@@ -68,6 +126,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     null = (-1, 0, 1, 0, 0, 0, -1, 0, 0, 0, 0, 0)
     tok_bases = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
     direct, split, combine = [], [], []
+    direct_arrays = []
     n_part = 0
 
     def splits(e):
@@ -85,13 +144,16 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
         rows = qt * group
         do_split = splits(e)
         tail = (int(tok_bases[e]), count, start, 0)
+        if vectorized and not do_split:
+            lengths, groups = _tile_tasks(e, start, count, int(tok_bases[e]), group, window, qt)
+            direct_arrays.append((lengths, groups))
+            continue
         for tok0 in range(0, count, qt):
             last = min(tok0 + qt, count)
             k_end = start + last
             lo = max(0, start + tok0 - window + 1) if window > 0 else 0
             # 32-row pieces of the tile that hold at least one live row (the last tile of an entry may be short)
-            live = [row0 for row0 in range(0, rows, 32)
-                    if any(tok0 + r % qt < count for r in range(row0, min(row0 + 32, rows)))]
+            live = _live_pieces(rows, qt, min(qt, count - tok0))
             if do_split:
                 c_first, c_last = lo // chunk, (k_end - 1) // chunk
                 slots = bucket * (CHUNK // chunk) if bucket is not None else c_last + 1
@@ -109,12 +171,19 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
                 while len(wave_tasks) % 4:
                     wave_tasks.append(null)
                 direct.append((k_end - kb, wave_tasks))
-    direct.sort(key=lambda x: -x[0])
-    main = [t for _, ws in direct for t in ws] + split
-    while len(main) % 4:
-        main.append(null)
-    arr = np.asarray(main + combine, dtype=np.int32).reshape(-1, 12)
-    return arr, (len(main), len(combine), n_part)
+    if direct_arrays:
+        lengths = np.concatenate([l for l, _ in direct_arrays])
+        groups = np.concatenate([g for _, g in direct_arrays])                 # [n, 4, 12]
+        order = np.argsort(-lengths, kind="stable")
+        head = groups[order].reshape(-1, 12)
+    else:
+        direct.sort(key=lambda x: -x[0])
+        head = np.asarray([t for _, ws in direct for t in ws], dtype=np.int32).reshape(-1, 12)
+    while len(split) % 4:
+        split.append(null)
+    rest = np.asarray(split + combine, dtype=np.int32).reshape(-1, 12)
+    arr = np.concatenate([head, rest])
+    return arr, (len(head) + len(split), len(combine), n_part)
 
 
 def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int):

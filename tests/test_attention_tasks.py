@@ -80,3 +80,22 @@ def test_decode_builder_equals_the_general_one(seed):
     other = rng.integers(0, bucket * 256, size=s).astype(np.int32)
     assert A.build_tasks(other, counts, group, window, bucket)[1] == mf or \
         A.chunk_for(s, int(other.max()) + 1) != A.chunk_for(s, int(starts.max()) + 1)
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_tile_builder_equals_the_general_one(seed):
+    """Entries that are not split along their keys are planned without a loop over their tiles; the plain loop
+    gives the same tasks."""
+    rng = np.random.default_rng(500 + seed)
+    s = int(rng.integers(1, 7))
+    group = int(rng.choice([1, 3, 4, 8, 40, 130]))
+    window = int(rng.choice([0, 0, 50, 700]))
+    counts = rng.choice([1, 1, 2, 7, 33, 150, 600], size=s).astype(np.int32)
+    starts = rng.integers(0, 2500, size=s).astype(np.int32)
+    fast, mf = A.build_tasks(starts, counts, group, window)
+    slow, ms = A.build_tasks(starts, counts, group, window, vectorized=False)
+    assert mf[1:] == ms[1:]
+    live = lambda arr, meta: sorted(map(tuple, arr[:meta[0]][arr[:meta[0], 0] >= 0].tolist()))
+    assert live(fast, mf) == live(slow, ms)
+    assert np.array_equal(fast[mf[0]:], slow[ms[0]:])
+    coverage(fast, mf, starts, counts, group, window)

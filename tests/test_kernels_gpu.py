@@ -290,17 +290,20 @@ def test_attention_reference_vectors():
     assert torch.allclose(got[:, 0], v[:, 0], atol=1e-6)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page", [(5, 2, 48, 4), (8, 2, 64, 16), (3, 1, 40, 16), (2, 2, 128, 16)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_rope_cache_write(dtype):
+@pytest.mark.parametrize("t", [9, 45])      # few tokens and many take different kernels in bfloat16
+def test_rope_cache_write(dtype, nh, nkv, hd, page, t):
     from atoma_infer_amd.kernels import ops
-    nh, nkv, hd, page, t = 5, 2, 48, 4, 9
     g = torch.Generator().manual_seed(3)
     qkv = torch.randn(t, (nh + 2 * nkv) * hd, generator=g).to(dtype)
-    pos = torch.tensor([0, 1, 2, 3, 4, 50, 51, 7, 8], dtype=torch.int32)
+    pos = torch.tensor(([0, 1, 2, 3, 4, 50, 51, 7, 8] * 5)[:t], dtype=torch.int32)
     inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))
     ang = torch.arange(64).float()[:, None] * inv[None]
     cos, sin = torch.cos(ang), torch.sin(ang)
-    slots = torch.tensor([8, 9, 10, 11, 0, 1, -1, 30, 31], dtype=torch.int32)
+    # slots in pages 0, 2 and 7 whatever the page size; pages 3..6 must stay untouched
+    slots = torch.tensor([2 * page, 2 * page + 1, 2 * page + 2, 2 * page + 3, 0, 1, -1, 8 * page - 2, 8 * page - 1]
+                         + [-1] * (t - 9), dtype=torch.int32)
     kc = torch.zeros(8, nkv, page, hd, dtype=dtype)
     vc = torch.zeros(8, nkv, hd, page, dtype=dtype)
     from atoma_infer_amd.cache.layout import pack_keys, pack_values, unpack_keys, unpack_values
