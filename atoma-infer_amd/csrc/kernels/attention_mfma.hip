@@ -312,6 +312,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
 }
 
 // Merge partial results: out = sum_s w_s O_s / sum_s w_s with w_s = exp2(lse_s - max lse).
+// A kernel of its own on purpose: letting the last wave to finish a row's chunks merge them needs device-scope
+// fences around a counter, and on this GPU those write back and invalidate the L2 of the wave's XCD, which
+// measured far dearer (a decode step 1.6 times as long) than this second launch.
 // One block per (combine task, KV head).  The log-sum-exps of all parts are first brought into LDS by all
 // threads at once and turned into weights there; then the valid rows of the task (group x tokens, at most 32)
 // times HD output values are spread over the 256 threads, and each adds its parts in order of their index with
