@@ -4,8 +4,8 @@
 
 * the hand-written weight-streaming MFMA kernel when M is small (decode steps, short portions) or when float32
   output is wanted (logits), running it over blocks of 64 rows of x;
-* the library product (hipBLASLt through ``torch.mm``) for large bfloat16-output products, as the reference uses
-  a library for its linears;
+* the library product (hipBLASLt through ``torch.mm``) for products with many rows of x (more than 64; more
+  than 32 on large weights; more than 16 for float32 output), as the reference uses a library for its linears;
 * nothing (None) when the shape fits neither: the caller then runs the float32 FMA kernel.
 """
 from __future__ import annotations
@@ -84,20 +84,46 @@ def skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, slices: int = 1,
            "gemm_bf16_skinny")
 
 
+def _library_wins(m: int, n: int, k: int, out_dtype: torch.dtype) -> bool:
+    """Measured on MI355X at the sizes of Llama-3.2-1B: where the library's tiles beat the streaming kernel.
+
+    The streaming kernel fetches the activations anew for every 16 or 32 rows of the weight, which costs little up
+    to 16 rows of activations and more than the weight itself beyond 32."""
+    if out_dtype is torch.float32:
+        return m > 16 and _MM_OUT_DTYPE
+    if m > SKINNY_MAX_M:
+        return True
+    return m > LIBRARY_MIN_M_WIDE and n * k >= (1 << 24)
+
+
+def _probe_mm_out_dtype() -> bool:
+    """Whether this torch has ``mm(..., out_dtype=float32)`` for bfloat16 operands (float32 accumulation either way)."""
+    import inspect
+    doc = getattr(torch.mm, "__doc__", "") or ""
+    return "out_dtype" in doc
+
+
+_MM_OUT_DTYPE = _probe_mm_out_dtype()
+
+
 def try_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None,
                ) -> Optional[torch.Tensor]:
     """x [M, K] @ w [N, K]^T if a fast kernel takes the shape, else None (the caller falls back to float32 FMAs)."""
     m, n = x.shape[0], w.shape[0]
+    k = x.shape[1]
     ok = skinny_ok(x, w)
-    # measured on MI355X: from 33 rows on, the library's tiles beat the streaming kernel on wide products
-    if ok and out_dtype is torch.bfloat16 and m > LIBRARY_MIN_M_WIDE and n >= 8192:
-        ok = False
-    if ok and (m <= SKINNY_MAX_M or out_dtype is torch.float32):
+    if not (ok and _library_wins(m, n, k, out_dtype)) and ok and (m <= SKINNY_MAX_M or out_dtype is torch.float32):
         if out is None:
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
         for lo in range(0, m, SKINNY_MAX_M):
             hi = min(lo + SKINNY_MAX_M, m)
             skinny(x[lo:hi], w, out[lo:hi])
+        return out
+    if out_dtype is torch.float32 and _MM_OUT_DTYPE and m > 16:
+        y = torch.mm(x, w.t(), out_dtype=torch.float32)
+        if out is None:
+            return y
+        out.copy_(y)
         return out
     if out_dtype is torch.bfloat16 and m > LIBRARY_MIN_M_WIDE:
         if out is None:
@@ -107,10 +133,11 @@ def try_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Op
 
 
 def linear_planes(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
-    """For M <= 64: float32 planes [slices, M, N] whose sum is x @ w^T (K split over the grid), else None."""
+    """For M <= 64: float32 planes [slices, M, N] whose sum is x @ w^T (K split over the grid), else None (also
+    where the library's product is the faster way to the same sum)."""
     m, k = x.shape
     n = w.shape[0]
-    if m > SKINNY_MAX_M or not skinny_ok(x, w):
+    if m > SKINNY_MAX_M or not skinny_ok(x, w) or _library_wins(m, n, k, torch.bfloat16):
         return None
     rt, wk, slices = _plan(m, n, k, True)
     out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)

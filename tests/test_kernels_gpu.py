@@ -107,22 +107,36 @@ def test_gemm_generic(m, n, k, adt, wdt, cdt):
 def test_gemm_bf16_skinny(m, n, k, cdt):
     from atoma_infer_amd.kernels import gemm_bf16
     a, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2)
-    c = gemm_bf16.try_linear(a, w, cdt)
-    assert c is not None and c.dtype is cdt
     want = a.double().cpu() @ w.double().cpu().T
     tol = 1e-5 if cdt is torch.float32 else 1e-2
+    # the kernel itself, with the plan the engine would pick, whole and split along K
+    c = torch.empty((m, n), dtype=cdt, device=DEV)
+    gemm_bf16.skinny(a, w, c)
+    assert (c.double().cpu() - want).abs().max() <= tol * want.abs().max()
+    rt, wk, slices = gemm_bf16._plan(m, n, k, True)
+    planes = torch.empty((slices, m, n), dtype=torch.float32, device=DEV)
+    gemm_bf16.skinny(a, w, planes, slices, rt, wk)
+    assert (planes.sum(0).double().cpu() - want).abs().max() <= 1e-5 * want.abs().max()
+    # the ways in which parts call it: this kernel or the library, whichever is quicker at the shape
+    c = gemm_bf16.try_linear(a, w, cdt)
+    assert c is not None and c.dtype is cdt
     assert (c.double().cpu() - want).abs().max() <= tol * want.abs().max()
     planes = gemm_bf16.linear_planes(a, w)
-    assert planes is not None and planes.dim() == 3
-    assert (planes.sum(0).double().cpu() - want).abs().max() <= 1e-5 * want.abs().max()
+    if gemm_bf16._library_wins(m, n, k, torch.bfloat16):
+        assert planes is None
+    else:
+        assert planes.dim() == 3
+        assert (planes.sum(0).double().cpu() - want).abs().max() <= 1e-5 * want.abs().max()
 
 
 def test_gemm_bf16_rows_do_not_depend_on_the_batch():
     from atoma_infer_amd.kernels import gemm_bf16
     a, w = rnd(64, 512, dtype=torch.bfloat16, seed=1), rnd(300, 512, dtype=torch.bfloat16, seed=2)
-    full = gemm_bf16.try_linear(a, w, torch.float32)
+    full = torch.empty((64, 300), dtype=torch.float32, device=DEV)
+    gemm_bf16.skinny(a, w, full)
     for lo, hi in [(0, 1), (5, 6), (10, 33), (63, 64)]:
-        part = gemm_bf16.try_linear(a[lo:hi], w, torch.float32)
+        part = torch.empty((hi - lo, 300), dtype=torch.float32, device=DEV)
+        gemm_bf16.skinny(a[lo:hi], w, part)
         assert torch.equal(part, full[lo:hi])
 
 
@@ -134,7 +148,12 @@ def test_gemm_bf16_float32_out_for_many_rows():
     assert (c.double().cpu() - want).abs().max() <= 1e-5 * want.abs().max()
     cb = gemm_bf16.try_linear(a, w, torch.bfloat16)   # the library product
     assert (cb.double().cpu() - want).abs().max() <= 1e-2 * want.abs().max()
-    assert gemm_bf16.try_linear(a[:, :40], w[:, :40], torch.float32) is None   # K no multiple of 32: refused
+    # K no multiple of 32: the streaming kernel refuses; few rows then go to the float32 kernel, many to the library
+    assert gemm_bf16.try_linear(a[:8, :40], w[:, :40], torch.float32) is None
+    c = gemm_bf16.try_linear(a[:, :40], w[:, :40], torch.float32)
+    if c is not None:
+        want = a[:, :40].double().cpu() @ w[:, :40].double().cpu().T
+        assert (c.double().cpu() - want).abs().max() <= 1e-5 * want.abs().max()
 
 
 # ----------------------------------------------------------------------------------------------------------
