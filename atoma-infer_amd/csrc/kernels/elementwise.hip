@@ -205,12 +205,15 @@ extern "C" int atoma_add_rmsnorm(float* resid, const void* delta, int delta_dtyp
 // A negative slot, or null caches, skip the cache write (the reference skips negative slots:
 // csrc/kernels/cache_manager.cu:151-155).  cos/sin may be null: then nothing is rotated.
 // Pairing and signs: csrc/kernels/rotary.h:116-131; rotation applies to q and k only: models/src/llama.rs:298-299.
+// With `q_out` ([T, q_stride], the whole head rotated): the rows of the q and k projections were reordered at load
+// time so that the members of pair i arrive as columns 2i and 2i + 1 of the head (which lets the projection's own
+// epilogue rotate, for few rows); the rotated q then goes to q_out and k to the cache in their own column order.
 template <typename TA, typename TC>
 __global__ void __launch_bounds__(256)
 rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __restrict__ positions,
                         const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim,
                         TC* __restrict__ kcache, TC* __restrict__ vcache, const int32_t* __restrict__ slot_mapping,
-                        int page_size, int nh, int nkv, int hd, int heads) {
+                        int page_size, int nh, int nkv, int hd, int heads, TA* __restrict__ q_out, int q_stride) {
   // One thread per item of a token: a rotated pair (or, beyond the rotary dimension, a pair of plain columns)
   // of a q or k head, or two columns of a v head.  `heads` is how many heads of the row are touched.
   const int t = blockIdx.x;
@@ -234,15 +237,18 @@ rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __r
   TC* ktile = is_k ? kcache + ((size_t)page * nkv + (head - nh)) * page_size * hd : nullptr;
   const int half = cos_t ? rotary_dim / 2 : 0;
   if (i < half) {
+    // with q_out, the members of pair i come in as neighbours (2i, 2i + 1) and leave to their own columns
+    const int a = q_out ? 2 * i : i, b = q_out ? 2 * i + 1 : i + half;
     const float c = cos_t[(size_t)positions[t] * half + i], sv = sin_t[(size_t)positions[t] * half + i];
-    const float x1 = to_f32(x[i]), x2 = to_f32(x[i + half]);
+    const float x1 = to_f32(x[a]), x2 = to_f32(x[b]);
     const float o1 = x1 * c - x2 * sv, o2 = x2 * c + x1 * sv;
     if (is_k) {
       ktile[key_offset(off, i, page_size)] = from_f32<TC>(o1);
       ktile[key_offset(off, i + half, page_size)] = from_f32<TC>(o2);
     } else {
-      x[i] = from_f32<TA>(o1);
-      x[i + half] = from_f32<TA>(o2);
+      TA* y = q_out ? q_out + (size_t)t * q_stride + (size_t)head * hd : x;
+      y[i] = from_f32<TA>(o1);
+      y[i + half] = from_f32<TA>(o2);
     }
   } else if (is_k) {
     // columns beyond the rotary dimension are copied as they are (all of them without tables)
@@ -259,7 +265,8 @@ __global__ void __launch_bounds__(256)
 rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const int32_t* __restrict__ positions,
                             const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                             uint16_t* __restrict__ kcache, uint16_t* __restrict__ vcache,
-                            const int32_t* __restrict__ slot_mapping, int page_size, int nh, int nkv, int hd) {
+                            const int32_t* __restrict__ slot_mapping, int page_size, int nh, int nkv, int hd,
+                            uint16_t* __restrict__ q_out, int q_stride) {
   const int t = blockIdx.x;
   const int half = hd >> 1;
   const int per_qk = hd >> 4, per_v = hd >> 3;             // items per head
@@ -284,7 +291,11 @@ rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const in
     const bool is_k = head >= nh;
     if (is_k && (!kcache || slot < 0)) continue;
     uint16_t* x = row + (size_t)head * hd;
-    const uint4 r1 = *reinterpret_cast<const uint4*>(x + i0), r2 = *reinterpret_cast<const uint4*>(x + i0 + half);
+    // where the eight pairs' members come from: columns i0.. and i0 + half.. (one member in each 16-byte piece), or,
+    // with q_out, neighbours 2 i0 .. 2 i0 + 15 (four pairs in each piece); they leave to columns i0.. and i0 + half..
+    const bool paired = q_out != nullptr;
+    const uint4 r1 = *reinterpret_cast<const uint4*>(x + (paired ? 2 * i0 : i0));
+    const uint4 r2 = *reinterpret_cast<const uint4*>(x + (paired ? 2 * i0 + 8 : i0 + half));
     const f4 c0 = load4(cos_t + pos * half + i0), c1 = load4(cos_t + pos * half + i0 + 4);
     const f4 s0 = load4(sin_t + pos * half + i0), s1 = load4(sin_t + pos * half + i0 + 4);
     const uint16_t* a = reinterpret_cast<const uint16_t*>(&r1);
@@ -295,7 +306,9 @@ rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const in
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float c = e < 4 ? c0.v[e] : c1.v[e - 4], sn = e < 4 ? s0.v[e] : s1.v[e - 4];
-      const float x1 = bf16_bits_to_f32(a[e]), x2 = bf16_bits_to_f32(b[e]);
+      const uint16_t m1 = paired ? (e < 4 ? a[2 * e] : b[2 * (e - 4)]) : a[e];
+      const uint16_t m2 = paired ? (e < 4 ? a[2 * e + 1] : b[2 * (e - 4) + 1]) : b[e];
+      const float x1 = bf16_bits_to_f32(m1), x2 = bf16_bits_to_f32(m2);
       o1[e] = f32_to_bf16_bits(x1 * c - x2 * sn);
       o2[e] = f32_to_bf16_bits(x2 * c + x1 * sn);
     }
@@ -304,8 +317,9 @@ rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const in
       *reinterpret_cast<uint4*>(ktile + key_offset(off, i0, page_size)) = w1;
       *reinterpret_cast<uint4*>(ktile + key_offset(off, i0 + half, page_size)) = w2;
     } else {
-      *reinterpret_cast<uint4*>(x + i0) = w1;
-      *reinterpret_cast<uint4*>(x + i0 + half) = w2;
+      uint16_t* y = paired ? q_out + (size_t)t * q_stride + (size_t)head * hd : x;
+      *reinterpret_cast<uint4*>(y + i0) = w1;
+      *reinterpret_cast<uint4*>(y + i0 + half) = w2;
     }
   }
 }
@@ -313,8 +327,10 @@ rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const in
 extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, const int32_t* positions,
                                       const float* cos_t, const float* sin_t, int rotary_dim, void* kcache,
                                       void* vcache, int cache_dtype, const int32_t* slot_mapping, int page_size,
-                                      int n_tokens, int nh, int nkv, int hd, hipStream_t stream) {
+                                      int n_tokens, int nh, int nkv, int hd, void* q_out, int q_stride,
+                                      hipStream_t stream) {
   if (n_tokens <= 0) return 0;
+  if (q_out && (cos_t == nullptr || rotary_dim != hd || q_stride < nh * hd)) return ATOMA_ERR_SHAPE;
   if (rotary_dim < 0 || rotary_dim > hd || (rotary_dim & 1) || row_stride < (nh + 2 * nkv) * hd || page_size <= 0)
     return ATOMA_ERR_SHAPE;
   if (nh + 2 * nkv > 65535) return ATOMA_ERR_SHAPE;
@@ -324,18 +340,20 @@ extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, 
   if (hd & 1) return ATOMA_ERR_SHAPE;
   // few tokens (decode steps) are quicker with many small blocks; measured on MI355X
   if (n_tokens >= 32 && act_dtype == kBF16 && cache_dtype == kBF16 && cos_t && sin_t && rotary_dim == hd && hd % 16 == 0 &&
-      row_stride % 8 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)kcache & 15) == 0 &&
+      row_stride % 8 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)kcache & 15) == 0 && q_stride % 8 == 0 &&
+      ((uintptr_t)q_out & 15) == 0 &&
       ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0) {
     hipLaunchKernelGGL(rope_cache_write_vec_kernel, dim3(n_tokens), dim3(256), 0, stream, (uint16_t*)qkv, row_stride,
                        positions, cos_t, sin_t, (uint16_t*)kcache, (uint16_t*)vcache, slot_mapping, page_size, nh,
-                       nkv, hd);
+                       nkv, hd, (uint16_t*)q_out, q_stride);
     ATOMA_LAUNCH_CHECK();
     return 0;
   }
   dim3 grid(n_tokens, (items + 255) / 256), block(256);
 #define ATOMA_ROPE(TA, TC)                                                                                        \
   hipLaunchKernelGGL((rope_cache_write_kernel<TA, TC>), grid, block, 0, stream, (TA*)qkv, row_stride, positions, \
-                     cos_t, sin_t, rotary_dim, (TC*)kcache, (TC*)vcache, slot_mapping, page_size, nh, nkv, hd, heads)
+                     cos_t, sin_t, rotary_dim, (TC*)kcache, (TC*)vcache, slot_mapping, page_size, nh, nkv, hd, heads, \
+                     (TA*)q_out, q_stride)
   if (act_dtype == kF32 && cache_dtype == kF32) ATOMA_ROPE(float, float);
   else if (act_dtype == kBF16 && cache_dtype == kBF16) ATOMA_ROPE(bf16_t, bf16_t);
   else if (act_dtype == kF32 && cache_dtype == kBF16) ATOMA_ROPE(float, bf16_t);

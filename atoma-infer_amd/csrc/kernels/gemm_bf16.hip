@@ -13,16 +13,28 @@
 //
 // Needs K % (32 * WK * slices) == 0 and 16-byte aligned rows; the host wrapper checks and otherwise refuses.
 #include "common.h"
+#include "cache_layout.h"
 
 using namespace atoma;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false>
+// What the rotary epilogue needs beside the product: see the ROPE branch below.
+struct RopeArgs {
+  const int32_t* positions;      // [M]
+  const float* cos_t;            // [positions, hd / 2]
+  const float* sin_t;
+  uint16_t* kcache;              // [pages, nkv, page_size * hd] tiles, bfloat16
+  uint16_t* vcache;
+  const int32_t* slot_mapping;   // [M]; negative: no cache write for the row
+  int page_size, nh, nkv, hd;
+};
+
+template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false, bool ROPE = false>
 __global__ void __launch_bounds__(64 * WN * WK)
 gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
-                   int K, int lda, int ldw, int ldc, size_t plane) {
+                   int K, int lda, int ldw, int ldc, size_t plane, RopeArgs ra) {
   // loads of U steps of K are issued together before their MFMAs, so that a wave keeps U * (RT + MT) 16-byte
   // loads per lane in flight: the product is bound by memory latency and bandwidth, not by arithmetic
   constexpr int U = (RT + MT <= 2) ? 4 : (RT + MT <= 5) ? 2 : 1;
@@ -158,6 +170,60 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
     return;
   }
 
+  if constexpr (ROPE) {
+    // W is the fused q, k, v projection with the rows of every q and k head ordered so that the members of
+    // rotary pair i = (column i, column i + hd/2) are outputs 2i and 2i + 1 of the head: a lane's four outputs are
+    // two whole pairs, i and i + 1.  They are rotated here and go to their own columns: q to C [M, nh * hd], k
+    // into the row's slot of the paged cache (the order inside a tile: cache_layout.h); v heads are copied into
+    // theirs.  The same arithmetic as the rotary kernel (csrc/kernels/rotary.h:116-131 of the reference), on the
+    // float32 sums before they are rounded.
+    static_assert(!ROPE || sizeof(TC) == 2, "the rotary epilogue writes bfloat16");
+    const int hd = ra.hd, half = hd >> 1;
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      const int n0 = n_base + r * 16 + kg * 4;
+      if (n0 + 3 >= N) continue;
+      const int head = n0 / hd, d0 = n0 % hd;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const int row = m * 16 + r16;
+        if (row >= M) continue;
+        const float x0 = acc[r][m][0], x1 = acc[r][m][1], x2 = acc[r][m][2], x3 = acc[r][m][3];
+        if (head >= ra.nh + ra.nkv) {
+          const int slot = ra.slot_mapping[row];
+          if (slot < 0) continue;
+          const int page = slot / ra.page_size, off = slot % ra.page_size;
+          uint16_t* tile = ra.vcache + ((size_t)page * ra.nkv + (head - ra.nh - ra.nkv)) * ra.page_size * hd;
+          tile[value_offset(d0, off, hd, ra.page_size)] = f32_to_bf16_bits(x0);
+          tile[value_offset(d0 + 1, off, hd, ra.page_size)] = f32_to_bf16_bits(x1);
+          tile[value_offset(d0 + 2, off, hd, ra.page_size)] = f32_to_bf16_bits(x2);
+          tile[value_offset(d0 + 3, off, hd, ra.page_size)] = f32_to_bf16_bits(x3);
+          continue;
+        }
+        const int i = d0 >> 1;                       // even: columns i, i + 1 and their partners lie together
+        const size_t at = (size_t)ra.positions[row] * half + i;
+        const float c0 = ra.cos_t[at], s0 = ra.sin_t[at], c1 = ra.cos_t[at + 1], s1 = ra.sin_t[at + 1];
+        const uint32_t lo = (uint32_t)f32_to_bf16_bits(x0 * c0 - x1 * s0) |
+                            ((uint32_t)f32_to_bf16_bits(x2 * c1 - x3 * s1) << 16);      // columns i, i + 1
+        const uint32_t hi = (uint32_t)f32_to_bf16_bits(x1 * c0 + x0 * s0) |
+                            ((uint32_t)f32_to_bf16_bits(x3 * c1 + x2 * s1) << 16);      // i + half, i + half + 1
+        if (head < ra.nh) {
+          uint16_t* q = reinterpret_cast<uint16_t*>(c) + (size_t)row * ldc + (size_t)head * hd;
+          *reinterpret_cast<uint32_t*>(q + i) = lo;
+          *reinterpret_cast<uint32_t*>(q + i + half) = hi;
+          continue;
+        }
+        const int slot = ra.slot_mapping[row];
+        if (slot < 0) continue;
+        const int page = slot / ra.page_size, off = slot % ra.page_size;
+        uint16_t* tile = ra.kcache + ((size_t)page * ra.nkv + (head - ra.nh)) * ra.page_size * hd;
+        *reinterpret_cast<uint32_t*>(tile + key_offset(off, i, ra.page_size)) = lo;
+        *reinterpret_cast<uint32_t*>(tile + key_offset(off, i + half, ra.page_size)) = hi;
+      }
+    }
+    return;
+  }
+
   // D[n = kg*4 + i][row of A = r16]: four consecutive columns of C per lane
   TC* cp = c + (size_t)blockIdx.y * plane;
 #pragma unroll
@@ -193,10 +259,10 @@ static int launch(const void* a, const void* w, void* c, int c_dtype, int M, int
   const size_t plane = (size_t)M * ldc;
   if (c_dtype == kF32)
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, float>), grid, block, 0, stream, (const uint16_t*)a,
-                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane);
+                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane, RopeArgs{});
   else if (c_dtype == kBF16)
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t>), grid, block, 0, stream, (const uint16_t*)a,
-                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane);
+                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane, RopeArgs{});
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();
@@ -242,7 +308,7 @@ static int launch_swiglu(const void* a, const void* w, void* c, int M, int N, in
                          hipStream_t stream) {
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, true>), grid, block, 0, stream, (const uint16_t*)a,
-                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0);
+                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, RopeArgs{});
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
@@ -271,4 +337,48 @@ extern "C" int atoma_gemm_bf16_skinny_swiglu(const void* a, const void* w, void*
     case 3: return launch_swiglu_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
     default: return launch_swiglu_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
   }
+}
+
+template <int MT, int RT, int WN, int WK>
+static int launch_rope(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
+                       const RopeArgs& ra, hipStream_t stream) {
+  dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, false, true>), grid, block, 0, stream,
+                     (const uint16_t*)a, (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, ra);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int MT>
+static int launch_rope_mt(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
+                          int rt, int wk, const RopeArgs& ra, hipStream_t stream) {
+  if (rt == 1 && wk == 4) return launch_rope<MT, 1, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  if (rt == 2 && wk == 4) return launch_rope<MT, 2, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  if (rt == 1 && wk == 8) return launch_rope<MT, 1, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  if (rt == 2 && wk == 8) return launch_rope<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  if (rt == 1 && wk == 1) return launch_rope<MT, 1, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  if (rt == 2 && wk == 1) return launch_rope<MT, 2, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  return ATOMA_ERR_SHAPE;
+}
+
+// The fused q, k, v projection of at most 32 rows with rotary encoding and the cache write in its epilogue.
+// w [(nh + 2 nkv) hd, K] with the rows of q and k heads in pair order (pair i: rows 2i, 2i + 1 of the head);
+// c [M, ldc >= nh hd] receives the rotated q in its own column order; rotated k and v go to the rows' slots of
+// the caches ([pages, nkv, page_size * hd] bfloat16 tiles).  hd % 4 == 0 (then hd / 2 is even and 4-byte stores
+// are aligned).
+extern "C" int atoma_gemm_bf16_skinny_rope(const void* a, const void* w, void* c, int M, int K, int lda, int ldw,
+                                           int ldc, int rt, int wk, const int32_t* positions, const float* cos_t,
+                                           const float* sin_t, void* kcache, void* vcache,
+                                           const int32_t* slot_mapping, int page_size, int nh, int nkv, int hd,
+                                           hipStream_t stream) {
+  if (M <= 0) return 0;
+  const int N = (nh + 2 * nkv) * hd;
+  if (M > 32 || K <= 0 || wk <= 0 || K % (32 * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K ||
+      ldc < nh * hd || (ldc & 1) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)c & 3) || (hd & 3) ||
+      nh <= 0 || nkv <= 0 || page_size <= 0 || !positions || !cos_t || !sin_t || !kcache || !vcache ||
+      !slot_mapping || ((uintptr_t)kcache & 3))
+    return ATOMA_ERR_SHAPE;
+  const RopeArgs ra{positions, cos_t, sin_t, (uint16_t*)kcache, (uint16_t*)vcache, slot_mapping, page_size, nh, nkv, hd};
+  if (M <= 16) return launch_rope_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
+  return launch_rope_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
 }

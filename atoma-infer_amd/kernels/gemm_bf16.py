@@ -163,3 +163,32 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
     _check(lib().atoma_gemm_bf16_skinny_swiglu(_p(x), _p(w), _p(out), m, n, k, x.stride(0) if m > 1 else k,
                                                w.stride(0), n // 2, rt, wk, _stream()), "gemm_bf16_skinny_swiglu")
     return out
+
+
+ROPE_MAX_M = 32
+
+
+def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                    kcache: torch.Tensor, vcache: torch.Tensor, slot_mapping: torch.Tensor, page_size: int, nh: int,
+                    nkv: int, hd: int) -> Optional[torch.Tensor]:
+    """The fused q, k, v projection with rotary encoding and the cache write in its epilogue, for few rows of x.
+
+    ``w`` has the rows of its q and k heads in pair order (see ``parts/attention.py``).  Returns the rotated q
+    [M, nh * hd]; k (rotated) and v are in the cache.  None when the shape is not taken.
+    """
+    m, k = x.shape
+    n = w.shape[0]
+    if (m > ROPE_MAX_M or n != (nh + 2 * nkv) * hd or hd % 4 or not skinny_ok(x, w)
+            or kcache.dtype is not torch.bfloat16 or vcache.dtype is not torch.bfloat16
+            or cos.dtype is not torch.float32 or cos.shape[1] != hd // 2 or not cos.is_contiguous()
+            or not sin.is_contiguous() or not kcache.is_contiguous() or not vcache.is_contiguous()):
+        return None
+    rt, wk, _ = _plan(m, n, k, False)
+    if rt > 2:
+        rt = 2
+    out = torch.empty((m, nh * hd), dtype=torch.bfloat16, device=x.device)
+    _check(lib().atoma_gemm_bf16_skinny_rope(_p(x), _p(w), _p(out), m, k, x.stride(0) if m > 1 else k, w.stride(0),
+                                             nh * hd, rt, wk, _p(positions), _p(cos), _p(sin), _p(kcache), _p(vcache),
+                                             _p(slot_mapping), int(page_size), nh, nkv, hd, _stream()),
+           "gemm_bf16_skinny_rope")
+    return out

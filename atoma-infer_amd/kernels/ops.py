@@ -126,10 +126,13 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
 def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torch.Tensor],
                      sin: Optional[torch.Tensor], rotary_dim: int, kcache: Optional[torch.Tensor],
                      vcache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], page_size: int, nh: int,
-                     nkv: int, hd: int) -> None:
+                     nkv: int, hd: int, q_out: Optional[torch.Tensor] = None) -> None:
     """Rotate q and k of ``qkv`` [T, (nh + 2 nkv) hd] (q in place), store rotated k and v at ``slot_mapping``.
 
     kcache and vcache are [pages, nkv, page_size * hd] tiles (order: cache/layout.py).  Null caches: rotate q only.
+    With ``q_out`` [T, nh hd] the members of pair i arrive as columns 2i and 2i + 1 of a q or k head (rows of the
+    projection reordered at load time); the rotated q is written to ``q_out`` and k to the cache in their own
+    column order, and ``qkv`` is left as it is.
     """
     _dev(qkv, positions, cos, sin, kcache, vcache, slot_mapping)
     t = qkv.shape[0]
@@ -140,6 +143,11 @@ def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[t
               and sin.is_contiguous() and cos.shape == sin.shape and cos.shape[1] == rotary_dim // 2,
               "rotary tables must be float32 [positions, rotary_dim/2]")
     cache_code = _code(qkv, "qkv")
+    if q_out is not None:
+        _dev(q_out)
+        _need(q_out.dtype is qkv.dtype and q_out.dim() == 2 and q_out.stride(1) == 1 and q_out.shape[0] == t
+              and q_out.shape[1] >= nh * hd and cos is not None and rotary_dim == hd,
+              "q_out must be [T, nh hd] of qkv's dtype, with the whole head rotated")
     if kcache is not None:
         _need(vcache is not None and slot_mapping is not None, "cache write needs k, v and slots")
         _i32(slot_mapping, "slot_mapping", t)
@@ -150,7 +158,8 @@ def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[t
         cache_code = _code(kcache, "cache")
     _check(core().atoma_rope_cache_write(_p(qkv), _code(qkv, "qkv"), qkv.stride(0), _p(positions), _p(cos), _p(sin),
                                          rotary_dim, _p(kcache), _p(vcache), cache_code, _p(slot_mapping), page_size,
-                                         t, nh, nkv, hd, _stream()), "rope_cache_write")
+                                         t, nh, nkv, hd, _p(q_out), q_out.stride(0) if q_out is not None else 0,
+                                         _stream()), "rope_cache_write")
 
 
 def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, out: torch.Tensor,

@@ -8,7 +8,11 @@ of q and k (:298-299), keys and values written to the cache before attention (mo
 last ``window`` of them) of its own request through the block table.
 
 The three projection matrices are fused into one [(nh + 2 nkv) hd, width] matrix at load time; results equal
-the separate products.
+the separate products.  When the position encoding rotates whole heads in half-split pairs (i, i + hd/2), the rows
+of every q and k head are reordered at load time so that a pair's members leave the projection as neighbours
+(2i, 2i + 1): then the projection's own epilogue can rotate q and k and write k and v into the cache, and decode
+steps need no kernel between the projection and attention.  Rotated q and cached k are always in their own column
+order, whoever rotated them, so any call may read any call's cache.
 """
 from __future__ import annotations
 
@@ -40,6 +44,7 @@ class PagedAttention(Mixer):
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
         self.act_dtype = torch.float32
+        self.paired = False      # q and k columns in pair order (set at load time)
 
     # -- declaration ----------------------------------------------------------------------------------
     def weight_specs(self) -> Dict[str, WeightSpec]:
@@ -53,11 +58,18 @@ class PagedAttention(Mixer):
     def load(self, get, device, act_dtype) -> None:
         ws = [get("q_proj.weight"), get("k_proj.weight"), get("v_proj.weight")]
         dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        if self.position is not None:
+            self.position.load(get, device, act_dtype)
+        tables = self.position.rotary_tables() if self.position is not None else None
+        self.paired = tables is not None and tables[2] == self.hd
+        if self.paired:
+            half = self.hd // 2
+            order = torch.stack([torch.arange(half), torch.arange(half) + half], dim=1).reshape(-1)   # 0, half, 1, ...
+            ws[0] = ws[0].reshape(self.nh, self.hd, self.width)[:, order].reshape(self.nh * self.hd, self.width)
+            ws[1] = ws[1].reshape(self.nkv, self.hd, self.width)[:, order].reshape(self.nkv * self.hd, self.width)
         self.w_qkv = torch.cat([w.to(device=device, dtype=dt) for w in ws], dim=0).contiguous()
         self.w_o = get("o_proj.weight").to(device).contiguous()
         self.act_dtype = act_dtype
-        if self.position is not None:
-            self.position.load(get, device, act_dtype)
 
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
@@ -79,17 +91,28 @@ class PagedAttention(Mixer):
         writes = cache.writable
         # a call that reads another call's cache needs its queries only
         w = self.w_qkv if writes else self.w_qkv[: nh * hd]
-        qkv = linear(x, w)
         k_cache, v_cache = cache.k, cache.v
         tables = self.position.rotary_tables() if self.position is not None else None
-        if tables is not None or self.position is None:
+        qkv = None
+        if self.paired and writes and x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            qkv = gemm_bf16.try_linear_rope(x, w, ctx.positions, tables[0], tables[1], k_cache, v_cache,
+                                            cache.slot_mapping, cache.page_size, nh, nkv, hd)
+        if qkv is not None:
+            pass        # rotated and stored by the product's epilogue
+        elif tables is not None or self.position is None:
+            raw = linear(x, w)
             cos, sin, rd = tables if tables is not None else (None, None, 0)
+            # pair order in, own order out: q cannot be rotated in place then
+            qkv = torch.empty((t, nh * hd), dtype=raw.dtype, device=raw.device) if self.paired else raw
+            q_out = qkv if self.paired else None
             if writes:
-                ops.rope_cache_write(qkv, ctx.positions, cos, sin, rd, k_cache, v_cache, cache.slot_mapping,
-                                     cache.page_size, nh, nkv, hd)
+                ops.rope_cache_write(raw, ctx.positions, cos, sin, rd, k_cache, v_cache, cache.slot_mapping,
+                                     cache.page_size, nh, nkv, hd, q_out)
             else:
-                ops.rope_cache_write(qkv, ctx.positions, cos, sin, rd, None, None, None, 1, nh, 0, hd)
+                ops.rope_cache_write(raw, ctx.positions, cos, sin, rd, None, None, None, 1, nh, 0, hd, q_out)
         else:
+            qkv = linear(x, w)
             q = qkv[:, : nh * hd].view(t, nh, hd)
             if writes:
                 k = qkv[:, nh * hd: (nh + nkv) * hd].view(t, nkv, hd)

@@ -312,8 +312,12 @@ def test_attention_reference_vectors():
 @pytest.mark.parametrize("nh,nkv,hd,page", [(5, 2, 48, 4), (8, 2, 64, 16), (3, 1, 40, 16), (2, 2, 128, 16)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("t", [9, 45])      # few tokens and many take different kernels in bfloat16
-def test_rope_cache_write(dtype, nh, nkv, hd, page, t):
+@pytest.mark.parametrize("paired", [False, True])
+def test_rope_cache_write(dtype, nh, nkv, hd, page, t, paired):
+    """``paired``: the members of pair i arrive as columns 2i and 2i + 1 and the rotated q leaves to a buffer of its
+    own: the same rows in pair order must give the plain result, in the plain order."""
     from atoma_infer_amd.kernels import ops
+    order = torch.stack([torch.arange(hd // 2), torch.arange(hd // 2) + hd // 2], dim=1).reshape(-1)
     g = torch.Generator().manual_seed(3)
     qkv = torch.randn(t, (nh + 2 * nkv) * hd, generator=g).to(dtype)
     pos = torch.tensor(([0, 1, 2, 3, 4, 50, 51, 7, 8] * 5)[:t], dtype=torch.int32)
@@ -326,9 +330,18 @@ def test_rope_cache_write(dtype, nh, nkv, hd, page, t):
     kc = torch.zeros(8, nkv, page, hd, dtype=dtype)
     vc = torch.zeros(8, nkv, hd, page, dtype=dtype)
     from atoma_infer_amd.cache.layout import pack_keys, pack_values, unpack_keys, unpack_values
-    d_qkv, d_kc, d_vc = qkv.to(DEV), pack_keys(kc).to(DEV), pack_values(vc).to(DEV)
-    ops.rope_cache_write(d_qkv, pos.to(DEV), cos.to(DEV), sin.to(DEV), hd, d_kc, d_vc, slots.to(DEV), page, nh, nkv, hd)
+    x_in = qkv.view(t, nh + 2 * nkv, hd).clone()
+    if paired:
+        x_in[:, :nh + nkv] = x_in[:, :nh + nkv][:, :, order]        # q and k heads in pair order, v as it is
+    d_qkv, d_kc, d_vc = x_in.reshape(t, -1).to(DEV), pack_keys(kc).to(DEV), pack_values(vc).to(DEV)
+    q_out = torch.empty(t, nh * hd, dtype=dtype, device=DEV) if paired else None
+    before = d_qkv.clone()
+    ops.rope_cache_write(d_qkv, pos.to(DEV), cos.to(DEV), sin.to(DEV), hd, d_kc, d_vc, slots.to(DEV), page, nh, nkv, hd,
+                         q_out)
     d_kc, d_vc = unpack_keys(d_kc, page, hd), unpack_values(d_vc, page, hd)
+    if paired:       # the rotated q is in q_out, in its own column order; the input is left alone
+        assert torch.equal(d_qkv, before)
+        d_qkv = torch.cat([q_out, d_qkv[:, nh * hd:]], dim=1)
     x = qkv.float().view(t, nh + 2 * nkv, hd)
     c, s = cos[pos.long()][:, None, :], sin[pos.long()][:, None, :]
     x1, x2 = x[..., : hd // 2], x[..., hd // 2:]
@@ -379,3 +392,49 @@ def test_gemm_with_swiglu_epilogue(m, inter, k):
     want = torch.nn.functional.silu(g) * u
     assert (out.double().cpu() - want).abs().max() <= 1e-2 * want.abs().max()
     assert gemm_bf16.try_linear_swiglu(rnd(40, k, dtype=torch.bfloat16), interleave16(wg, wu)) is None   # too many rows
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 23])
+@pytest.mark.parametrize("nh,nkv,hd,k", [(8, 2, 64, 256), (3, 1, 16, 64), (32, 8, 64, 2048), (5, 5, 48, 96)])
+def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
+    """The q, k, v projection that rotates and stores in its epilogue against product, rotation and store done
+    apart."""
+    from atoma_infer_amd.kernels import gemm_bf16, ops
+    from atoma_infer_amd.cache.layout import pack_keys, pack_values
+    page, pages = 16, 6
+    n = (nh + 2 * nkv) * hd
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    w = rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.2)
+    g = torch.Generator().manual_seed(5)
+    pos = torch.randint(0, 90, (m,), generator=g).int().to(DEV)
+    slots = torch.randperm(pages * page, generator=g)[:m].int()
+    if m > 2:
+        slots[2] = -1
+    slots = slots.to(DEV)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))
+    ang = torch.arange(96).float()[:, None] * inv[None]
+    cos, sin = torch.cos(ang).to(DEV), torch.sin(ang).to(DEV)
+
+    def caches():
+        gg = torch.Generator().manual_seed(9)
+        return (pack_keys(torch.randn(pages, nkv, page, hd, generator=gg).bfloat16()).to(DEV),
+                pack_values(torch.randn(pages, nkv, hd, page, generator=gg).bfloat16()).to(DEV))
+    kc1, vc1 = caches()
+    q1 = gemm_bf16.try_linear_rope(x, w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv, hd)
+    assert q1 is not None and tuple(q1.shape) == (m, nh * hd)
+    # apart, with float32 in between (the fused kernel rotates the float32 sums)
+    kc2, vc2 = caches()
+    qkv = ops.gemm_generic(x, w, torch.float32)
+    kc2f, vc2f = kc2.float(), vc2.float()
+    q2 = torch.empty(m, nh * hd, dtype=torch.float32, device=DEV)
+    ops.rope_cache_write(qkv, pos, cos, sin, hd, kc2f, vc2f, slots, page, nh, nkv, hd, q2)
+    tol = 1e-2
+    assert (q1.float() - q2).abs().max() <= tol * q2.abs().max()
+    assert (kc1.float() - kc2f).abs().max() <= tol * kc2f.abs().max()
+    assert (vc1.float() - vc2f).abs().max() <= tol * vc2f.abs().max()
+    # the row without a slot wrote nothing, and untouched slots keep what they held
+    kc0, vc0 = caches()
+    same = (kc1 == kc0)
+    assert int((~same).sum()) <= (m - (1 if m > 2 else 0)) * nkv * hd
+    assert gemm_bf16.try_linear_rope(rnd(40, k, dtype=torch.bfloat16), w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv,
+                                     hd) is None   # too many rows
