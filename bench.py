@@ -53,7 +53,10 @@ def decode_run(model, batch, prompt_len, steps, warmup, context, seed=0):
     eng = make_engine(model, batch, context)
     g = torch.Generator().manual_seed(seed)
     vocab = model.vocab_size
-    params = GenerateParameters(do_sample=False, max_new_tokens=steps + warmup + batch + 8, ignore_eos_token=True)
+    # requests that finish their prompt early decode while the others are still in theirs
+    prompt_steps = batch * (-(-prompt_len // max(2048, batch)))
+    params = GenerateParameters(do_sample=False, max_new_tokens=steps + warmup + prompt_steps + 8,
+                                ignore_eos_token=True)
     for _ in range(batch):
         eng.add_request(torch.randint(0, vocab, (prompt_len,), generator=g).tolist(), params)
     while any(r.in_prefill for r in eng.scheduler.running) or eng.scheduler.waiting:
@@ -118,7 +121,7 @@ def main() -> int:
     if int(os.environ.get("WORLD_SIZE", "1")) > 1:
         print("bench.py: started with WORLD_SIZE > 1; this engine runs on one GPU", flush=True)
         return 2
-    if args.prompt_len + args.steps + args.warmup + 72 > args.context:
+    if args.prompt_len + args.steps + args.warmup + args.batch * (-(-args.prompt_len // 2048)) + 8 > args.context:
         print("bench.py: prompt + steps exceed the context", file=sys.stderr)
         return 1
 
