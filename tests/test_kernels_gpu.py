@@ -185,12 +185,15 @@ class FakeCache:
         self.block_tables, self.page_size = block_tables, page
 
 
-def paged_setup(lens, nkv, hd, page, dtype, seed=0):
+def paged_setup(lens, nkv, hd, page, dtype, seed=0, edit=None):
     """Random keys/values for requests of the given lengths, laid into shuffled pages.  Returns
-    (k list, v list as float32 [len, nkv, hd]), kcache, vcache, block_tables."""
+    (k list, v list as float32 [len, nkv, hd]), kcache, vcache, block_tables.  ``edit(ks, vs)`` may change them
+    before they are laid out."""
     g = torch.Generator().manual_seed(seed)
     ks = [torch.randn(n, nkv, hd, generator=g).to(dtype) for n in lens]
     vs = [torch.randn(n, nkv, hd, generator=g).to(dtype) for n in lens]
+    if edit is not None:
+        edit(ks, vs)
     blocks = [-(-n // page) for n in lens]
     total = sum(blocks) + 3
     perm = torch.randperm(total, generator=g).tolist()
@@ -271,6 +274,62 @@ def test_paged_attention(nh, nkv, hd, page, window, entries, kind):
         err = (got - want).abs().max() / want.abs().max()
         assert err < tol, f"entry {e} ({s}, {c}): {err:.3e}"
         row += c
+
+
+STAND_OUT = [
+    # (window, [(start, count)], key that gets the large score)
+    (0, [(699, 1)], 0), (0, [(699, 1)], 15), (0, [(699, 1)], 16), (0, [(699, 1)], 127), (0, [(699, 1)], 128),
+    (0, [(699, 1)], 255), (0, [(699, 1)], 256), (0, [(699, 1)], 511), (0, [(699, 1)], 512), (0, [(699, 1)], 698),
+    (0, [(699, 1)], 699),
+    (100, [(699, 1)], 599),      # just outside the window: must not be seen
+    (100, [(699, 1)], 600),      # the window's first key
+    (0, [(480, 40)], 479), (0, [(480, 40)], 500), (0, [(480, 40)], 519),      # a portion: all rows, some rows, one row
+    (64, [(480, 40)], 440), (64, [(480, 40)], 456),      # a window's edge that moves through the portion's rows
+    (0, [(0, 300)], 0), (0, [(0, 300)], 31), (0, [(0, 300)], 32), (0, [(0, 300)], 287),
+]
+
+
+@pytest.mark.parametrize("window,entries,key", STAND_OUT)
+@pytest.mark.parametrize("kind", ["generic_f32", "generic_bf16", "mfma"])
+def test_attention_when_one_key_stands_out(window, entries, key, kind):
+    """Among hundreds of random keys a wrong one changes the result by less than the tolerance.  Here every query
+    points at one key, whose weight is then nearly one wherever the row may see it: a fault at a page's edge, at
+    a chunk's border, at the window's edge or in the causal mask shows as a wrong row."""
+    from atoma_infer_amd.kernels import attention_bf16, ops
+    nh, nkv, hd, page = 4, 2, 64, 16
+    dtype = torch.float32 if kind == "generic_f32" else torch.bfloat16
+    starts, counts = [s for s, _ in entries], [c for _, c in entries]
+    lens = [s + c for s, c in entries]
+    ks, vs, kc, vc, bt = paged_setup(lens, nkv, hd, page, dtype, seed=key + 1)
+    t = sum(counts)
+    # every head's query is three times its KV head's key at `key`: that score is about 24, the others' about 3
+    q = (3.0 * ks[0][key].float()).repeat_interleave(nh // nkv, dim=0)        # [nh, hd]
+    qkv = torch.zeros(t, (nh + 2 * nkv) * hd)
+    qkv[:, : nh * hd] = q.reshape(1, nh * hd)
+    qkv = qkv.to(dtype).to(DEV)
+    out = torch.empty(t, nh * hd, dtype=dtype, device=DEV)
+    ctx, cache = FakeCtx(starts, counts), FakeCache(bt, page)
+    scale = 1.0 / math.sqrt(hd)
+    if kind == "mfma":
+        assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, cache, scale, window, nh, nkv, hd)
+    else:
+        ops.paged_attention_generic(qkv, kc, vc, out, bt, ctx.token_seq, ctx.positions, scale, window, page, nh,
+                                    nkv, hd)
+    (s0, c0) = entries[0]
+    qq = qkv[:, : nh * hd].cpu().view(c0, nh, hd)
+    want = plain_attention(qq, ks[0], vs[0], s0, scale, window, nh // nkv).reshape(c0, nh * hd)
+    got = out.double().cpu()
+    tol = 2e-5 if dtype is torch.float32 else 2e-2
+    for r in range(c0):
+        err = (got[r] - want[r]).abs().max() / want[r].abs().max()
+        assert err < tol, f"row at position {s0 + r}: {err:.3e}"
+    # the test means what it says: rows that may see the key return its value, nearly
+    p = torch.arange(s0, s0 + c0)
+    sees = (key <= p) & ((key > p - window) if window else torch.ones_like(p, dtype=torch.bool))
+    vj = vs[0][key].double().repeat_interleave(nh // nkv, dim=0).reshape(nh * hd)
+    for r in range(c0):
+        close = (want[r] - vj).abs().max() < 0.05
+        assert bool(close) == bool(sees[r]), (r, float((want[r] - vj).abs().max()))
 
 
 def test_attention_reference_vectors():

@@ -101,6 +101,93 @@ def test_embedding_and_head_parts():
                        table.float()[[4, 0, 49]])
 
 
+class PartCtx:
+    """What a mixer reads of a step's context, for one request that brings tokens start .. start + count - 1."""
+
+    def __init__(self, start, count):
+        import numpy as np
+        self.h_starts, self.h_counts = np.asarray([start], dtype=np.int32), np.asarray([count], dtype=np.int32)
+        self.positions = torch.arange(start, start + count, dtype=torch.int32, device=DEV)
+        self.token_seq = torch.zeros(count, dtype=torch.int32, device=DEV)
+        self.scratch, self.plans = {}, {}
+
+
+def attention_part(act, nh, nkv, hd, width, window, seed):
+    from atoma_infer_amd.parts import PagedAttention, RotaryEncoding
+    g = torch.Generator().manual_seed(seed)
+    ws = {n: (torch.randn(*sh, generator=g) * 0.2).to(torch.bfloat16) for n, sh in
+          (("q_proj.weight", (nh * hd, width)), ("k_proj.weight", (nkv * hd, width)),
+           ("v_proj.weight", (nkv * hd, width)), ("o_proj.weight", (width, nh * hd)))}
+    part = PagedAttention(width, nh, nkv, hd, RotaryEncoding(hd, 10000.0, 256), window)
+    assert {k: v.shape for k, v in part.weight_specs().items()} == {k: tuple(v.shape) for k, v in ws.items()}
+    assert part.cache_spec().kv_heads == nkv and part.cache_spec().head_size == hd and part.cache_spec().window == window
+    part.load(getter(ws), torch.device(DEV), act)
+    return part, ws
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,width,window", [(4, 2, 16, 48, None), (3, 3, 32, 96, 20), (8, 2, 64, 64, None)])
+def test_attention_part(act, nh, nkv, hd, width, window):
+    """The mixer alone over a cache of its own: a prompt in two portions, then tokens one by one, against the plain
+    attention of the whole sequence (projections, rotation, grouped heads, window, output projection)."""
+    from atoma_infer_amd.cache.pool import LayerCache
+    part, ws = attention_part(act, nh, nkv, hd, width, window, seed=nh + hd)
+    page, pages, n = 16, 8, 70
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(n, width, generator=g).to(act)
+    cfg = {"hidden_size": nh * hd, "num_attention_heads": nh, "num_key_value_heads": nkv, "rope_theta": 10000.0}
+    fw = {"p.self_attn." + k: v.float() for k, v in ws.items()}
+    # the plain function projects from width to nh * hd itself; it reads hidden_size only for the head size
+    want = P.self_attention(x.float(), fw, "p.self_attn.", cfg, torch.arange(n), window)
+    order = torch.randperm(pages, generator=g)[: -(-n // page)]
+    bt = order.int().view(1, -1).to(DEV)
+    k = torch.zeros(pages, nkv, page * hd, dtype=act, device=DEV)
+    v = torch.zeros(pages, nkv, page * hd, dtype=act, device=DEV)
+    got = []
+    for start, count in [(0, 37), (37, 20)] + [(i, 1) for i in range(57, n)]:
+        pos = torch.arange(start, start + count)
+        slots = (order[pos // page] * page + pos % page).int().to(DEV)
+        cache = LayerCache(k=k, v=v, page_size=page, writable=True, group=0, slot_mapping=slots, block_tables=bt)
+        y = part.forward(x[start:start + count].to(DEV), PartCtx(start, count), cache)
+        got.append((y.sum(0) if y.dim() == 3 else y).float().cpu())
+    err = frob_err(torch.cat(got), want)
+    assert err < (TOL_F32 if act is torch.float32 else TOL_BF16), err
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+def test_pre_norm_block_part(act):
+    """The arrangement alone: h = x + mixer(norm(x)), y = h + ffn(norm(h)), with the sums left to the next norm."""
+    from atoma_infer_amd.cache.pool import LayerCache
+    from atoma_infer_amd.parts import PreNormBlock, RMSNorm, SwiGLU
+    nh, nkv, hd, width, inter, eps = 4, 2, 16, 64, 96, 1e-5
+    mixer, ws = attention_part(act, nh, nkv, hd, width, None, seed=7)
+    g = torch.Generator().manual_seed(8)
+    fw = {n: (torch.randn(*sh, generator=g) * 0.1).to(torch.bfloat16) for n, sh in
+          (("gate_proj.weight", (inter, width)), ("up_proj.weight", (inter, width)), ("down_proj.weight", (width, inter)))}
+    n1, n2 = (1 + 0.1 * torch.randn(width, generator=g)).bfloat16(), (1 + 0.1 * torch.randn(width, generator=g)).bfloat16()
+    block = PreNormBlock(RMSNorm(width, eps), mixer, RMSNorm(width, eps), SwiGLU(width, inter))
+    tensors = {"input_layernorm.weight": n1, "post_attention_layernorm.weight": n2}
+    tensors.update({"self_attn." + k: v for k, v in ws.items()})
+    tensors.update({"mlp." + k: v for k, v in fw.items()})
+    assert set(block.weight_specs()) == set(tensors)
+    block.load(getter(tensors), torch.device(DEV), act)
+    n, page = 21, 16
+    x = torch.randn(n, width, generator=g)
+    cfg = {"hidden_size": width, "num_attention_heads": nh, "num_key_value_heads": nkv, "rope_theta": 10000.0,
+           "rms_norm_eps": eps}
+    pw = {"model.layers.0." + k: v.float() for k, v in tensors.items()}
+    want = P.block(x, pw, 0, cfg, torch.arange(n))
+    resid = x.clone().to(DEV)
+    cache = LayerCache(k=torch.zeros(2, nkv, page * hd, dtype=act, device=DEV),
+                       v=torch.zeros(2, nkv, page * hd, dtype=act, device=DEV), page_size=page, writable=True, group=0,
+                       slot_mapping=torch.arange(n, dtype=torch.int32, device=DEV),
+                       block_tables=torch.tensor([[0, 1]], dtype=torch.int32, device=DEV))
+    delta = block.forward(resid, None, PartCtx(0, n), cache)
+    y = resid.cpu() + (delta.sum(0) if delta.dim() == 3 else delta).float().cpu()
+    err = frob_err(y, want)
+    assert err < (TOL_F32 if act is torch.float32 else TOL_BF16), err
+
+
 def test_part_registries():
     from atoma_infer_amd.parts import make_part, registered_kinds
     assert "attention" in registered_kinds("mixer") and "swiglu" in registered_kinds("feed_forward")
