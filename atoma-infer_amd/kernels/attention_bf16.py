@@ -5,7 +5,7 @@ has 16-token pages; otherwise it returns False and the caller runs the general k
 
 The step's entries are cut into tasks of 32 query rows (row = token x query head of one KV group) against a key
 range.  An entry with few tokens and many keys (a decoded token, a short portion late in a prompt) is split into
-256-key chunks whose partial results a second kernel merges; everything else runs each tile against all its
+128- or 256-key chunks whose partial results a second kernel merges; everything else runs each tile against all its
 keys.  The cut depends only on the entry's own start and length.  The task list is built once per step and
 shared by all layers with the same grouping and window.
 """
