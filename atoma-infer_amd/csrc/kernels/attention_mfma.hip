@@ -61,34 +61,40 @@ __device__ __forceinline__ bf16x8 pack8(const float* v) {
   return r;
 }
 
-// DEPTH blocks of keys and values are in flight per wave.  Measured on MI355X, more than one gains nothing at any
-// batch size (a decode step of few requests is bound by the start of the kernel and of the memory system, one of
-// many requests by bandwidth) and costs registers, so one is what is launched.
-template <int DEPTH>
-__global__ void __launch_bounds__(256)
+// KSPLIT waves share a task: wave h of them takes the blocks of 32 keys number h, h + KSPLIT, ... of the task's
+// range, and the KSPLIT partial results are merged through LDS at the end.  A wave walks its blocks one after the
+// other at a pace set by latencies (MFMA, exponentials, cross-lane moves), not by any unit's throughput, and a
+// launch lasts as long as its longest wave: with two waves per task the last tile of a long prompt, which sees
+// all keys, takes half the time.  Decode steps, whose tasks are short chunks, run with KSPLIT = 1.
+template <int KSPLIT>
+__global__ void __launch_bounds__(256 * KSPLIT)
 attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
                       const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
                       float* __restrict__ part_o, float* __restrict__ part_lse, const Task* __restrict__ tasks,
                       int n_tasks, const int32_t* __restrict__ block_tables, int max_blocks, float scale,
                       int window, int nh, int nkv) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int ti = blockIdx.x * 4 + wave;
-  if (ti >= n_tasks) return;
-  const Task task = tasks[ti];
-  if (task.entry < 0) return;
-  const int kvh = blockIdx.y;
+  const int slot = wave & 3, part = wave >> 2;      // which of the workgroup's four tasks, which share of its keys
+  // workgroups are numbered with the KV head running fastest: neighbours read the same block tables and finish
+  // together, and the longest tasks (which come first) start first
+  const int kvh = blockIdx.x % nkv;
+  const int ti = (blockIdx.x / nkv) * 4 + slot;
+  // with KSPLIT > 1 every wave must reach the barrier below: a wave without work runs an empty range
+  const bool has_task = ti < n_tasks && tasks[ti < n_tasks ? ti : 0].entry >= 0;
+  if (KSPLIT == 1 && !has_task) return;
+  const Task task = tasks[has_task ? ti : 0];
   const int g = nh / nkv;
   const int c = lane & 31, hg = lane >> 5;
   // the same in every lane; saying so keeps loop control and page arithmetic in scalar registers
   const int k_begin = __builtin_amdgcn_readfirstlane(task.k_begin);
-  const int k_end = __builtin_amdgcn_readfirstlane(task.k_end);
-  const int entry = __builtin_amdgcn_readfirstlane(task.entry);
+  const int k_end = has_task ? __builtin_amdgcn_readfirstlane(task.k_end) : k_begin;
+  const int entry = has_task ? __builtin_amdgcn_readfirstlane(task.entry) : 0;
 
   // this lane's row
   const int r = task.row0 + c;
   const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
-  const bool row_ok = hq < g && tok < task.count;
-  const int trow = task.tok_base + (row_ok ? tok : 0);
+  const bool row_ok = has_task && hq < g && tok < task.count;
+  const int trow = row_ok ? task.tok_base + tok : 0;
   const int p_row = row_ok ? task.pos0 + tok : -1;
   const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
   const int head = kvh * g + (row_ok ? hq : 0);
@@ -174,103 +180,128 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     }
   };
 
-  // With one block in flight, the next block's loads are issued right after S^T (the values move aside first)
-  // when registers allow; with more, buffer j is refilled for block + DEPTH once block's products are issued.
-  constexpr bool EARLY = DEPTH == 1 && HD <= 128;
-  bf16x8 kf[DEPTH][KSTEPS];
-  bf16x8 vf[DEPTH][2][DTILES];
-  {
+  // One block is in flight: the next block's loads are issued right after S^T (the values move aside first) when
+  // registers allow, else at the end of the block.
+  constexpr bool EARLY = HD <= 128;
+  constexpr int STRIDE = 32 * KSPLIT;
+  const int k_first = k_begin + 32 * part;
+  bf16x8 kf[KSTEPS];
+  bf16x8 vf[2][DTILES];
+  if (k_first < k_end) {
     int p0, p1;
-#pragma unroll
-    for (int j = 0; j < DEPTH; ++j)
-      if (k_begin + 32 * j < k_end) {
-        pages_of(k_begin + 32 * j, p0, p1);
-        load_keys(p0, p1, kf[j]);
-        load_vals(p0, p1, vf[j]);
-      }
+    pages_of(k_first, p0, p1);
+    load_keys(p0, p1, kf);
+    load_vals(p0, p1, vf);
   }
 
-  for (int kb0 = k_begin; kb0 < k_end; kb0 += 32 * DEPTH) {
+  for (int kb = k_first; kb < k_end; kb += STRIDE) {
+    // S^T = K Q^T
+    f32x16 s;
 #pragma unroll
-    for (int j = 0; j < DEPTH; ++j) {
-      const int kb = kb0 + 32 * j;
-      if (kb >= k_end) break;
-      // S^T = K Q^T
-      f32x16 s;
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    for (int st = 0; st < KSTEPS; ++st) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[st], s, 0, 0, 0);
+    const bool has_next = kb + STRIDE < k_end;
+    bf16x8 vc[2][DTILES];
 #pragma unroll
-      for (int st = 0; st < KSTEPS; ++st) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[j][st], qf[st], s, 0, 0, 0);
-      const int kb_next = kb + 32 * DEPTH;
-      bf16x8 vc[2][DTILES];
+    for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-      for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt) vc[jj][dt] = vf[j][jj][dt];
-      if (EARLY && kb_next < k_end) {
-        int p0, p1;
-        pages_of(kb_next, p0, p1);
-        load_keys(p0, p1, kf[j]);
-        load_vals(p0, p1, vf[j]);
-      }
+      for (int dt = 0; dt < DTILES; ++dt) vc[jj][dt] = vf[jj][dt];
+    if (EARLY && has_next) {
+      int p0, p1;
+      pages_of(kb + STRIDE, p0, p1);
+      load_keys(p0, p1, kf);
+      load_vals(p0, p1, vf);
+    }
 
-      // Online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4.  The running maximum is kept in
-      // units of the scaled score (score * scale * log2 e), so one fused multiply-add feeds exp2.  Only blocks
-      // that touch a row's own position, the window's edge or the end of the key range need the mask.
-      const bool edge = kb + 31 > p_lo || kb < lo_hi || kb + 32 > k_end;
-      float sv[16];
-      float bmax = -INFINITY;
-      if (edge) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
-          const bool ok = key <= p_row && key >= lo_row && key < k_end;
-          sv[i] = ok ? s[i] : -INFINITY;
-          bmax = fmaxf(bmax, sv[i]);
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          sv[i] = s[i];
-          bmax = fmaxf(bmax, sv[i]);
-        }
-      }
-      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64)) * sc2;
-      const float m_new = fmaxf(m, bmax);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      float psum = 0.f;
+    // Online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4.  The running maximum is kept in
+    // units of the scaled score (score * scale * log2 e), so one fused multiply-add feeds exp2.  Only blocks
+    // that touch a row's own position, the window's edge or the end of the key range need the mask.
+    const bool edge = kb + 31 > p_lo || kb < lo_hi || kb + 32 > k_end;
+    float sv[16];
+    float bmax = -INFINITY;
+    if (edge) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
-        psum += sv[i];
+        const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
+        const bool ok = key <= p_row && key >= lo_row && key < k_end;
+        sv[i] = ok ? s[i] : -INFINITY;
+        bmax = fmaxf(bmax, sv[i]);
       }
-      psum += __shfl_xor(psum, 32, 64);
-      // the accumulators are rescaled only when some row's maximum has grown (a wave-uniform decision)
-      const bool grew = __ballot(m_new > m) != 0;
-      if (grew) {
-        const float corr = __builtin_amdgcn_exp2f(m - m_use);
-        l *= corr;
+    } else {
 #pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
-        m = m_new;
+      for (int i = 0; i < 16; ++i) {
+        sv[i] = s[i];
+        bmax = fmaxf(bmax, sv[i]);
       }
-      l += psum;
+    }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64)) * sc2;
+    const float m_new = fmaxf(m, bmax);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
+      psum += sv[i];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    // the accumulators are rescaled only when some row's maximum has grown (a wave-uniform decision)
+    const bool grew = __ballot(m_new > m) != 0;
+    if (grew) {
+      const float corr = __builtin_amdgcn_exp2f(m - m_use);
+      l *= corr;
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
+      m = m_new;
+    }
+    l += psum;
 
-      // O^T += V^T P^T
-      const bf16x8 pf0 = pack8(sv), pf1 = pack8(sv + 8);
+    // O^T += V^T P^T
+    const bf16x8 pf0 = pack8(sv), pf1 = pack8(sv + 8);
 #pragma unroll
-      for (int dt = 0; dt < DTILES; ++dt) {
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[0][dt], pf0, o[dt], 0, 0, 0);
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[1][dt], pf1, o[dt], 0, 0, 0);
-      }
-      if (!EARLY && kb_next < k_end) {
-        int p0, p1;
-        pages_of(kb_next, p0, p1);
-        load_keys(p0, p1, kf[j]);
-        load_vals(p0, p1, vf[j]);
-      }
+    for (int dt = 0; dt < DTILES; ++dt) {
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[0][dt], pf0, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[1][dt], pf1, o[dt], 0, 0, 0);
+    }
+    if (!EARLY && has_next) {
+      int p0, p1;
+      pages_of(kb + STRIDE, p0, p1);
+      load_keys(p0, p1, kf);
+      load_vals(p0, p1, vf);
+    }
+  }
+
+  if constexpr (KSPLIT > 1) {
+    // Merge the shares of a task: the waves with part > 0 lay down (m, l, o), lane by lane; the wave with part 0
+    // rescales all to the common maximum and adds them in order.  Same lanes hold the same (row, column) in all.
+    constexpr int PER_LANE = DTILES * 16 + 2;
+    __shared__ float merge[(KSPLIT - 1) * 4 * PER_LANE * 64];
+    if (part > 0) {
+      float* dst = merge + (size_t)((part - 1) * 4 + slot) * PER_LANE * 64 + lane;
+      dst[0] = m;
+      dst[64] = l;
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[(2 + dt * 16 + i) * 64] = o[dt][i];
+    }
+    __syncthreads();
+    if (part > 0 || !has_task) return;
+#pragma unroll
+    for (int h = 1; h < KSPLIT; ++h) {
+      const float* src = merge + (size_t)((h - 1) * 4 + slot) * PER_LANE * 64 + lane;
+      const float m2 = src[0], l2 = src[64];
+      const float m_all = fmaxf(m, m2);
+      const float m_use = (m_all == -INFINITY) ? 0.f : m_all;
+      const float a = __builtin_amdgcn_exp2f(m - m_use), b2 = __builtin_amdgcn_exp2f(m2 - m_use);
+      l = l * a + l2 * b2;
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[dt][i] = o[dt][i] * a + src[(2 + dt * 16 + i) * 64] * b2;
+      m = m_all;
     }
   }
 
@@ -401,21 +432,34 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
   }
 }
 
+// two waves per task need (DTILES * 16 + 2) floats per lane of four waves in LDS
+constexpr bool kSplitFits = (DTILES * 16 + 2) * 64 * 4 * sizeof(float) <= 65536;
+
 extern "C" int atoma_attention_mfma_head_size() { return HD; }
+extern "C" int atoma_attention_mfma_max_ksplit() { return kSplitFits ? 2 : 1; }
 
 // tasks: device array of n_tasks Task records (main kernel), followed by n_combine records for the combine kernel.
 extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kcache, const void* vcache, void* out,
                                     int out_stride, float* part_o, float* part_lse, const int32_t* tasks, int n_tasks,
                                     int n_combine, const int32_t* block_tables, int max_blocks, float scale,
-                                    int window, int nh, int nkv, hipStream_t stream) {
+                                    int window, int nh, int nkv, int ksplit, hipStream_t stream) {
   if (n_tasks <= 0) return 0;
   if (nkv <= 0 || nh % nkv || nkv > 65535 || max_blocks <= 0 || (q_stride & 7) || (out_stride & 3) ||
       ((uintptr_t)q & 15) || ((uintptr_t)out & 7))
     return ATOMA_ERR_SHAPE;
   const Task* t = reinterpret_cast<const Task*>(tasks);
-  hipLaunchKernelGGL(attention_mfma_kernel<1>, dim3((n_tasks + 3) / 4, nkv), dim3(256), 0, stream,
-                     (const uint16_t*)q, q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out,
-                     out_stride, part_o, part_lse, t, n_tasks, block_tables, max_blocks, scale, window, nh, nkv);
+  // ksplit: waves that share a task's keys (1, or 2 for head sizes whose merge fits in LDS)
+  const dim3 grid(((n_tasks + 3) / 4) * nkv);
+  if (ksplit == 1)
+    hipLaunchKernelGGL(attention_mfma_kernel<1>, grid, dim3(256), 0, stream, (const uint16_t*)q, q_stride,
+                       (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride, part_o, part_lse,
+                       t, n_tasks, block_tables, max_blocks, scale, window, nh, nkv);
+  else if (ksplit == 2 && kSplitFits)
+    hipLaunchKernelGGL(attention_mfma_kernel<kSplitFits ? 2 : 1>, grid, dim3(512), 0, stream, (const uint16_t*)q,
+                       q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride, part_o,
+                       part_lse, t, n_tasks, block_tables, max_blocks, scale, window, nh, nkv);
+  else
+    return ATOMA_ERR_SHAPE;
   ATOMA_LAUNCH_CHECK();
   if (n_combine > 0) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(n_combine, nkv), dim3(256), 0, stream, part_o, part_lse,

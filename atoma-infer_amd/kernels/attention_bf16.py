@@ -25,6 +25,7 @@ CHUNK = 256          # keys per partial task, at most; fewer when few requests a
 MAX_SPLIT_TASKS = 1024
 SPLIT_MAX_TOKENS = 16  # entries with at most this many tokens may be split along the keys
 SPLIT_MIN_KEYS = 2 * CHUNK
+SPLIT_WAVES_MIN_KEYS = 128   # a task of at least this many keys is walked by two waves, every other block each
 _libs: Dict[int, ctypes.CDLL] = {}
 
 
@@ -114,7 +115,8 @@ def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, windo
 
 def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket: Optional[int] = None,
                 vectorized: bool = True) -> Tuple[np.ndarray, Tuple[int, int, int]]:
-    """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials).
+    """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials, keys of
+    the longest task that is not a chunk).
 
     Main tasks are padded to a multiple of 4 (one workgroup runs 4) and ordered so that tasks sharing keys are
     neighbours and long tasks come first.  With ``bucket`` (decode graphs: one token per entry) every entry is
@@ -183,7 +185,8 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
         split.append(null)
     rest = np.asarray(split + combine, dtype=np.int32).reshape(-1, 12)
     arr = np.concatenate([head, rest])
-    return arr, (len(head) + len(split), len(combine), n_part)
+    longest = int((head[:, 5] - head[:, 4]).max()) if len(head) else 0
+    return arr, (len(head) + len(split), len(combine), n_part, longest)
 
 
 def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int):
@@ -228,7 +231,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     comb[..., 9] = 1
     comb[..., 10] = starts[:, None]
     arr = np.concatenate([main, comb.reshape(-1, 12)])
-    return arr, (len(main), s * row_chunks, s * row_chunks * slots)
+    return arr, (len(main), s * row_chunks, s * row_chunks * slots, 0)
 
 
 def plan_key(group: int, window: int):
@@ -253,7 +256,9 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
             arr, meta = build_tasks(ctx.h_starts, ctx.h_counts, group, window)
             plan = (torch.from_numpy(arr).to(q.device), meta)
             ctx.scratch[key] = plan
-    tasks, (n_main, n_comb, n_part) = plan
+    tasks, (n_main, n_comb, n_part, longest) = plan
+    # tasks that walk many keys (prompt tiles) get two waves each
+    ksplit = 2 if longest >= SPLIT_WAVES_MIN_KEYS and lib(hd).atoma_attention_mfma_max_ksplit() >= 2 else 1
     part_o = part_lse = None
     if n_part:
         ws_key = ("attention_partials", nkv, hd)
@@ -266,5 +271,6 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
     bt = cache.block_tables
     _check(lib(hd).atoma_attention_mfma(_p(q), q.stride(0), _p(k_cache), _p(v_cache), _p(out), out.stride(0),
                                         _p(part_o), _p(part_lse), _p(tasks), n_main, n_comb, _p(bt), bt.shape[1],
-                                        ctypes.c_float(scale), int(window), nh, nkv, _stream()), "attention_mfma")
+                                        ctypes.c_float(scale), int(window), nh, nkv, ksplit, _stream()),
+           "attention_mfma")
     return True
