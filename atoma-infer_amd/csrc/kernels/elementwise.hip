@@ -403,11 +403,43 @@ swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int 
   }
 }
 
+// eight bfloat16 values per thread (16-byte loads and stores); needs inter % 8 == 0 and 16-byte aligned rows
+__global__ void __launch_bounds__(256)
+swiglu_vec8_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ out, int inter, int n_tokens, int block) {
+  const int octs = inter >> 3;
+  const size_t total = (size_t)n_tokens * octs;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
+    const size_t t = idx / octs;
+    const int i = (int)(idx % octs) * 8;
+    const uint4 graw = *reinterpret_cast<const uint4*>(gu + t * 2 * inter + gate_index(i, block));
+    const uint4 uraw = *reinterpret_cast<const uint4*>(gu + t * 2 * inter + up_index(i, inter, block));
+    const uint16_t* g = reinterpret_cast<const uint16_t*>(&graw);
+    const uint16_t* u = reinterpret_cast<const uint16_t*>(&uraw);
+    uint4 oraw;
+    uint16_t* o = reinterpret_cast<uint16_t*>(&oraw);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gv = bf16_bits_to_f32(g[e]);
+      o[e] = f32_to_bf16_bits(gv / (1.0f + expf(-gv)) * bf16_bits_to_f32(u[e]));
+    }
+    *reinterpret_cast<uint4*>(out + t * inter + i) = oraw;
+  }
+}
+
 extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, int block,
                             hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (block != 0 && (block != 16 || inter % 16)) return ATOMA_ERR_SHAPE;
   const size_t total = (size_t)n_tokens * inter;
+  if (dtype == kBF16 && inter % 8 == 0 && ((uintptr_t)gu & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    size_t octs = total / 8;
+    int vb = (int)((octs + 255) / 256);
+    if (vb > 16384) vb = 16384;
+    hipLaunchKernelGGL(swiglu_vec8_kernel, dim3(vb), dim3(256), 0, stream, (const uint16_t*)gu, (uint16_t*)out, inter,
+                       n_tokens, block);
+    ATOMA_LAUNCH_CHECK();
+    return 0;
+  }
   if (inter % 4 == 0 && ((uintptr_t)gu & 15) == 0 && ((uintptr_t)out & 15) == 0) {
     size_t quads = total / 4;
     int vb = (int)((quads + 255) / 256);

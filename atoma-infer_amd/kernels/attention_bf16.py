@@ -26,6 +26,7 @@ MAX_SPLIT_TASKS = 1024
 SPLIT_MAX_TOKENS = 16  # entries with at most this many tokens may be split along the keys
 SPLIT_MIN_KEYS = 2 * CHUNK
 SPLIT_WAVES_MIN_KEYS = 128   # a task of at least this many keys is walked by two waves, every other block each
+CHUNK_WAVES = 1              # waves per chunk of a decode step
 _libs: Dict[int, ctypes.CDLL] = {}
 
 
@@ -258,7 +259,8 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
             ctx.scratch[key] = plan
     tasks, (n_main, n_comb, n_part, longest) = plan
     # tasks that walk many keys (prompt tiles) get two waves each
-    ksplit = 2 if longest >= SPLIT_WAVES_MIN_KEYS and lib(hd).atoma_attention_mfma_max_ksplit() >= 2 else 1
+    ksplit = 2 if longest >= SPLIT_WAVES_MIN_KEYS else CHUNK_WAVES
+    ksplit = min(ksplit, lib(hd).atoma_attention_mfma_max_ksplit())
     part_o = part_lse = None
     if n_part:
         ws_key = ("attention_partials", nkv, hd)

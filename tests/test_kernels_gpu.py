@@ -67,7 +67,7 @@ def test_rmsnorm_properties():
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("inter", [10, 250, 1024])
+@pytest.mark.parametrize("inter", [10, 100, 250, 1024])
 def test_swiglu(dt, inter):
     from atoma_infer_amd.kernels import ops
     gu = rnd(5, 2 * inter, dtype=dt, seed=4, scale=3.0)
