@@ -361,7 +361,7 @@ static int launch_rope_mt(const void* a, const void* w, void* c, int M, int N, i
   return ATOMA_ERR_SHAPE;
 }
 
-// The fused q, k, v projection of at most 32 rows with rotary encoding and the cache write in its epilogue.
+// The fused q, k, v projection of at most 64 rows with rotary encoding and the cache write in its epilogue.
 // w [(nh + 2 nkv) hd, K] with the rows of q and k heads in pair order (pair i: rows 2i, 2i + 1 of the head);
 // c [M, ldc >= nh hd] receives the rotated q in its own column order; rotated k and v go to the rows' slots of
 // the caches ([pages, nkv, page_size * hd] bfloat16 tiles).  hd % 4 == 0 (then hd / 2 is even and 4-byte stores
@@ -373,12 +373,16 @@ extern "C" int atoma_gemm_bf16_skinny_rope(const void* a, const void* w, void* c
                                            hipStream_t stream) {
   if (M <= 0) return 0;
   const int N = (nh + 2 * nkv) * hd;
-  if (M > 32 || K <= 0 || wk <= 0 || K % (32 * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K ||
+  if (M > 64 || K <= 0 || wk <= 0 || K % (32 * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K ||
       ldc < nh * hd || (ldc & 1) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)c & 3) || (hd & 3) ||
       nh <= 0 || nkv <= 0 || page_size <= 0 || !positions || !cos_t || !sin_t || !kcache || !vcache ||
       !slot_mapping || ((uintptr_t)kcache & 3))
     return ATOMA_ERR_SHAPE;
   const RopeArgs ra{positions, cos_t, sin_t, (uint16_t*)kcache, (uint16_t*)vcache, slot_mapping, page_size, nh, nkv, hd};
-  if (M <= 16) return launch_rope_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
-  return launch_rope_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
+  switch ((M + 15) / 16) {
+    case 1: return launch_rope_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
+    case 2: return launch_rope_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
+    case 3: return launch_rope_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
+    default: return launch_rope_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
+  }
 }

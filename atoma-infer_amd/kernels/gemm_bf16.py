@@ -165,7 +165,7 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
     return out
 
 
-ROPE_MAX_M = 32
+ROPE_MAX_M = SKINNY_MAX_M
 
 
 def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,

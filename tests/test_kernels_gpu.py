@@ -453,7 +453,7 @@ def test_gemm_with_swiglu_epilogue(m, inter, k):
     assert gemm_bf16.try_linear_swiglu(rnd(40, k, dtype=torch.bfloat16), interleave16(wg, wu)) is None   # too many rows
 
 
-@pytest.mark.parametrize("m", [1, 8, 16, 23])
+@pytest.mark.parametrize("m", [1, 8, 16, 23, 40, 64])
 @pytest.mark.parametrize("nh,nkv,hd,k", [(8, 2, 64, 256), (3, 1, 16, 64), (32, 8, 64, 2048), (5, 5, 48, 96)])
 def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
     """The q, k, v projection that rotates and stores in its epilogue against product, rotation and store done
@@ -462,7 +462,7 @@ def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
     from atoma_infer_amd.cache.layout import pack_keys, pack_values
     page, pages = 16, 6
     n = (nh + 2 * nkv) * hd
-    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)   # (96 slots: enough for 64 rows)
     w = rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.2)
     g = torch.Generator().manual_seed(5)
     pos = torch.randint(0, 90, (m,), generator=g).int().to(DEV)
@@ -495,5 +495,5 @@ def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
     kc0, vc0 = caches()
     same = (kc1 == kc0)
     assert int((~same).sum()) <= (m - (1 if m > 2 else 0)) * nkv * hd
-    assert gemm_bf16.try_linear_rope(rnd(40, k, dtype=torch.bfloat16), w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv,
+    assert gemm_bf16.try_linear_rope(rnd(70, k, dtype=torch.bfloat16), w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv,
                                      hd) is None   # too many rows
