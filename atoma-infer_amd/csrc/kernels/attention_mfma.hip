@@ -34,6 +34,7 @@ constexpr int KSTEPS = HD / 16;        // MFMA steps over the head dimension for
 constexpr int DTILES = (HD + 31) / 32; // 32-row tiles of O^T
 constexpr int PAGE = 16;
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kSlack = 8.0f;   // see the softmax in the kernel
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -236,19 +237,14 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       }
     }
     bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64)) * sc2;
+    // The reference point m of a row's exponentials follows its maximum only in jumps: as long as no row of the
+    // wave has grown by more than kSlack (in powers of two) beyond its m, m stays, the weights may exceed one (by
+    // at most 2^kSlack, nothing to float32 sums or to bfloat16 weights, whose precision is relative) and the
+    // accumulators need no rescaling, which is most of a block's vector work.  out = o / l does not depend on m.
     const float m_new = fmaxf(m, bmax);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
-      psum += sv[i];
-    }
-    psum += __shfl_xor(psum, 32, 64);
-    // the accumulators are rescaled only when some row's maximum has grown (a wave-uniform decision)
-    const bool grew = __ballot(m_new > m) != 0;
+    const bool grew = __ballot(m_new > m + kSlack) != 0;    // (-inf + kSlack = -inf: a row's first key always counts)
     if (grew) {
-      const float corr = __builtin_amdgcn_exp2f(m - m_use);
+      const float corr = __builtin_amdgcn_exp2f(m - ((m_new == -INFINITY) ? 0.f : m_new));
       l *= corr;
 #pragma unroll
       for (int dt = 0; dt < DTILES; ++dt)
@@ -256,6 +252,14 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
         for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
       m = m_new;
     }
+    const float m_use = (m == -INFINITY) ? 0.f : m;
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
+      psum += sv[i];
+    }
+    psum += __shfl_xor(psum, 32, 64);
     l += psum;
 
     // O^T += V^T P^T
