@@ -55,6 +55,12 @@ struct Task {
   int32_t pad;
 };
 
+// x of the lane 32 away, by one cross-half register swap (no trip through LDS as a shuffle would take)
+__device__ __forceinline__ float from_other_half(float x, bool upper) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(upper ? r[0] : r[1]);
+}
+
 __device__ __forceinline__ bf16x8 pack8(const float* v) {
   bf16x8 r;
 #pragma unroll
@@ -236,7 +242,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
         bmax = fmaxf(bmax, sv[i]);
       }
     }
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64)) * sc2;
+    bmax = fmaxf(bmax, from_other_half(bmax, hg != 0)) * sc2;
     // The reference point m of a row's exponentials follows its maximum only in jumps: as long as no row of the
     // wave has grown by more than kSlack (in powers of two) beyond its m, m stays, the weights may exceed one (by
     // at most 2^kSlack, nothing to float32 sums or to bfloat16 weights, whose precision is relative) and the
@@ -259,7 +265,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
       psum += sv[i];
     }
-    psum += __shfl_xor(psum, 32, 64);
+    psum += from_other_half(psum, hg != 0);
     l += psum;
 
     // O^T += V^T P^T
