@@ -260,40 +260,33 @@ rope_cache_write_kernel(TA* __restrict__ qkv, int row_stride, const int32_t* __r
 
 // The same for bfloat16 rows and caches with hd % 16 == 0, the whole head rotated and 16-byte aligned rows: a
 // thread takes eight neighbouring pairs of a q or k head (two 16-byte loads, and since eight columns of a key are
-// one piece of its cache tile, two 16-byte stores) or eight columns of a v head.  One block per token.
+// one piece of its cache tile, two 16-byte stores).  One block per four tokens: a value tile keeps four
+// neighbouring tokens of a column side by side, so when the block's tokens fill four neighbouring slots of a
+// page (as a prompt's do), a thread turns four columns of the four tokens into four 8-byte stores.
+constexpr int kRopeTokens = 4;
+
 __global__ void __launch_bounds__(256)
 rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const int32_t* __restrict__ positions,
                             const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                             uint16_t* __restrict__ kcache, uint16_t* __restrict__ vcache,
                             const int32_t* __restrict__ slot_mapping, int page_size, int nh, int nkv, int hd,
-                            uint16_t* __restrict__ q_out, int q_stride) {
-  const int t = blockIdx.x;
+                            uint16_t* __restrict__ q_out, int q_stride, int n_tokens) {
+  const int t0 = blockIdx.x * kRopeTokens;
+  const int nt = n_tokens - t0 < kRopeTokens ? n_tokens - t0 : kRopeTokens;
   const int half = hd >> 1;
-  const int per_qk = hd >> 4, per_v = hd >> 3;             // items per head
+  const int per_qk = hd >> 4;                              // items per head
   const int n_qk = (nh + nkv) * per_qk;
-  const int n_items = n_qk + (kcache ? nkv * per_v : 0);
-  const int slot = (kcache && slot_mapping) ? slot_mapping[t] : -1;
-  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
-  uint16_t* row = qkv + (size_t)t * row_stride;
-  const size_t pos = (size_t)positions[t];
-  for (int item = threadIdx.x; item < n_items; item += 256) {
-    if (item >= n_qk) {
-      if (slot < 0) continue;
-      const int head = (item - n_qk) / per_v, d0 = ((item - n_qk) % per_v) * 8;
-      const uint4 raw = *reinterpret_cast<const uint4*>(row + (size_t)(nh + nkv + head) * hd + d0);
-      const uint16_t* v = reinterpret_cast<const uint16_t*>(&raw);
-      uint16_t* tile = vcache + ((size_t)page * nkv + head) * hd * page_size;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) tile[value_offset(d0 + e, off, hd, page_size)] = v[e];
-      continue;
-    }
-    const int head = item / per_qk, i0 = (item % per_qk) * 8;
+  const bool paired = q_out != nullptr;
+  for (int item = threadIdx.x; item < nt * n_qk; item += 256) {
+    const int t = t0 + item / n_qk, it = item % n_qk;
+    const int head = it / per_qk, i0 = (it % per_qk) * 8;
     const bool is_k = head >= nh;
-    if (is_k && (!kcache || slot < 0)) continue;
-    uint16_t* x = row + (size_t)head * hd;
+    const int slot = (kcache && slot_mapping) ? slot_mapping[t] : -1;
+    if (is_k && slot < 0) continue;
+    uint16_t* x = qkv + (size_t)t * row_stride + (size_t)head * hd;
+    const size_t pos = (size_t)positions[t];
     // where the eight pairs' members come from: columns i0.. and i0 + half.. (one member in each 16-byte piece), or,
     // with q_out, neighbours 2 i0 .. 2 i0 + 15 (four pairs in each piece); they leave to columns i0.. and i0 + half..
-    const bool paired = q_out != nullptr;
     const uint4 r1 = *reinterpret_cast<const uint4*>(x + (paired ? 2 * i0 : i0));
     const uint4 r2 = *reinterpret_cast<const uint4*>(x + (paired ? 2 * i0 + 8 : i0 + half));
     const f4 c0 = load4(cos_t + pos * half + i0), c1 = load4(cos_t + pos * half + i0 + 4);
@@ -313,6 +306,7 @@ rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const in
       o2[e] = f32_to_bf16_bits(x2 * c + x1 * sn);
     }
     if (is_k) {
+      const int page = slot / page_size, off = slot % page_size;
       uint16_t* ktile = kcache + ((size_t)page * nkv + (head - nh)) * page_size * hd;
       *reinterpret_cast<uint4*>(ktile + key_offset(off, i0, page_size)) = w1;
       *reinterpret_cast<uint4*>(ktile + key_offset(off, i0 + half, page_size)) = w2;
@@ -320,6 +314,49 @@ rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const in
       uint16_t* y = paired ? q_out + (size_t)t * q_stride + (size_t)head * hd : x;
       *reinterpret_cast<uint4*>(y + i0) = w1;
       *reinterpret_cast<uint4*>(y + i0 + half) = w2;
+    }
+  }
+  if (!kcache || !slot_mapping) return;
+
+  // values: four columns of the block's tokens per thread
+  int slots[kRopeTokens];
+#pragma unroll
+  for (int j = 0; j < kRopeTokens; ++j) slots[j] = j < nt ? slot_mapping[t0 + j] : -1;
+  const int off0 = slots[0] >= 0 ? slots[0] % page_size : 0;
+  const bool together = nt == kRopeTokens && slots[0] >= 0 && (off0 & 3) == 0 && (page_size & 3) == 0 &&
+                        slots[1] == slots[0] + 1 &&
+                        slots[2] == slots[0] + 2 && slots[3] == slots[0] + 3;    // (then all in one page)
+  const int quads = hd >> 2;
+  for (int item = threadIdx.x; item < nkv * quads; item += 256) {
+    const int head = item / quads, d0 = (item % quads) * 4;
+    uint2 raw[kRopeTokens];
+#pragma unroll
+    for (int j = 0; j < kRopeTokens; ++j)
+      if (j < nt)
+        raw[j] = *reinterpret_cast<const uint2*>(qkv + (size_t)(t0 + j) * row_stride + (size_t)(nh + nkv + head) * hd + d0);
+    if (together) {
+      uint16_t* tile = vcache + ((size_t)(slots[0] / page_size) * nkv + head) * hd * page_size;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        // column d0 + e of the four tokens: 16 bits out of each token's 8 bytes
+        uint2 col;
+        const uint32_t v0 = ((e < 2 ? raw[0].x : raw[0].y) >> ((e & 1) * 16)) & 0xffffu;
+        const uint32_t v1 = ((e < 2 ? raw[1].x : raw[1].y) >> ((e & 1) * 16)) & 0xffffu;
+        const uint32_t v2 = ((e < 2 ? raw[2].x : raw[2].y) >> ((e & 1) * 16)) & 0xffffu;
+        const uint32_t v3 = ((e < 2 ? raw[3].x : raw[3].y) >> ((e & 1) * 16)) & 0xffffu;
+        col.x = v0 | (v1 << 16);
+        col.y = v2 | (v3 << 16);
+        *reinterpret_cast<uint2*>(tile + value_offset(d0 + e, off0, hd, page_size)) = col;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kRopeTokens; ++j) {
+        if (j >= nt || slots[j] < 0) continue;
+        uint16_t* tile = vcache + ((size_t)(slots[j] / page_size) * nkv + head) * hd * page_size;
+        const uint16_t* v = reinterpret_cast<const uint16_t*>(&raw[j]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) tile[value_offset(d0 + e, slots[j] % page_size, hd, page_size)] = v[e];
+      }
     }
   }
 }
@@ -340,12 +377,13 @@ extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, 
   if (hd & 1) return ATOMA_ERR_SHAPE;
   // few tokens (decode steps) are quicker with many small blocks; measured on MI355X
   if (n_tokens >= 32 && act_dtype == kBF16 && cache_dtype == kBF16 && cos_t && sin_t && rotary_dim == hd && hd % 16 == 0 &&
-      row_stride % 8 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)kcache & 15) == 0 && q_stride % 8 == 0 &&
+      row_stride % 8 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 7) == 0 &&
+      q_stride % 8 == 0 &&
       ((uintptr_t)q_out & 15) == 0 &&
       ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0) {
-    hipLaunchKernelGGL(rope_cache_write_vec_kernel, dim3(n_tokens), dim3(256), 0, stream, (uint16_t*)qkv, row_stride,
-                       positions, cos_t, sin_t, (uint16_t*)kcache, (uint16_t*)vcache, slot_mapping, page_size, nh,
-                       nkv, hd, (uint16_t*)q_out, q_stride);
+    hipLaunchKernelGGL(rope_cache_write_vec_kernel, dim3((n_tokens + kRopeTokens - 1) / kRopeTokens), dim3(256), 0,
+                       stream, (uint16_t*)qkv, row_stride, positions, cos_t, sin_t, (uint16_t*)kcache,
+                       (uint16_t*)vcache, slot_mapping, page_size, nh, nkv, hd, (uint16_t*)q_out, q_stride, n_tokens);
     ATOMA_LAUNCH_CHECK();
     return 0;
   }
