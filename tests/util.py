@@ -31,8 +31,19 @@ TINY_C = {
     "num_attention_heads": 4, "num_key_value_heads": 2, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
     "max_position_embeddings": 512, "tie_word_embeddings": True,
 }
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-NORM_JITTER = {"A": 0.0, "B": 0.1, "C": 0.1}
+# the serving shape in small: heads of 64 in groups of four over two KV heads, sizes that take every fused bfloat16
+# kernel (products with rotary and SiLU epilogues, K-split planes), llama3 scaling as Llama 3.2 has it, and room
+# for contexts long enough that a decoded token's keys are split into chunks and merged
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 512, "intermediate_size": 1024, "vocab_size": 2003, "num_hidden_layers": 2,
+    "num_attention_heads": 8, "num_key_value_heads": 2, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192, "rope_type": "llama3"},
+    "max_position_embeddings": 2048, "tie_word_embeddings": True,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+NORM_JITTER = {"A": 0.0, "B": 0.1, "C": 0.1, "D": 0.1}
 
 
 def make_model_dir(path: str, cfg: dict, seed: int, dtype: str, norm_jitter: float = 0.0) -> str:
