@@ -74,6 +74,7 @@ class LlmEngine:
         self._requests: Dict[str, Request] = {}
         self.tokenizer = None
         self._in_flight: Optional[_InFlight] = None
+        self._undelivered: List[GenerateRequestOutput] = []     # finished while aborting another request
         self.stats = {"steps": 0, "tokens": 0, "sampled": 0, "preemptions": 0}
 
     # -- construction from the reference's TOML ----------------------------------------------------------
@@ -133,14 +134,16 @@ class LlmEngine:
         return rid
 
     def abort(self, request_id: str) -> Optional[GenerateRequestOutput]:
-        self.drain()
+        """Stop a request wherever it is.  The step in flight is read first; requests that it finished are handed
+        out by the next ``step`` (or ``drain``), the aborted one (if it had not just finished) here."""
+        self._undelivered = self.drain()
         r = self.scheduler.abort(request_id)
         if r is None:
             return None
         return self._output(r)
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_unfinished() or self._in_flight is not None
+        return self.scheduler.has_unfinished() or self._in_flight is not None or bool(self._undelivered)
 
     # -- one step ------------------------------------------------------------------------------------------
     def step(self) -> List[GenerateRequestOutput]:
@@ -164,7 +167,7 @@ class LlmEngine:
         if launched is not None and launched.sync:
             finished += self._resolve(launched)
             self._in_flight = None
-        outs = []
+        outs, self._undelivered = self._undelivered, []
         for r in finished:
             r.metrics.finished_time = time.monotonic()
             outs.append(self._output(r))
@@ -223,7 +226,7 @@ class LlmEngine:
 
     def drain(self) -> List[GenerateRequestOutput]:
         """Read what is still in flight (call before reading clocks or state from outside)."""
-        outs = []
+        outs, self._undelivered = self._undelivered, []
         if self._in_flight is not None:
             for r in self._resolve(self._in_flight):
                 r.metrics.finished_time = time.monotonic()

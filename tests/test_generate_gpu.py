@@ -334,3 +334,30 @@ max_total_tokens = 64
                           cwd=ROOT)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert json.loads(proc.stdout.strip().splitlines()[-1])["inference_outputs"][0]["token_ids"] == want
+
+
+def test_abort_loses_no_other_request(model_dirs):
+    """Aborting reads the step in flight; what that step finished must still be handed out."""
+    from atoma_infer_amd.sampling import GenerateParameters
+    d = model_dirs["A"]
+    w, cfg = plain_weights(d), plain_config(d)
+    prompts = [random_tokens(5, 512, 21), random_tokens(7, 512, 22), random_tokens(6, 512, 23)]
+    for steps_before in (1, 2, 3, 4):
+        eng = engine(d, "float32", 4, 32)
+        short = GenerateParameters(do_sample=False, max_new_tokens=3, ignore_eos_token=True)
+        ids = [eng.add_request(prompts[0], short), eng.add_request(prompts[1], short),
+               eng.add_request(prompts[2], GenerateParameters(do_sample=False, max_new_tokens=30, ignore_eos_token=True))]
+        seen = []
+        for _ in range(steps_before):
+            seen += eng.step()
+        gone = eng.abort(ids[2])
+        assert gone is not None and gone.request_id == ids[2]
+        assert gone.inference_outputs[0].token_ids == plain_llama.greedy_generate(
+            prompts[2], 30, w, cfg)[:len(gone.inference_outputs[0].token_ids)]
+        while eng.has_unfinished():
+            seen += eng.step()
+        assert sorted(o.request_id for o in seen) == sorted(ids[:2])
+        for o in seen:
+            want = plain_llama.greedy_generate(prompts[ids.index(o.request_id)], 3, w, cfg)
+            assert o.inference_outputs[0].token_ids == want
+        assert eng.runner.manager.num_requests() == 0 and eng.runner.manager.num_free_pages() == 32
