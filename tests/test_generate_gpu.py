@@ -361,3 +361,46 @@ def test_abort_loses_no_other_request(model_dirs):
             want = plain_llama.greedy_generate(prompts[ids.index(o.request_id)], 3, w, cfg)
             assert o.inference_outputs[0].token_ids == want
         assert eng.runner.manager.num_requests() == 0 and eng.runner.manager.num_free_pages() == 32
+
+
+def test_text_in_and_out_with_a_tokenizer(model_dirs, tmp_path):
+    """With tokenizer.json in the model folder prompts may be text, outputs carry text, ``stop`` strings end a
+    request at the piece that equals one of them, ``truncate`` keeps the end of the prompt's text and
+    ``return_full_text`` puts the prompt before the output."""
+    import shutil
+    from tokenizers import Tokenizer, models, pre_tokenizers, decoders
+    from atoma_infer_amd.config import CacheConfig, SchedulerConfig
+    from atoma_infer_amd.engine.engine import LlmEngine
+    from atoma_infer_amd.sampling import GenerateParameters
+    d = str(tmp_path / "model")
+    shutil.copytree(model_dirs["A"], d)
+    vocab = {f"w{i}": i for i in range(512)}
+    tok = Tokenizer(models.WordLevel(vocab, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.save(os.path.join(d, "tokenizer.json"))
+    w, cfg = plain_weights(d), plain_config(d)
+    eng = LlmEngine(d, "float32", cache=CacheConfig(block_size=4, num_gpu_blocks_override=32),
+                    scheduler=SchedulerConfig(max_num_batched_tokens=64, max_num_sequences=4, max_model_len=128))
+    assert eng.load_tokenizer(d)
+    eng.eos_ids = set()
+    ids = [5, 17, 3, 250]
+    text = " ".join(f"w{i}" for i in ids)
+    free = plain_llama.greedy_generate(ids, 8, w, cfg)
+    out = eng.generate([text], GenerateParameters(do_sample=False, max_new_tokens=8, ignore_eos_token=True))[0]
+    assert out.prompt == text and out.prompt_token_ids == ids
+    assert out.inference_outputs[0].token_ids == free
+    assert out.inference_outputs[0].output_text == tok.decode(free)
+    # a stop string: the piece of the third new token (if it did not occur before)
+    piece = tok.decode([free[2]])
+    cut = next(i for i, t in enumerate(free) if tok.decode([t]) == piece)
+    out = eng.generate([text], GenerateParameters(do_sample=False, max_new_tokens=8, stop=[piece]))[0].inference_outputs[0]
+    assert out.token_ids == free[:cut + 1] and out.finish_reason == "stopped" and out.stop_reason == piece
+    # the prompt before the output
+    out = eng.generate([text], GenerateParameters(do_sample=False, max_new_tokens=3, return_full_text=True,
+                                                  ignore_eos_token=True))[0].inference_outputs[0]
+    assert out.output_text == text + tok.decode(free[:3])
+    # truncate keeps the last characters of the text (the reference cuts text, not tokens: tokenizer.rs:185-206)
+    keep = len("w3 w250")
+    out = eng.generate([text], GenerateParameters(do_sample=False, max_new_tokens=2, truncate=keep, ignore_eos_token=True))[0]
+    assert out.prompt_token_ids == [3, 250]
+    assert out.inference_outputs[0].token_ids == plain_llama.greedy_generate([3, 250], 2, w, cfg)
