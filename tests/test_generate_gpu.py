@@ -404,3 +404,76 @@ def test_text_in_and_out_with_a_tokenizer(model_dirs, tmp_path):
     out = eng.generate([text], GenerateParameters(do_sample=False, max_new_tokens=2, truncate=keep, ignore_eos_token=True))[0]
     assert out.prompt_token_ids == [3, 250]
     assert out.inference_outputs[0].token_ids == plain_llama.greedy_generate([3, 250], 2, w, cfg)
+
+
+def random_trace(rng, requests, max_live=4):
+    """Steps in the replay program's format for the given requests: up to four live, portions of random sizes down
+    to two tokens beside single tokens, requests that sit out steps, random wanted places (also none).  Returns
+    (steps, the most tokens live at a time with every request rounded up to 64)."""
+    waiting, live, done, steps, peak = list(requests), [], {k: 0 for k in requests}, [], 0
+    while waiting or live:
+        while waiting and len(live) < max_live and (rng.random() < 0.6 or not live):
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for k in live:
+            left = len(requests[k]) - done[k]
+            if rng.random() < 0.2 and len(live) > 1:
+                continue
+            mode = rng.random()
+            if left <= rng.randint(1, 10) or mode < 0.3:
+                n = 1
+            elif mode < 0.5:
+                n = min(2, left)
+            else:
+                n = min(rng.choice([2, 3, 7, 16, 17, 31, 64, 100]), left)
+            want = sorted(rng.sample(range(n), rng.randint(0, min(n, 3))))
+            entries.append({"id": k, "tokens": requests[k][done[k]:done[k] + n], "want": want})
+            done[k] += n
+            if done[k] == len(requests[k]):
+                end.append(k)
+        if not entries:
+            continue
+        rng.shuffle(entries)
+        peak = max(peak, sum(-(-done[k] // 64) * 64 for k in live))
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+        live = [k for k in live if k not in end]
+    return steps, peak
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,seed", [("A", 0), ("B", 1), ("C", 2), ("D", 3), ("D", 4)])
+def test_random_traces_replay_like_the_plain_model(model_dirs, tmp_path, name, seed, dtype):
+    import io
+    import random
+    from atoma_infer_amd.engine.replay import make_runner, replay
+    rng = random.Random(seed)
+    cfg = TINY[name]
+    vocab = cfg["vocab_size"]
+    longest = 400 if name == "D" else min(cfg["max_position_embeddings"], 120)
+    requests = {f"q{i}": random_tokens(rng.randint(1, longest), vocab, 900 * seed + i) for i in range(rng.randint(3, 7))}
+    steps, peak = random_trace(rng, requests)
+    runner = make_runner(model_dirs[name], dtype, peak)
+    report = io.StringIO()
+    assert replay(runner, io.StringIO("\n".join(json.dumps(s) for s in steps) + "\n"), str(tmp_path), report) == 0
+    assert report.getvalue().split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+    w, c = plain_weights(model_dirs[name]), plain_config(model_dirs[name])
+    want = {k: plain_llama.forward(v, w, c) for k, v in requests.items()}
+    pos = {k: 0 for k in requests}
+    for s in steps:
+        n_want = sum(len(e["want"]) for e in s["entries"])
+        path = tmp_path / f"{s['step']}.f32"
+        assert path.exists() == (n_want > 0)
+        if n_want:
+            got = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(n_want, vocab))
+            row = 0
+            for e in s["entries"]:
+                for i in e["want"]:
+                    ref = want[e["id"]][pos[e["id"]] + i]
+                    if dtype == "float32":
+                        assert rel_err(got[row], ref) < TOL_F32, (s["step"], e["id"], i)
+                    else:
+                        assert frob_err(got[row], ref) < 2.5 * TOL_BF16, (s["step"], e["id"], i)
+                    row += 1
+        for e in s["entries"]:
+            pos[e["id"]] += len(e["tokens"])
+    assert runner.manager.num_requests() == 0
