@@ -497,3 +497,29 @@ def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
     assert int((~same).sum()) <= (m - (1 if m > 2 else 0)) * nkv * hd
     assert gemm_bf16.try_linear_rope(rnd(70, k, dtype=torch.bfloat16), w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv,
                                      hd) is None   # too many rows
+
+
+@pytest.mark.parametrize("m,n,k,cdt", [(40, 2048, 8192, torch.bfloat16), (64, 16384, 2048, torch.bfloat16),
+                                       (48, 40000, 2048, torch.float32), (64, 3072, 2048, torch.bfloat16)])
+def test_products_replay_in_graphs(m, n, k, cdt):
+    """Decode steps of large batches are captured in HIP graphs together with the library's products.  A captured
+    product must give, on every replay, what an eager call gives for the operand's current content, also with
+    eager work and synchronisations between the replays."""
+    from atoma_infer_amd.kernels import gemm_bf16
+    w = rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    gemm_bf16.try_linear(x, w, cdt)                       # loads every kernel before capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = gemm_bf16.try_linear(x, w, cdt)
+    other = rnd(512, 512, dtype=torch.bfloat16, seed=3)
+    for i in range(6):
+        x.copy_(rnd(m, k, dtype=torch.bfloat16, seed=10 + i))
+        graph.replay()
+        got = y.clone()
+        want = gemm_bf16.try_linear(x, w, cdt)            # eager, between replays
+        assert torch.equal(got, want), f"replay {i}"
+        (other @ other).sum().item()                      # more eager work and a synchronisation
+        if i == 3:
+            torch.cuda.synchronize()
