@@ -12,7 +12,7 @@ from __future__ import annotations
 import dataclasses
 from typing import Any, Dict, Optional, Tuple
 
-from .base import (ConfigError, ModelConfig, as_bool, as_float, as_int, as_positive_int, key, optional,
+from .base import (ConfigError, ModelConfig, as_bool, as_float, as_int, as_positive_int, key,
                    parse_fields)
 
 

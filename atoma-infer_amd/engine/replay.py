@@ -17,7 +17,6 @@ import os
 import sys
 from typing import Dict, IO
 
-import numpy as np
 import torch
 
 from ..cache.pool import CachePool, pages_for_tokens, plan_cache

@@ -10,13 +10,12 @@
 """
 from __future__ import annotations
 
-import ctypes
 from typing import Optional
 
 import torch
 
 from .library import load_hip_module
-from .ops import BF16, F32, KernelError, _check, _p, _stream
+from .ops import BF16, F32, _check, _p, _stream
 
 SKINNY_MAX_M = 64
 LIBRARY_MIN_M_WIDE = 32
@@ -98,7 +97,6 @@ def _library_wins(m: int, n: int, k: int, out_dtype: torch.dtype) -> bool:
 
 def _probe_mm_out_dtype() -> bool:
     """Whether this torch has ``mm(..., out_dtype=float32)`` for bfloat16 operands (float32 accumulation either way)."""
-    import inspect
     doc = getattr(torch.mm, "__doc__", "") or ""
     return "out_dtype" in doc
 
