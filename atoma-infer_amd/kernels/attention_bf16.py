@@ -26,7 +26,6 @@ MAX_SPLIT_TASKS = 1024
 SPLIT_MAX_TOKENS = 16  # entries with at most this many tokens may be split along the keys
 SPLIT_MIN_KEYS = 2 * CHUNK
 SPLIT_WAVES_MIN_KEYS = 128   # a task of at least this many keys is walked by two waves, every other block each
-CHUNK_WAVES = 1              # waves per chunk of a decode step
 _libs: Dict[int, ctypes.CDLL] = {}
 
 
@@ -42,18 +41,21 @@ def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
     return _libs[hd]
 
 
-def chunk_for(n_split: int, max_keys: int) -> int:
-    """Keys per partial task: 128 or 256, the smaller if that keeps the step's partial tasks under a bound.
+def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8) -> Tuple[int, int]:
+    """(keys per partial task, waves that share a task) for the entries of a step that are split along their keys.
 
-    A wave walks its keys one 32-key block after another, so short chunks shorten the chain when few requests
-    decode, and long ones save partial results (and time in the combine kernel) when many do; measured on
-    MI355X, 128 wins up to about 8 requests of 2,000 tokens and 256 beyond.  ``max_keys`` is rounded up to 256.
+    A wave walks its keys one 32-key block after another, so few keys per wave shorten the chain when few requests
+    decode, and long chunks save partial results (and time in the merging kernel) when many do.  Measured on
+    MI355X with 2,000-token contexts and 8 KV heads: one or two requests want 128-key chunks, three to about
+    eleven 256-key chunks walked by two waves each, more requests 256-key chunks with a wave each.  The count that
+    decides is that of 256-key tasks over all KV heads; ``max_keys`` is rounded up to 256.
     """
-    buckets = -(-max_keys // CHUNK)
-    for chunk in (128,):
-        if n_split * buckets * (CHUNK // chunk) <= MAX_SPLIT_TASKS:
-            return chunk
-    return CHUNK
+    tasks = n_split * -(-max_keys // CHUNK) * kv_heads
+    if tasks <= 160:
+        return 128, 1
+    if tasks <= 800:
+        return CHUNK, 2
+    return CHUNK, 1
 
 
 def _live_pieces(rows: int, qt: int, live_tokens: int):
@@ -115,16 +117,16 @@ def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, windo
 
 
 def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket: Optional[int] = None,
-                vectorized: bool = True) -> Tuple[np.ndarray, Tuple[int, int, int]]:
-    """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials, keys of
-    the longest task that is not a chunk).
+                vectorized: bool = True, kv_heads: int = 8) -> Tuple[np.ndarray, Tuple[int, int, int, int]]:
+    """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials, waves that
+    share a task: two when a prompt tile walks many keys, else what ``chunk_for`` says for the split entries).
 
     Main tasks are padded to a multiple of 4 (one workgroup runs 4) and ordered so that tasks sharing keys are
     neighbours and long tasks come first.  With ``bucket`` (decode graphs: one token per entry) every entry is
     split and owns ``bucket`` chunk slots, used or not, so all counts depend on (entries, bucket) alone.
     """
     if vectorized and bucket is not None and len(counts) and int(counts.max()) == 1:
-        return _build_decode_tasks(starts, group, window, bucket)
+        return _build_decode_tasks(starts, group, window, bucket, kv_heads)
     qt_max = max(1, 128 // group)
     null = (-1, 0, 1, 0, 0, 0, -1, 0, 0, 0, 0, 0)
     tok_bases = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
@@ -138,9 +140,10 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
                                       and int(starts[e]) + int(counts[e]) - first_key >= SPLIT_MIN_KEYS)
 
     split_entries = [e for e in range(len(starts)) if splits(e)]
-    chunk = CHUNK
+    chunk, waves = CHUNK, 1
     if split_entries:
-        chunk = chunk_for(len(split_entries), max(int(starts[e]) + int(counts[e]) for e in split_entries))
+        chunk, waves = chunk_for(len(split_entries), max(int(starts[e]) + int(counts[e]) for e in split_entries),
+                                 kv_heads)
     for e in range(len(starts)):
         start, count = int(starts[e]), int(counts[e])
         qt = min(qt_max, count)
@@ -186,17 +189,18 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
         split.append(null)
     rest = np.asarray(split + combine, dtype=np.int32).reshape(-1, 12)
     arr = np.concatenate([head, rest])
-    longest = int((head[:, 5] - head[:, 4]).max()) if len(head) else 0
-    return arr, (len(head) + len(split), len(combine), n_part, longest)
+    if len(head) and int((head[:, 5] - head[:, 4]).max()) >= SPLIT_WAVES_MIN_KEYS:
+        waves = 2
+    return arr, (len(head) + len(split), len(combine), n_part, waves)
 
 
-def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int):
+def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int, kv_heads: int = 8):
     """``build_tasks`` for a step in which every entry brings one token, without a Python loop over entries."""
     s = len(starts)
     starts = starts.astype(np.int64)
     k_end = starts + 1
     lo = np.maximum(0, starts - window + 1) if window > 0 else np.zeros(s, dtype=np.int64)
-    chunk = chunk_for(s, int(k_end.max()))
+    chunk, waves = chunk_for(s, int(k_end.max()), kv_heads)
     slots = bucket * (CHUNK // chunk)
     row_chunks = -(-group // 32)
     c = np.arange(slots, dtype=np.int64)
@@ -232,11 +236,11 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     comb[..., 9] = 1
     comb[..., 10] = starts[:, None]
     arr = np.concatenate([main, comb.reshape(-1, 12)])
-    return arr, (len(main), s * row_chunks, s * row_chunks * slots, 0)
+    return arr, (len(main), s * row_chunks, s * row_chunks * slots, waves)
 
 
-def plan_key(group: int, window: int):
-    return ("attention_mfma_tasks", group, window)
+def plan_key(group: int, window: int, kv_heads: int = 8):
+    return ("attention_mfma_tasks", group, window, kv_heads)
 
 
 def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, hd) -> bool:
@@ -248,19 +252,17 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
     if tuple(k_cache.shape[1:]) != (nkv, PAGE * hd) or tuple(v_cache.shape[1:]) != (nkv, PAGE * hd):
         raise ValueError("cache tensors must be [pages, nkv, page_size * hd] tiles")
     group = nh // nkv
-    plan = getattr(ctx, "plans", {}).get(plan_key(group, window))
+    plan = getattr(ctx, "plans", {}).get(plan_key(group, window, nkv))
     if plan is None:
         # a caller without a step planner (a kernel test): plan here and now
-        key = ("attention_tasks_adhoc", group, window)
+        key = ("attention_tasks_adhoc", group, window, nkv)
         plan = ctx.scratch.get(key)
         if plan is None:
-            arr, meta = build_tasks(ctx.h_starts, ctx.h_counts, group, window)
+            arr, meta = build_tasks(ctx.h_starts, ctx.h_counts, group, window, kv_heads=nkv)
             plan = (torch.from_numpy(arr).to(q.device), meta)
             ctx.scratch[key] = plan
-    tasks, (n_main, n_comb, n_part, longest) = plan
-    # tasks that walk many keys (prompt tiles) get two waves each
-    ksplit = 2 if longest >= SPLIT_WAVES_MIN_KEYS else CHUNK_WAVES
-    ksplit = min(ksplit, lib(hd).atoma_attention_mfma_max_ksplit())
+    tasks, (n_main, n_comb, n_part, waves) = plan
+    ksplit = min(waves, lib(hd).atoma_attention_mfma_max_ksplit())
     part_o = part_lse = None
     if n_part:
         ws_key = ("attention_partials", nkv, hd)

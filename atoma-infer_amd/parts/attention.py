@@ -80,9 +80,10 @@ class PagedAttention(Mixer):
         from ..kernels import attention_bf16
         if cache_dtype is not torch.bfloat16 or page_size != attention_bf16.PAGE:
             return None
-        group, window = self.nh // self.nkv, self.window or 0
-        return (attention_bf16.plan_key(group, window),
-                lambda starts, counts, bucket: attention_bf16.build_tasks(starts, counts, group, window, bucket))
+        group, window, nkv = self.nh // self.nkv, self.window or 0, self.nkv
+        return (attention_bf16.plan_key(group, window, nkv),
+                lambda starts, counts, bucket: attention_bf16.build_tasks(starts, counts, group, window, bucket,
+                                                                          kv_heads=nkv))
 
     # -- execution ------------------------------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:

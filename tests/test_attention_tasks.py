@@ -7,7 +7,8 @@ from atoma_infer_amd.kernels import attention_bf16 as A
 
 
 def coverage(arr, meta, starts, counts, group, window):
-    n_main, n_comb, n_part, _longest = meta
+    n_main, n_comb, n_part, waves = meta
+    assert waves in (1, 2)
     main, comb = arr[:n_main], arr[n_main:]
     assert len(comb) == n_comb and n_main % 4 == 0
     seen = {}          # (entry, token, head) -> list of key ranges, direct
