@@ -72,20 +72,24 @@ __device__ __forceinline__ bf16x8 pack8(const float* v) {
 // range, and the KSPLIT partial results are merged through LDS at the end.  A wave walks its blocks one after the
 // other at a pace set by latencies (MFMA, exponentials, cross-lane moves), not by any unit's throughput, and a
 // launch lasts as long as its longest wave: with two waves per task the last tile of a long prompt, which sees
-// all keys, takes half the time.  Decode steps, whose tasks are short chunks, run with KSPLIT = 1.
-template <int KSPLIT>
-__global__ void __launch_bounds__(256 * KSPLIT)
+// all keys, takes half the time.  A workgroup runs TASKS tasks, so it has TASKS * KSPLIT waves:
+//   4 x 1  decode steps of few requests: the tasks are short chunks of keys, merged by the second kernel;
+//   4 x 2  prompts and mixed steps;
+//   1 x 8  decode steps of many requests: a task is all keys of a request's token, so nothing is left to the
+//          second kernel (there are enough requests and KV heads to fill the GPU without cutting keys into tasks).
+template <int TASKS, int KSPLIT>
+__global__ void __launch_bounds__(64 * TASKS * KSPLIT)
 attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
                       const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
                       float* __restrict__ part_o, float* __restrict__ part_lse, const Task* __restrict__ tasks,
                       int n_tasks, const int32_t* __restrict__ block_tables, int max_blocks, float scale,
                       int window, int nh, int nkv) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int slot = wave & 3, part = wave >> 2;      // which of the workgroup's four tasks, which share of its keys
+  const int slot = wave % TASKS, part = wave / TASKS;   // which of the workgroup's tasks, which share of its keys
   // workgroups are numbered with the KV head running fastest: neighbours read the same block tables and finish
   // together, and the longest tasks (which come first) start first
   const int kvh = blockIdx.x % nkv;
-  const int ti = (blockIdx.x / nkv) * 4 + slot;
+  const int ti = (blockIdx.x / nkv) * TASKS + slot;
   // with KSPLIT > 1 every wave must reach the barrier below: a wave without work runs an empty range
   const bool has_task = ti < n_tasks && tasks[ti < n_tasks ? ti : 0].entry >= 0;
   if (KSPLIT == 1 && !has_task) return;
@@ -287,9 +291,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     // Merge the shares of a task: the waves with part > 0 lay down (m, l, o), lane by lane; the wave with part 0
     // rescales all to the common maximum and adds them in order.  Same lanes hold the same (row, column) in all.
     constexpr int PER_LANE = DTILES * 16 + 2;
-    __shared__ float merge[(KSPLIT - 1) * 4 * PER_LANE * 64];
+    __shared__ float merge[(KSPLIT - 1) * TASKS * PER_LANE * 64];
     if (part > 0) {
-      float* dst = merge + (size_t)((part - 1) * 4 + slot) * PER_LANE * 64 + lane;
+      float* dst = merge + (size_t)((part - 1) * TASKS + slot) * PER_LANE * 64 + lane;
       dst[0] = m;
       dst[64] = l;
 #pragma unroll
@@ -301,7 +305,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     if (part > 0 || !has_task) return;
 #pragma unroll
     for (int h = 1; h < KSPLIT; ++h) {
-      const float* src = merge + (size_t)((h - 1) * 4 + slot) * PER_LANE * 64 + lane;
+      const float* src = merge + (size_t)((h - 1) * TASKS + slot) * PER_LANE * 64 + lane;
       const float m2 = src[0], l2 = src[64];
       const float m_all = fmaxf(m, m2);
       const float m_use = (m_all == -INFINITY) ? 0.f : m_all;
@@ -442,11 +446,12 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
   }
 }
 
-// two waves per task need (DTILES * 16 + 2) floats per lane of four waves in LDS
-constexpr bool kSplitFits = (DTILES * 16 + 2) * 64 * 4 * sizeof(float) <= 65536;
+// the merge needs (DTILES * 16 + 2) floats per lane of (KSPLIT - 1) * TASKS waves in LDS: 4 waves for 4 x 2, 7 for 1 x 8
+constexpr bool kSplit2Fits = (DTILES * 16 + 2) * 64 * 4 * sizeof(float) <= 65536;
+constexpr bool kSplit8Fits = (DTILES * 16 + 2) * 64 * 7 * sizeof(float) <= 65536;
 
 extern "C" int atoma_attention_mfma_head_size() { return HD; }
-extern "C" int atoma_attention_mfma_max_ksplit() { return kSplitFits ? 2 : 1; }
+extern "C" int atoma_attention_mfma_max_ksplit() { return kSplit8Fits ? 8 : kSplit2Fits ? 2 : 1; }
 
 // tasks: device array of n_tasks Task records (main kernel), followed by n_combine records for the combine kernel.
 extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kcache, const void* vcache, void* out,
@@ -458,18 +463,18 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
       ((uintptr_t)q & 15) || ((uintptr_t)out & 7))
     return ATOMA_ERR_SHAPE;
   const Task* t = reinterpret_cast<const Task*>(tasks);
-  // ksplit: waves that share a task's keys (1, or 2 for head sizes whose merge fits in LDS)
-  const dim3 grid(((n_tasks + 3) / 4) * nkv);
-  if (ksplit == 1)
-    hipLaunchKernelGGL(attention_mfma_kernel<1>, grid, dim3(256), 0, stream, (const uint16_t*)q, q_stride,
-                       (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride, part_o, part_lse,
-                       t, n_tasks, block_tables, max_blocks, scale, window, nh, nkv);
-  else if (ksplit == 2 && kSplitFits)
-    hipLaunchKernelGGL(attention_mfma_kernel<kSplitFits ? 2 : 1>, grid, dim3(512), 0, stream, (const uint16_t*)q,
-                       q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride, part_o,
-                       part_lse, t, n_tasks, block_tables, max_blocks, scale, window, nh, nkv);
-  else
-    return ATOMA_ERR_SHAPE;
+  // ksplit: waves that share a task's keys: 1, 2 (four tasks a workgroup) or 8 (one task a workgroup), the latter
+  // two for head sizes whose merge fits in LDS
+#define ATOMA_ATTN(T, KS)                                                                                          \
+  hipLaunchKernelGGL((attention_mfma_kernel<T, KS>), dim3(((n_tasks + T - 1) / T) * nkv), dim3(64 * T * KS), 0,   \
+                     stream, (const uint16_t*)q, q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,      \
+                     (uint16_t*)out, out_stride, part_o, part_lse, t, n_tasks, block_tables, max_blocks, scale,   \
+                     window, nh, nkv)
+  if (ksplit == 1) ATOMA_ATTN(4, 1);
+  else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1));
+  else if (ksplit == 8 && kSplit8Fits) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1));
+  else return ATOMA_ERR_SHAPE;
+#undef ATOMA_ATTN
   ATOMA_LAUNCH_CHECK();
   if (n_combine > 0) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(n_combine, nkv), dim3(256), 0, stream, part_o, part_lse,

@@ -38,11 +38,28 @@ def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
         _libs[hd] = load_hip_module(module_name(hd), ("attention_mfma.hip",), (f"ATOMA_HD={hd}",),
                                     force_build=force_build)
         assert _libs[hd].atoma_attention_mfma_head_size() == hd
+        assert _libs[hd].atoma_attention_mfma_max_ksplit() == max_waves_for(hd)
     return _libs[hd]
 
 
-def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8) -> Tuple[int, int]:
-    """(keys per partial task, waves that share a task) for the entries of a step that are split along their keys.
+def max_waves_for(hd: int) -> int:
+    """Waves that may share a task for this head size: their merge must fit into LDS (the kernel module says the
+    same: ``atoma_attention_mfma_max_ksplit``)."""
+    per_lane = -(-hd // 32) * 16 + 2
+    if per_lane * 64 * 7 * 4 <= 65536:
+        return 8
+    return 2 if per_lane * 64 * 4 * 4 <= 65536 else 1
+
+
+WHOLE_MIN_PAIRS = 256      # (request, KV head) pairs from which on a decoded token's keys are not cut into chunks
+WHOLE_MAX_KEYS = 4096
+
+
+def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = False) -> Tuple[int, int]:
+    """(keys per partial task, waves that share a task) for the entries of a step that are split along their keys;
+    keys per task 0 means all of them: with ``whole_ok`` (a decode step, head size that allows eight waves) and at
+    least as many (request, KV head) pairs as the GPU has CUs, eight waves walk all keys of a pair and merge in LDS,
+    which leaves nothing to the merging kernel.
 
     A wave walks its keys one 32-key block after another, so few keys per wave shorten the chain when few requests
     decode, and long chunks save partial results (and time in the merging kernel) when many do.  Measured on
@@ -50,6 +67,8 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8) -> Tuple[int, int]
     eleven 256-key chunks walked by two waves each, more requests 256-key chunks with a wave each.  The count that
     decides is that of 256-key tasks over all KV heads; ``max_keys`` is rounded up to 256.
     """
+    if whole_ok and n_split * kv_heads >= WHOLE_MIN_PAIRS and max_keys <= WHOLE_MAX_KEYS:
+        return 0, 8
     tasks = n_split * -(-max_keys // CHUNK) * kv_heads
     if tasks <= 160:
         return 128, 1
@@ -117,7 +136,8 @@ def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, windo
 
 
 def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket: Optional[int] = None,
-                vectorized: bool = True, kv_heads: int = 8) -> Tuple[np.ndarray, Tuple[int, int, int, int]]:
+                vectorized: bool = True, kv_heads: int = 8, max_waves: int = 2,
+                ) -> Tuple[np.ndarray, Tuple[int, int, int, int]]:
     """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials, waves that
     share a task: two when a prompt tile walks many keys, else what ``chunk_for`` says for the split entries).
 
@@ -126,7 +146,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     split and owns ``bucket`` chunk slots, used or not, so all counts depend on (entries, bucket) alone.
     """
     if vectorized and bucket is not None and len(counts) and int(counts.max()) == 1:
-        return _build_decode_tasks(starts, group, window, bucket, kv_heads)
+        return _build_decode_tasks(starts, group, window, bucket, kv_heads, max_waves)
     qt_max = max(1, 128 // group)
     null = (-1, 0, 1, 0, 0, 0, -1, 0, 0, 0, 0, 0)
     tok_bases = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
@@ -142,8 +162,9 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     split_entries = [e for e in range(len(starts)) if splits(e)]
     chunk, waves = CHUNK, 1
     if split_entries:
-        chunk, waves = chunk_for(len(split_entries), max(int(starts[e]) + int(counts[e]) for e in split_entries),
-                                 kv_heads)
+        most = bucket * CHUNK if bucket is not None else max(int(starts[e]) + int(counts[e]) for e in split_entries)
+        chunk, waves = chunk_for(len(split_entries), most, kv_heads)
+        waves = min(waves, max_waves)
     for e in range(len(starts)):
         start, count = int(starts[e]), int(counts[e])
         qt = min(qt_max, count)
@@ -194,15 +215,30 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     return arr, (len(head) + len(split), len(combine), n_part, waves)
 
 
-def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int, kv_heads: int = 8):
+def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int, kv_heads: int = 8,
+                        max_waves: int = 2):
     """``build_tasks`` for a step in which every entry brings one token, without a Python loop over entries."""
     s = len(starts)
     starts = starts.astype(np.int64)
     k_end = starts + 1
     lo = np.maximum(0, starts - window + 1) if window > 0 else np.zeros(s, dtype=np.int64)
-    chunk, waves = chunk_for(s, int(k_end.max()), kv_heads)
-    slots = bucket * (CHUNK // chunk)
     row_chunks = -(-group // 32)
+    # the bucket, not the step's longest request, decides between whole ranges and chunks: a graph holds one of them
+    chunk, waves = chunk_for(s, bucket * CHUNK, kv_heads, whole_ok=max_waves >= 8)
+    waves = min(waves, max_waves)
+    if chunk == 0:
+        whole = np.zeros((s, row_chunks, 12), dtype=np.int32)
+        whole[..., 0] = np.arange(s)[:, None]
+        whole[..., 2] = 1
+        whole[..., 3] = 32 * np.arange(row_chunks)[None, :]
+        whole[..., 4] = ((lo // 32) * 32)[:, None]
+        whole[..., 5] = k_end[:, None]
+        whole[..., 6] = -1
+        whole[..., 8] = np.arange(s)[:, None]
+        whole[..., 9] = 1
+        whole[..., 10] = starts[:, None]
+        return whole.reshape(-1, 12), (s * row_chunks, 0, 0, waves)
+    slots = bucket * (CHUNK // chunk)
     c = np.arange(slots, dtype=np.int64)
     c_first, c_last = lo // chunk, (k_end - 1) // chunk
     valid = (c[None, :] >= c_first[:, None]) & (c[None, :] <= c_last[:, None])          # [s, slots]
@@ -239,8 +275,8 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     return arr, (len(main), s * row_chunks, s * row_chunks * slots, waves)
 
 
-def plan_key(group: int, window: int, kv_heads: int = 8):
-    return ("attention_mfma_tasks", group, window, kv_heads)
+def plan_key(group: int, window: int, kv_heads: int, hd: int):
+    return ("attention_mfma_tasks", group, window, kv_heads, hd)
 
 
 def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, hd) -> bool:
@@ -252,13 +288,14 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
     if tuple(k_cache.shape[1:]) != (nkv, PAGE * hd) or tuple(v_cache.shape[1:]) != (nkv, PAGE * hd):
         raise ValueError("cache tensors must be [pages, nkv, page_size * hd] tiles")
     group = nh // nkv
-    plan = getattr(ctx, "plans", {}).get(plan_key(group, window, nkv))
+    plan = getattr(ctx, "plans", {}).get(plan_key(group, window, nkv, hd))
     if plan is None:
         # a caller without a step planner (a kernel test): plan here and now
-        key = ("attention_tasks_adhoc", group, window, nkv)
+        key = ("attention_tasks_adhoc", group, window, nkv, hd)
         plan = ctx.scratch.get(key)
         if plan is None:
-            arr, meta = build_tasks(ctx.h_starts, ctx.h_counts, group, window, kv_heads=nkv)
+            arr, meta = build_tasks(ctx.h_starts, ctx.h_counts, group, window, kv_heads=nkv,
+                                    max_waves=max_waves_for(hd))
             plan = (torch.from_numpy(arr).to(q.device), meta)
             ctx.scratch[key] = plan
     tasks, (n_main, n_comb, n_part, waves) = plan

@@ -81,9 +81,10 @@ class PagedAttention(Mixer):
         if cache_dtype is not torch.bfloat16 or page_size != attention_bf16.PAGE:
             return None
         group, window, nkv = self.nh // self.nkv, self.window or 0, self.nkv
-        return (attention_bf16.plan_key(group, window, nkv),
-                lambda starts, counts, bucket: attention_bf16.build_tasks(starts, counts, group, window, bucket,
-                                                                          kv_heads=nkv))
+        return (attention_bf16.plan_key(group, window, nkv, self.hd),
+                lambda starts, counts, bucket: attention_bf16.build_tasks(
+                    starts, counts, group, window, bucket, kv_heads=nkv,
+                    max_waves=attention_bf16.max_waves_for(self.hd)))
 
     # -- execution ------------------------------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:

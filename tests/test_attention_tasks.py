@@ -8,9 +8,9 @@ from atoma_infer_amd.kernels import attention_bf16 as A
 
 def coverage(arr, meta, starts, counts, group, window):
     n_main, n_comb, n_part, waves = meta
-    assert waves in (1, 2)
+    assert waves in (1, 2, 8)
     main, comb = arr[:n_main], arr[n_main:]
-    assert len(comb) == n_comb and n_main % 4 == 0
+    assert len(comb) == n_comb and (n_main % 4 == 0 or waves == 8)    # (eight waves: one task a workgroup)
     seen = {}          # (entry, token, head) -> list of key ranges, direct
     parts = {}         # partial index -> (entry, token/head rows, key range)
     for t in main:
@@ -79,8 +79,26 @@ def test_decode_builder_equals_the_general_one(seed):
     coverage(fast, mf, starts, counts, group, window)
     # sizes depend on (entries, bucket) alone
     other = rng.integers(0, bucket * 256, size=s).astype(np.int32)
-    assert A.build_tasks(other, counts, group, window, bucket)[1] == mf or \
-        A.chunk_for(s, int(other.max()) + 1) != A.chunk_for(s, int(starts.max()) + 1)
+    assert A.build_tasks(other, counts, group, window, bucket)[1] == mf
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_whole_ranges_for_many_decoding_requests(seed):
+    """Enough (request, KV head) pairs to fill the GPU: a decoded token's keys are one task for eight waves, and
+    nothing is left to merge."""
+    rng = np.random.default_rng(900 + seed)
+    s = int(rng.integers(32, 100))
+    group, window = int(rng.choice([1, 4, 8])), int(rng.choice([0, 0, 300]))
+    starts = rng.integers(0, 3000, size=s).astype(np.int32)
+    counts = np.ones(s, dtype=np.int32)
+    bucket = -(-int(starts.max() + 1) // 256)
+    arr, meta = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
+    assert meta == (s * -(-group // 32), 0, 0, 8)
+    coverage(arr, meta, starts, counts, group, window)
+    # a head size that does not allow eight waves, or few pairs: chunks as before
+    assert A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=2)[1][1] > 0
+    assert A.build_tasks(starts[:8], counts[:8], group, window, bucket, kv_heads=8, max_waves=8)[1][1] > 0
+    assert A.max_waves_for(64) == 8 and A.max_waves_for(96) == 2 and A.max_waves_for(128) == 1
 
 
 @pytest.mark.parametrize("seed", range(20))

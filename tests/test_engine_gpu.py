@@ -248,3 +248,20 @@ def test_decode_graphs_replay_like_eager_steps(model_dirs, name, dtype):
     # and all of it equals the plain model
     got = {("a", graphed.computed_len(0) - 1): g[1], ("b", graphed.computed_len(1) - 1): g[0]}
     check_against_plain(model_dirs[name], {k: v for k, v in toks.items() if k != "c"}, got, dtype)
+
+
+def test_decoding_with_whole_key_ranges(model_dirs, monkeypatch):
+    """Many decoding requests make every (request, KV head) pair one attention task for eight waves.  Here the
+    threshold is lowered so that three requests do it: decoded through graphs, against the plain model."""
+    from atoma_infer_amd.kernels import attention_bf16
+    monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 2)
+    name, dtype = "D", "bfloat16"
+    vocab = TINY[name]["vocab_size"]
+    requests = {"a": random_tokens(700, vocab, 31), "b": random_tokens(90, vocab, 32), "c": random_tokens(300, vocab, 33)}
+    runner = make_runner(model_dirs[name], dtype, PAGE[name], 80)
+    steps = [([("a", 660), ("b", 50), ("c", 260)], [])] + [([("a", 1), ("b", 1), ("c", 1)], []) for _ in range(40)]
+    got = run_schedule(runner, requests, steps)
+    check_against_plain(model_dirs[name], requests, got, dtype)
+    g = runner._graphs.get((3, 3))
+    assert g is not None and g.graph is not None, "the decode steps were meant to replay as a graph"
+    assert attention_bf16.chunk_for(3, 700, 2, whole_ok=True) == (0, 8)

@@ -523,3 +523,30 @@ def test_products_replay_in_graphs(m, n, k, cdt):
         (other @ other).sum().item()                      # more eager work and a synchronisation
         if i == 3:
             torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("window", [0, 200])
+def test_attention_whole_ranges_with_eight_waves(window):
+    """A decode step of many requests: every (request, KV head) pair is one task whose keys eight waves share and
+    merge in LDS.  Lengths from one key to a few thousand, so that waves with nothing to do sit beside full ones."""
+    from atoma_infer_amd.kernels import attention_bf16 as A
+    nh, nkv, hd, page = 32, 8, 64, 16
+    g = torch.Generator().manual_seed(7)
+    starts = [0, 1, 30, 31, 32, 255, 256, 257, 511, 1000] + torch.randint(0, 2500, (30,), generator=g).tolist()
+    counts = [1] * len(starts)
+    lens = [s + 1 for s in starts]
+    ks, vs, kc, vc, bt = paged_setup(lens, nkv, hd, page, torch.bfloat16, seed=3)
+    q = (torch.randn(len(starts), (nh + 2 * nkv) * hd, generator=g) * 1.5).bfloat16().to(DEV)
+    out = torch.empty(len(starts), nh * hd, dtype=torch.bfloat16, device=DEV)
+    ctx, cache = FakeCtx(starts, counts), FakeCache(bt, page)
+    bucket = -(-max(lens) // 256)
+    arr, meta = A.build_tasks(ctx.h_starts, ctx.h_counts, nh // nkv, window, bucket, kv_heads=nkv, max_waves=8)
+    assert meta[1:] == (0, 0, 8)
+    ctx.plans = {A.plan_key(nh // nkv, window, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
+    scale = 1.0 / math.sqrt(hd)
+    assert A.try_attention(q, kc, vc, out, ctx, cache, scale, window, nh, nkv, hd)
+    for e, s in enumerate(starts):
+        qq = q[e:e + 1, : nh * hd].cpu().view(1, nh, hd)
+        want = plain_attention(qq, ks[e], vs[e], s, scale, window, nh // nkv).reshape(nh * hd)
+        err = (out[e].double().cpu() - want).abs().max() / want.abs().max()
+        assert err < 2e-2, f"request {e} of length {s + 1}: {err:.3e}"
