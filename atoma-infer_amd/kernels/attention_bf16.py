@@ -51,15 +51,18 @@ def max_waves_for(hd: int) -> int:
     return 2 if per_lane * 64 * 4 * 4 <= 65536 else 1
 
 
-WHOLE_MIN_PAIRS = 256      # (request, KV head) pairs from which on a decoded token's keys are not cut into chunks
+# (request, KV head) pairs from which on a decoded token's keys are not cut into chunks: measured on MI355X (256 CUs),
+# half as many pairs as CUs win already at contexts up to 4,096, three quarters at any context
+WHOLE_MIN_PAIRS = 128
 WHOLE_MAX_KEYS = 4096
+WHOLE_MIN_PAIRS_LONG = 192
 
 
 def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = False) -> Tuple[int, int]:
     """(keys per partial task, waves that share a task) for the entries of a step that are split along their keys;
-    keys per task 0 means all of them: with ``whole_ok`` (a decode step, head size that allows eight waves) and at
-    least as many (request, KV head) pairs as the GPU has CUs, eight waves walk all keys of a pair and merge in LDS,
-    which leaves nothing to the merging kernel.
+    keys per task 0 means all of them: with ``whole_ok`` (a decode step, head size that allows eight waves) and
+    enough (request, KV head) pairs to occupy the GPU, eight waves walk all keys of a pair and merge in LDS, which
+    leaves nothing to the merging kernel.
 
     A wave walks its keys one 32-key block after another, so few keys per wave shorten the chain when few requests
     decode, and long chunks save partial results (and time in the merging kernel) when many do.  Measured on
@@ -67,7 +70,9 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = F
     eleven 256-key chunks walked by two waves each, more requests 256-key chunks with a wave each.  The count that
     decides is that of 256-key tasks over all KV heads; ``max_keys`` is rounded up to 256.
     """
-    if whole_ok and n_split * kv_heads >= WHOLE_MIN_PAIRS and max_keys <= WHOLE_MAX_KEYS:
+    pairs = n_split * kv_heads
+    if whole_ok and (pairs >= max(WHOLE_MIN_PAIRS_LONG, WHOLE_MIN_PAIRS) or
+                     (pairs >= WHOLE_MIN_PAIRS and max_keys <= WHOLE_MAX_KEYS)):
         return 0, 8
     tasks = n_split * -(-max_keys // CHUNK) * kv_heads
     if tasks <= 160:

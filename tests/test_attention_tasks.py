@@ -87,7 +87,7 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     """Enough (request, KV head) pairs to fill the GPU: a decoded token's keys are one task for eight waves, and
     nothing is left to merge."""
     rng = np.random.default_rng(900 + seed)
-    s = int(rng.integers(32, 100))
+    s = int(rng.integers(24, 100))
     group, window = int(rng.choice([1, 4, 8])), int(rng.choice([0, 0, 300]))
     starts = rng.integers(0, 3000, size=s).astype(np.int32)
     counts = np.ones(s, dtype=np.int32)
