@@ -37,7 +37,8 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
                    int K, int lda, int ldw, int ldc, size_t plane, RopeArgs ra) {
   // loads of U steps of K are issued together before their MFMAs, so that a wave keeps U * (RT + MT) 16-byte
   // loads per lane in flight: the product is bound by memory latency and bandwidth, not by arithmetic
-  constexpr int U = (RT + MT <= 2) ? 4 : (RT + MT <= 5) ? 2 : 1;
+  // (eight waves of many tiles have 256 registers each: one step)
+  constexpr int U = (RT + MT <= 2) ? 4 : (RT + MT > 5 && WK > 4) ? 1 : 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wn = wave % WN, wk = wave / WN;
   const int r16 = lane & 15, kg = lane >> 4;
@@ -281,13 +282,14 @@ static int launch_mt(const void* a, const void* w, void* c, int c_dtype, int M, 
   ATOMA_CASE(2, 1, 4);
   ATOMA_CASE(1, 1, 8);
   ATOMA_CASE(2, 1, 8);
+  ATOMA_CASE(4, 1, 4);
 #undef ATOMA_CASE
   return ATOMA_ERR_SHAPE;
 }
 
 // a [M <= 64, K] bf16, w [N, K] bf16 -> c [slices][M, N] (bf16 only with slices == 1, or float32).
 // rt: tiles of 16 rows of W per wave (1, 2, 4); wk: 1 (four waves on different rows), 4 or 8 (that many waves
-// split K for the same rows); slices: K split across the grid.
+// split K for the same rows; four tiles only with 4); slices: K split across the grid.
 extern "C" int atoma_gemm_bf16_skinny(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
                                       int lda, int ldw, int ldc, int rt, int wk, int slices, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -319,7 +321,10 @@ static int launch_swiglu_mt(const void* a, const void* w, void* c, int M, int N,
   if (rt == 2 && wk == 1) return launch_swiglu<MT, 2, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, stream);
   if (rt == 4 && wk == 1) return launch_swiglu<MT, 4, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, stream);
   if (rt == 2 && wk == 4) return launch_swiglu<MT, 2, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, stream);
-  if (rt == 2 && wk == 8) return launch_swiglu<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+  if constexpr (MT < 4) {   // with four tiles of rows the epilogue does not fit the registers of eight waves
+    if (rt == 2 && wk == 8) return launch_swiglu<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+  }
+  if (rt == 4 && wk == 4) return launch_swiglu<MT, 4, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, stream);
   return ATOMA_ERR_SHAPE;
 }
 
@@ -355,7 +360,9 @@ static int launch_rope_mt(const void* a, const void* w, void* c, int M, int N, i
   if (rt == 1 && wk == 4) return launch_rope<MT, 1, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
   if (rt == 2 && wk == 4) return launch_rope<MT, 2, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
   if (rt == 1 && wk == 8) return launch_rope<MT, 1, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
-  if (rt == 2 && wk == 8) return launch_rope<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  if constexpr (MT < 4) {   // with four tiles of rows the epilogue does not fit the registers of eight waves
+    if (rt == 2 && wk == 8) return launch_rope<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  }
   if (rt == 1 && wk == 1) return launch_rope<MT, 1, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
   if (rt == 2 && wk == 1) return launch_rope<MT, 2, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
   return ATOMA_ERR_SHAPE;

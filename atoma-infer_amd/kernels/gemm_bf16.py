@@ -36,31 +36,51 @@ def _aligned(t: torch.Tensor) -> bool:
 def _plan(m: int, n: int, k: int, allow_slices: bool):
     """(rows-of-16 per wave, waves splitting K, K slices over the grid) for x [m, k] @ w [n, k]^T.
 
-    Chosen from measurements on MI355X at the sizes of Llama-3.2-1B: few rows of x want many waves that split K
-    (every wave's loads are in flight at once); many rows want waves that own several row tiles of W, so that
-    each fragment of x feeds several MFMAs.
+    Chosen from measurements on MI355X at the sizes of Llama-3.2-1B.  Up to 16 rows of x want many waves that split
+    K (every wave's loads are in flight at once).  With more rows the fragments of x weigh as much as the weight,
+    so a wave owns 32 or 64 rows of W for each fragment of x it fetches; where N is small that leaves too few
+    workgroups, and K is split over the grid into float32 planes, about 256 workgroups in all, if the caller takes
+    planes.
     """
     tiles = -(-n // 16)
-    small_m = m <= 16
-    if tiles >= 4096:
-        rt, wk = (2, 8) if small_m else (4, 1)
+    if m <= 16:
+        if tiles >= 4096:
+            rt, wk = 2, 8
+        elif tiles >= 512:
+            rt, wk = 2, 4
+        else:
+            rt, wk = 1, 4
+        max_slices = 2        # two planes already put enough workgroups in flight (more measured no faster)
+    elif tiles >= 4096:
+        rt, wk, max_slices = 4, 1, 1
     elif tiles >= 512:
-        rt, wk = 2, 4
+        rt, wk, max_slices = 4, 4, 1
+    elif not allow_slices:
+        rt, wk, max_slices = 1, 4, 1
     else:
-        rt, wk = (1, 4) if small_m or not allow_slices else (2, 4)
+        # 64 rows of W per wave where K is long enough to feed four waves of 256 workgroups, else 32
+        rt, wk, max_slices = 4, 4, 8
+        if k // (4 * _slices_for(tiles, 4, 8)) < 256:
+            rt = 2
     while wk > 1 and k % (32 * wk):
         wk //= 2
     if wk == 2:
         wk = 1
     slices = 1
-    if allow_slices:
-        groups = -(-tiles // ((4 if wk == 1 else 1) * rt))
-        # two planes already put enough workgroups in flight (more measured no faster) and keep the consumer,
-        # which adds the planes, cheap
-        slices = 2
-        while slices > 1 and (k % (32 * wk * slices) or k // (wk * slices) < 128 or groups * slices > 1024):
+    if allow_slices and max_slices > 1:
+        slices = min(max_slices, _slices_for(tiles, (4 if wk == 1 else 1) * rt, max_slices))
+        while slices > 1 and (k % (32 * wk * slices) or k // (wk * slices) < 128):
             slices //= 2
     return rt, wk, slices
+
+
+def _slices_for(tiles: int, tiles_per_group: int, most: int) -> int:
+    """The power of two, at most ``most``, of K slices that brings the grid to about 256 workgroups."""
+    groups = -(-tiles // tiles_per_group)
+    slices = 1
+    while slices < most and groups * slices * 2 <= 256:
+        slices *= 2
+    return slices
 
 
 def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -131,11 +151,10 @@ def try_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Op
 
 
 def linear_planes(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
-    """For M <= 64: float32 planes [slices, M, N] whose sum is x @ w^T (K split over the grid), else None (also
-    where the library's product is the faster way to the same sum)."""
+    """For M <= 64: float32 planes [slices, M, N] whose sum is x @ w^T (K split over the grid), else None."""
     m, k = x.shape
     n = w.shape[0]
-    if m > SKINNY_MAX_M or not skinny_ok(x, w) or _library_wins(m, n, k, torch.bfloat16):
+    if m > SKINNY_MAX_M or not skinny_ok(x, w):
         return None
     rt, wk, slices = _plan(m, n, k, True)
     out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
@@ -150,12 +169,12 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
     """
     m, k = x.shape
     n = w.shape[0]
-    if m > LIBRARY_MIN_M_WIDE or n % 32 or not skinny_ok(x, w):
+    if m > SKINNY_MAX_M or n % 32 or not skinny_ok(x, w):
         return None
     rt, wk, _ = _plan(m, n, k, False)
     if rt % 2:
         rt = 2
-    if (rt, wk) not in ((2, 1), (4, 1), (2, 4), (2, 8)):
+    if (rt, wk) not in ((2, 1), (4, 1), (2, 4), (2, 8), (4, 4)):
         return None
     out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     _check(lib().atoma_gemm_bf16_skinny_swiglu(_p(x), _p(w), _p(out), m, n, k, x.stride(0) if m > 1 else k,

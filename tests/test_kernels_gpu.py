@@ -122,11 +122,23 @@ def test_gemm_bf16_skinny(m, n, k, cdt):
     assert c is not None and c.dtype is cdt
     assert (c.double().cpu() - want).abs().max() <= tol * want.abs().max()
     planes = gemm_bf16.linear_planes(a, w)
-    if gemm_bf16._library_wins(m, n, k, torch.bfloat16):
-        assert planes is None
-    else:
-        assert planes.dim() == 3
-        assert (planes.sum(0).double().cpu() - want).abs().max() <= 1e-5 * want.abs().max()
+    assert planes.dim() == 3
+    assert (planes.sum(0).double().cpu() - want).abs().max() <= 1e-5 * want.abs().max()
+
+
+@pytest.mark.parametrize("m", [3, 20, 33, 64])
+@pytest.mark.parametrize("rt,wk,slices", [(1, 1, 1), (2, 1, 2), (4, 1, 1), (1, 4, 8), (2, 4, 4), (4, 4, 8), (4, 4, 1),
+                                          (1, 8, 2), (2, 8, 1)])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (200, 4096), (72, 2048)])
+def test_gemm_bf16_skinny_every_shape_of_wave(m, rt, wk, slices, n, k):
+    """Every way of dealing the rows of W and the steps of K to waves gives the same product, whatever the plan
+    would pick at the size."""
+    from atoma_infer_amd.kernels import gemm_bf16
+    a, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2)
+    want = a.double().cpu() @ w.double().cpu().T
+    planes = torch.full((slices, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    gemm_bf16.skinny(a, w, planes, slices, rt, wk)
+    assert (planes.sum(0).double().cpu() - want).abs().max() <= 1e-5 * want.abs().max()
 
 
 def test_gemm_bf16_rows_do_not_depend_on_the_batch():
@@ -439,8 +451,8 @@ def test_swiglu_interleaved_layout(dt):
     assert torch.allclose(out.float(), want, rtol=tol, atol=tol)
 
 
-@pytest.mark.parametrize("m", [1, 8, 17, 32])
-@pytest.mark.parametrize("inter,k", [(16, 32), (160, 64), (8192, 2048), (1024, 96)])
+@pytest.mark.parametrize("m", [1, 8, 17, 32, 50, 64])
+@pytest.mark.parametrize("inter,k", [(16, 32), (160, 64), (8192, 2048), (1024, 96), (8208, 256)])
 def test_gemm_with_swiglu_epilogue(m, inter, k):
     from atoma_infer_amd.kernels import gemm_bf16
     x = rnd(m, k, dtype=torch.bfloat16, seed=1)
@@ -450,7 +462,7 @@ def test_gemm_with_swiglu_epilogue(m, inter, k):
     g, u = x.double().cpu() @ wg.double().cpu().T, x.double().cpu() @ wu.double().cpu().T
     want = torch.nn.functional.silu(g) * u
     assert (out.double().cpu() - want).abs().max() <= 1e-2 * want.abs().max()
-    assert gemm_bf16.try_linear_swiglu(rnd(40, k, dtype=torch.bfloat16), interleave16(wg, wu)) is None   # too many rows
+    assert gemm_bf16.try_linear_swiglu(rnd(70, k, dtype=torch.bfloat16), interleave16(wg, wu)) is None   # too many rows
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 23, 40, 64])
