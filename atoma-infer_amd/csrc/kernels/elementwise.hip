@@ -277,7 +277,9 @@ rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const in
   const int per_qk = hd >> 4;                              // items per head
   const int n_qk = (nh + nkv) * per_qk;
   const bool paired = q_out != nullptr;
-  for (int item = threadIdx.x; item < nt * n_qk; item += 256) {
+  // the block's items are dealt over gridDim.y blocks, which keeps the GPU busy when the tokens are few
+  const int first = blockIdx.y * 256 + threadIdx.x, stride = gridDim.y * 256;
+  for (int item = first; item < nt * n_qk; item += stride) {
     const int t = t0 + item / n_qk, it = item % n_qk;
     const int head = it / per_qk, i0 = (it % per_qk) * 8;
     const bool is_k = head >= nh;
@@ -327,7 +329,7 @@ rope_cache_write_vec_kernel(uint16_t* __restrict__ qkv, int row_stride, const in
                         slots[1] == slots[0] + 1 &&
                         slots[2] == slots[0] + 2 && slots[3] == slots[0] + 3;    // (then all in one page)
   const int quads = hd >> 2;
-  for (int item = threadIdx.x; item < nkv * quads; item += 256) {
+  for (int item = first; item < nkv * quads; item += stride) {
     const int head = item / quads, d0 = (item % quads) * 4;
     uint2 raw[kRopeTokens];
 #pragma unroll
@@ -381,7 +383,11 @@ extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, 
       q_stride % 8 == 0 &&
       ((uintptr_t)q_out & 15) == 0 &&
       ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0) {
-    hipLaunchKernelGGL(rope_cache_write_vec_kernel, dim3((n_tokens + kRopeTokens - 1) / kRopeTokens), dim3(256), 0,
+    const int groups = (n_tokens + kRopeTokens - 1) / kRopeTokens;
+    const int passes = (kRopeTokens * (nh + nkv) * (hd >> 4) + 255) / 256;      // of 256 threads over a block's items
+    int split = (512 + groups - 1) / groups;                                   // aim at 512 blocks
+    split = split > passes ? passes : split;
+    hipLaunchKernelGGL(rope_cache_write_vec_kernel, dim3(groups, split), dim3(256), 0,
                        stream, (uint16_t*)qkv, row_stride, positions, cos_t, sin_t, (uint16_t*)kcache,
                        (uint16_t*)vcache, slot_mapping, page_size, nh, nkv, hd, (uint16_t*)q_out, q_stride, n_tokens);
     ATOMA_LAUNCH_CHECK();

@@ -18,7 +18,8 @@ from .library import load_hip_module
 from .ops import BF16, F32, _check, _p, _stream
 
 SKINNY_MAX_M = 64
-LIBRARY_MIN_M_WIDE = 32
+LIBRARY_MIN_M_WIDE = 32       # beyond this many rows the library takes products whose weight has 2^24 elements or more
+SWIGLU_WIDE = 1 << 25         # weights up to this size keep the fused SiLU-multiply up to 64 rows
 _lib = None
 
 
@@ -53,22 +54,22 @@ def _plan(m: int, n: int, k: int, allow_slices: bool):
         max_slices = 2        # two planes already put enough workgroups in flight (more measured no faster)
     elif tiles >= 4096:
         rt, wk, max_slices = 4, 1, 1
-    elif tiles >= 512:
-        rt, wk, max_slices = 4, 4, 1
-    elif not allow_slices:
-        rt, wk, max_slices = 1, 4, 1
-    else:
-        # 64 rows of W per wave where K is long enough to feed four waves of 256 workgroups, else 32
+    elif allow_slices and tiles < 640:
+        # 64 rows of W per wave where K is long enough for the four waves of each of about 256 workgroups, else 32
         rt, wk, max_slices = 4, 4, 8
-        if k // (4 * _slices_for(tiles, 4, 8)) < 256:
+        if k // (4 * _slices_for(tiles, 4, 8)) < 128:
             rt = 2
+    else:
+        # as many rows of W per wave as still leave 160 workgroups
+        rt, wk, max_slices = (4 if tiles >= 640 else 2 if tiles >= 320 else 1), 4, 1
     while wk > 1 and k % (32 * wk):
         wk //= 2
     if wk == 2:
         wk = 1
     slices = 1
     if allow_slices and max_slices > 1:
-        slices = min(max_slices, _slices_for(tiles, (4 if wk == 1 else 1) * rt, max_slices))
+        per_group = (4 if wk == 1 else 1) * rt
+        slices = 2 if m <= 16 and -(-tiles // per_group) <= 512 else _slices_for(tiles, per_group, max_slices)
         while slices > 1 and (k % (32 * wk * slices) or k // (wk * slices) < 128):
             slices //= 2
     return rt, wk, slices
@@ -104,10 +105,11 @@ def skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, slices: int = 1,
 
 
 def _library_wins(m: int, n: int, k: int, out_dtype: torch.dtype) -> bool:
-    """Measured on MI355X at the sizes of Llama-3.2-1B: where the library's tiles beat the streaming kernel.
+    """Measured on MI355X at the layer shapes of Llama 1B, 3B and 8B: where the library's tiles beat the streaming
+    kernel for a product with output in ``out_dtype``.
 
-    The streaming kernel fetches the activations anew for every 16 or 32 rows of the weight, which costs little up
-    to 16 rows of activations and more than the weight itself beyond 32."""
+    The streaming kernel fetches the activations anew for every 16 to 64 rows of the weight, which costs little up
+    to 16 rows of activations and as much as the weight itself beyond 32."""
     if out_dtype is torch.float32:
         return m > 16 and _MM_OUT_DTYPE
     if m > SKINNY_MAX_M:
@@ -169,7 +171,7 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
     """
     m, k = x.shape
     n = w.shape[0]
-    if m > SKINNY_MAX_M or n % 32 or not skinny_ok(x, w):
+    if m > SKINNY_MAX_M or (m > LIBRARY_MIN_M_WIDE and n * k > SWIGLU_WIDE) or n % 32 or not skinny_ok(x, w):
         return None
     rt, wk, _ = _plan(m, n, k, False)
     if rt % 2:
@@ -187,15 +189,16 @@ ROPE_MAX_M = SKINNY_MAX_M
 
 def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                     kcache: torch.Tensor, vcache: torch.Tensor, slot_mapping: torch.Tensor, page_size: int, nh: int,
-                    nkv: int, hd: int) -> Optional[torch.Tensor]:
+                    nkv: int, hd: int, always: bool = False) -> Optional[torch.Tensor]:
     """The fused q, k, v projection with rotary encoding and the cache write in its epilogue, for few rows of x.
 
     ``w`` has the rows of its q and k heads in pair order (see ``parts/attention.py``).  Returns the rotated q
-    [M, nh * hd]; k (rotated) and v are in the cache.  None when the shape is not taken.
+    [M, nh * hd]; k (rotated) and v are in the cache.  None when the shape is not taken, or when the library's
+    product followed by the rotary kernel is the quicker way (unless ``always``).
     """
     m, k = x.shape
     n = w.shape[0]
-    if (m > ROPE_MAX_M or n != (nh + 2 * nkv) * hd or hd % 4 or not skinny_ok(x, w)
+    if (m > ROPE_MAX_M or (not always and _library_wins(m, n, k, torch.bfloat16)) or n != (nh + 2 * nkv) * hd or hd % 4 or not skinny_ok(x, w)
             or kcache.dtype is not torch.bfloat16 or vcache.dtype is not torch.bfloat16
             or cos.dtype is not torch.float32 or cos.shape[1] != hd // 2 or not cos.is_contiguous()
             or not sin.is_contiguous() or not kcache.is_contiguous() or not vcache.is_contiguous()):

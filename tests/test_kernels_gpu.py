@@ -491,7 +491,7 @@ def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
         return (pack_keys(torch.randn(pages, nkv, page, hd, generator=gg).bfloat16()).to(DEV),
                 pack_values(torch.randn(pages, nkv, hd, page, generator=gg).bfloat16()).to(DEV))
     kc1, vc1 = caches()
-    q1 = gemm_bf16.try_linear_rope(x, w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv, hd)
+    q1 = gemm_bf16.try_linear_rope(x, w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv, hd, always=True)
     assert q1 is not None and tuple(q1.shape) == (m, nh * hd)
     # apart, with float32 in between (the fused kernel rotates the float32 sums)
     kc2, vc2 = caches()
