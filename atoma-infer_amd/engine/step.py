@@ -149,7 +149,8 @@ class ModelRunner:
     def __init__(self, model, pool: CachePool, use_graphs: bool = True):
         self.model, self.pool = model, pool
         self.manager = pool.manager
-        self.use_graphs = use_graphs
+        # decode steps are recorded into graphs only if every part of the model can be replayed
+        self.use_graphs = use_graphs and model.spec.graph_safe()
         self._stage = _Staging(model.device)
         self._computed: Dict[int, int] = {}       # request -> tokens in the cache
         self._graphs: "OrderedDict[Tuple[int, int], _Graph]" = OrderedDict()

@@ -50,6 +50,10 @@ class ModelSpec:
                     raise ValueError(f"run order entry {pos}: its cache needs {a} differ from entry "
                                      f"{call.kv_from}'s {b}")
 
+    def graph_safe(self) -> bool:
+        """Whether every part allows its steps to be recorded into HIP graphs (``Part.graph_safe``)."""
+        return all(part.graph_safe() for _, part in self.parts())
+
     def parts(self) -> List[Tuple[str, Part]]:
         """Every (prefix, part) that binds tensors, in checkpoint order."""
         return [self.embedding] + list(self.layers) + [self.final_norm, self.head]

@@ -47,6 +47,10 @@ class PagedAttention(Mixer):
         self.paired = False      # q and k columns in pair order (set at load time)
 
     # -- declaration ----------------------------------------------------------------------------------
+    def graph_safe(self) -> bool:
+        # the kernels take the step from device tensors and from the plan made before the step is recorded
+        return self.position is None or self.position.graph_safe()
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         q, kv = self.nh * self.hd, self.nkv * self.hd
         return {"q_proj.weight": WeightSpec((q, self.width)), "k_proj.weight": WeightSpec((kv, self.width)),

@@ -70,6 +70,16 @@ class Part:
         """Bytes of weights this part reads once per step (for the roofline)."""
         return 0
 
+    def graph_safe(self) -> bool:
+        """Whether a step through this part may be recorded once into a HIP graph and replayed.
+
+        True only if ``forward`` launches the same kernels with the same arguments for every step of the same shape
+        and takes whatever differs between such steps (positions, block tables, state slots, plans) from the
+        context's device tensors.  A part that branches on the context's host copies, loops over requests on the
+        host or waits for the device says False, the default; a model that holds such a part runs every step
+        directly."""
+        return False
+
 
 class Norm(Part):
     def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,

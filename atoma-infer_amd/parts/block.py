@@ -27,6 +27,9 @@ class PreNormBlock(Block):
         for n, part in self._children():
             part.load(lambda rel, _n=n: get(f"{_n}.{rel}"), device, act_dtype)
 
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe() for _, part in self._children())
+
     def device_bytes(self) -> int:
         return sum(part.device_bytes() for _, part in self._children())
 

@@ -20,6 +20,9 @@ class TokenEmbedding(Part):
         self.vocab_size, self.width = int(vocab_size), int(width)
         self.weight: Optional[torch.Tensor] = None
 
+    def graph_safe(self) -> bool:
+        return True
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {"weight": WeightSpec((self.vocab_size, self.width), "embedding")}
 
@@ -37,6 +40,9 @@ class OutputHead(Part):
     def __init__(self, width: int, vocab_size: int, tied_to: Optional[TokenEmbedding] = None):
         self.width, self.vocab_size, self.tied_to = int(width), int(vocab_size), tied_to
         self.weight: Optional[torch.Tensor] = None
+
+    def graph_safe(self) -> bool:
+        return True
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {} if self.tied_to is not None else {"weight": WeightSpec((self.vocab_size, self.width))}

@@ -23,6 +23,9 @@ class SwiGLU(FeedForward):
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
+    def graph_safe(self) -> bool:
+        return True
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {"gate_proj.weight": WeightSpec((self.inter, self.width)),
                 "up_proj.weight": WeightSpec((self.inter, self.width)),

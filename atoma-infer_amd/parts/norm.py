@@ -19,6 +19,9 @@ class RMSNorm(Norm):
         self.weight: Optional[torch.Tensor] = None
         self.act_dtype = torch.float32
 
+    def graph_safe(self) -> bool:
+        return True
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {"weight": WeightSpec((self.width,), "norm")}
 

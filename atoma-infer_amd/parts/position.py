@@ -50,6 +50,9 @@ class RotaryEncoding(PositionEncoding):
         sc = tuple(sorted(self.scaling.items())) if self.scaling else None
         return (self.rotary_dim, self.theta, self.max_positions, sc, str(device))
 
+    def graph_safe(self) -> bool:
+        return True
+
     def prepare(self, device) -> None:
         key = self._key(device)
         if key not in _TABLES:
@@ -76,6 +79,9 @@ class RotaryEncoding(PositionEncoding):
 class NoPosition(PositionEncoding):
     def __init__(self, **_):
         pass
+
+    def graph_safe(self) -> bool:
+        return True
 
     def apply(self, q, k, positions) -> None:
         return None

@@ -205,9 +205,10 @@ def test_part_registries():
 
 
 def _toy_parts():
-    """Parts that exist only in this test: a mixer with state of its own and another position encoding."""
-    from atoma_infer_amd.parts import (Mixer, PositionEncoding, StateSpec, WeightSpec, register_mixer,
-                                       register_position)
+    """Parts that exist only in this test: a mixer with state of its own, another position encoding and a
+    feed-forward that routes every token to some of its experts."""
+    from atoma_infer_amd.parts import (FeedForward, Mixer, PositionEncoding, StateSpec, WeightSpec,
+                                       register_feed_forward, register_mixer, register_position)
 
     class DecayMixer(Mixer):
         """state <- decay * state + x W_in (per token, in order); y = state W_out.  State: [inner] per request."""
@@ -261,7 +262,44 @@ def _toy_parts():
                 x[..., 0::2] = (a * c - b * s).to(x.dtype)
                 x[..., 1::2] = (b * c + a * s).to(x.dtype)
 
+    class RoutedFeedForward(FeedForward):
+        """Every token goes to the ``top`` experts with its largest router logits (float32); their outputs are
+        weighted by the softmax over those logits.  An expert is a small gate/up/down feed-forward."""
+
+        def __init__(self, width: int, inter: int, experts: int, top: int):
+            self.width, self.inter, self.n, self.top = width, inter, experts, top
+
+        def weight_specs(self):
+            d = {"router.weight": WeightSpec((self.n, self.width))}
+            for e in range(self.n):
+                d[f"experts.{e}.gate_proj.weight"] = WeightSpec((self.inter, self.width))
+                d[f"experts.{e}.up_proj.weight"] = WeightSpec((self.inter, self.width))
+                d[f"experts.{e}.down_proj.weight"] = WeightSpec((self.width, self.inter))
+            return d
+
+        def load(self, get, device, act_dtype):
+            self.router = get("router.weight").to(device)
+            self.experts = [(torch.cat([get(f"experts.{e}.gate_proj.weight"), get(f"experts.{e}.up_proj.weight")]).to(device),
+                             get(f"experts.{e}.down_proj.weight").to(device)) for e in range(self.n)]
+
+        def forward(self, x, ctx):
+            from atoma_infer_amd.kernels import ops
+            from atoma_infer_amd.parts import linear
+            logits = linear(x, self.router, torch.float32)
+            val, idx = torch.topk(logits, self.top, dim=-1)
+            gate = torch.softmax(val, dim=-1)
+            out = torch.zeros(x.shape[0], self.width, dtype=torch.float32, device=x.device)
+            for e, (w_gate_up, w_down) in enumerate(self.experts):
+                hit = idx == e
+                rows = hit.any(-1).nonzero().flatten()        # read on the host: this part is not graph-safe
+                if rows.numel() == 0:
+                    continue
+                y = linear(ops.swiglu(linear(x[rows], w_gate_up)), w_down, torch.float32)
+                out.index_add_(0, rows, y * (gate * hit)[rows].sum(-1, keepdim=True))
+            return out
+
     register_mixer("toy_decay", DecayMixer, replace=True)
+    register_feed_forward("toy_routed", RoutedFeedForward, replace=True)
     register_position("toy_interleaved", InterleavedRotary, replace=True)
 
 
@@ -304,9 +342,14 @@ def _toy_architecture():
                                   num_kv_heads=cfg.kv_heads, head_size=hd, position=pos, window=ld.get("window"))
             else:
                 mixer = make_part("mixer", "toy_decay", width=cfg.width, inner=ld["inner"], decay=ld["decay"])
+            if "experts" in ld:
+                ffn = make_part("feed_forward", "toy_routed", width=cfg.width, inter=ld["expert_inter"],
+                                experts=ld["experts"], top=ld["top"])
+            else:
+                ffn = make_part("feed_forward", "swiglu", width=cfg.width, intermediate=cfg.inter)
             block = make_part("block", "pre_norm", norm1=make_part("norm", "rmsnorm", width=cfg.width, eps=cfg.eps),
                               mixer=mixer, norm2=make_part("norm", "rmsnorm", width=cfg.width, eps=cfg.eps),
-                              feed_forward=make_part("feed_forward", "swiglu", width=cfg.width, intermediate=cfg.inter),
+                              feed_forward=ffn,
                               names=("norm_a", "mixer", "norm_b", "ffn"))
             layers.append((f"toy.layers.{i}", block))
         emb = TokenEmbedding(cfg.vocab, cfg.width)
@@ -333,6 +376,15 @@ TOY = {
     "order": [{"layer": 0}, {"layer": 1}, {"layer": 2}, {"layer": 3}, {"layer": 1}, {"layer": 4},
               {"layer": 4, "kv_from": 0}],
 }
+
+
+# the same kinds of layers with routed feed-forwards of different sizes.  Compared with the plain model in float32
+# only: where two router logits nearly tie, bfloat16 rounding may pick the other expert, which is no fault
+TOY_ROUTED = dict(TOY, vocab=157, layers=[
+    {"mixer": "attention", "position": "rotary", "experts": 3, "top": 2, "expert_inter": 48},
+    {"mixer": "toy_decay", "inner": 24, "decay": 0.8},
+    {"mixer": "attention", "position": "rotary", "window": 24, "experts": 5, "top": 1, "expert_inter": 32},
+], order=[{"layer": 0}, {"layer": 1}, {"layer": 2}])
 
 
 def toy_plain_forward(tokens: List[int], w: Dict[str, torch.Tensor], cfg: dict) -> torch.Tensor:
@@ -385,7 +437,17 @@ def toy_plain_forward(tokens: List[int], w: Dict[str, torch.Tensor], cfg: dict) 
                 ys.append(st)
             a = torch.stack(ys) @ w[p + "mixer.out_proj.weight"].T
         x = x + a
-        x = x + P.swiglu_mlp(P.rms_norm(x, w[p + "norm_b.weight"], cfg["eps"]), w, p + "ffn.")
+        h = P.rms_norm(x, w[p + "norm_b.weight"], cfg["eps"])
+        if "experts" in ld:
+            val, idx = torch.topk(h @ w[p + "ffn.router.weight"].T, ld["top"], dim=-1)
+            gate = torch.softmax(val, dim=-1)
+            y = torch.zeros_like(x)
+            for i in range(t):
+                for j in range(ld["top"]):
+                    y[i] += gate[i, j] * P.swiglu_mlp(h[i:i + 1], w, p + f"ffn.experts.{int(idx[i, j])}.")[0]
+            x = x + y
+        else:
+            x = x + P.swiglu_mlp(h, w, p + "ffn.")
     return P.rms_norm(x, w["toy.final_norm.weight"], cfg["eps"]) @ w["toy.head.weight"].T
 
 
@@ -412,10 +474,44 @@ def test_toy_cache_plan(toy_dir):
     assert plan.where[6] == (0, 0, False) and sorted(plan.states) == [1, 4] and plan.states[1] == (40,)
 
 
+def _toy_run(model, plan, reqs, schedule, pages):
+    """Step ``schedule`` ([(request name, tokens), ...], [names that end]) and collect the logits of every position."""
+    from atoma_infer_amd.cache import CachePool
+    from atoma_infer_amd.engine import ModelRunner, StepEntry
+    pool = CachePool(plan, 16, pages, 3, model.act_dtype, model.device)
+    runner = ModelRunner(model, pool)
+    ids, got = {}, {}
+    for entries, end in schedule:
+        batch, places = [], []
+        for name, n in entries:
+            if name not in ids:
+                ids[name] = len(ids)
+                runner.add_request(ids[name])
+            s = runner.computed_len(ids[name])
+            batch.append(StepEntry(ids[name], reqs[name][s:s + n], s, list(range(n))))
+            places += [(name, s + i) for i in range(n)]
+        logits = runner.step(batch).cpu()
+        for r, key in enumerate(places):
+            got[key] = logits[r].clone()
+        for name in end:
+            runner.free_request(ids[name])
+        runner.manager.check()
+    return got, runner
+
+
+def _toy_check(got, want, dtype):
+    for n in want:
+        rows = sorted(p for (m, p) in got if m == n)
+        mine, ref = torch.stack([got[(n, p)] for p in rows]), want[n][rows]
+        if dtype == "float32":
+            assert rel_err(mine, ref) < TOL_F32, n
+        else:
+            assert frob_err(mine, ref) < TOL_BF16, n
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_architecture_steps_like_its_plain_model(toy_dir, dtype):
-    from atoma_infer_amd.cache import CachePool, plan_cache
-    from atoma_infer_amd.engine import ModelRunner, StepEntry
+    from atoma_infer_amd.cache import plan_cache
     from atoma_infer_amd.models import load_model
     model = load_model(toy_dir, dtype)
     plan = plan_cache(model.spec)
@@ -423,47 +519,53 @@ def test_toy_architecture_steps_like_its_plain_model(toy_dir, dtype):
     reqs = {n: random_tokens(ln, TOY["vocab"], 60 + i) for i, (n, ln) in enumerate([("a", 120), ("b", 75), ("c", 90)])}
     want = {n: toy_plain_forward(t, w, TOY) for n, t in reqs.items()}
 
-    def run(schedule, pages):
-        pool = CachePool(plan, 16, pages, 3, model.act_dtype, model.device)
-        runner = ModelRunner(model, pool)
-        ids, got = {}, {}
-        for entries, end in schedule:
-            batch, places = [], []
-            for name, n in entries:
-                if name not in ids:
-                    ids[name] = len(ids)
-                    runner.add_request(ids[name])
-                s = runner.computed_len(ids[name])
-                batch.append(StepEntry(ids[name], reqs[name][s:s + n], s, list(range(n))))
-                places += [(name, s + i) for i in range(n)]
-            logits = runner.step(batch).cpu()
-            for r, key in enumerate(places):
-                got[key] = logits[r]
-            for name in end:
-                runner.free_request(ids[name])
-            runner.manager.check()
-        return got, runner
-
-    def check(got):
-        for n in reqs:
-            rows = sorted(p for (m, p) in got if m == n)
-            mine, ref = torch.stack([got[(n, p)] for p in rows]), want[n][rows]
-            if dtype == "float32":
-                assert rel_err(mine, ref) < TOL_F32, n
-            else:
-                assert frob_err(mine, ref) < TOL_BF16, n
-
     # whole prompts, one request at a time
-    got, _ = run([([(n, len(t))], [n]) for n, t in reqs.items()], [8, 8])
-    check(got)
+    got, _ = _toy_run(model, plan, reqs, [([(n, len(t))], [n]) for n, t in reqs.items()], [8, 8])
+    _toy_check(got, want, dtype)
     # portions of changing size beside decoded tokens of other requests; the windowed group has so few pages
     # (12 of 16 tokens, where the three requests would need 19 without giving any back) that it only works because passed pages return
     sched = [([("a", 50), ("b", 2)], []), ([("a", 1), ("b", 33), ("c", 17)], []), ([("a", 30), ("c", 2)], []),
              ([("b", 40), ("a", 1), ("c", 1)], ["b"]), ([("a", 38), ("c", 3)], ["a"]), ([("c", 60)], []),
              ([("c", 1)], []), ([("c", 1)], []), ([("c", 5)], ["c"])]
-    got, runner = run(sched, [19, 12])
-    check(got)
+    got, runner = _toy_run(model, plan, reqs, sched, [19, 12])
+    _toy_check(got, want, dtype)
     assert runner.manager.num_free_pages(0) == 19 and runner.manager.num_free_pages(1) == 12
+
+
+@pytest.fixture(scope="module")
+def routed_dir(tmp_path_factory, toy_dir):
+    from atoma_infer_amd.weights import write_random_model
+    d = str(tmp_path_factory.mktemp("toy_routed"))
+    write_random_model(d, TOY_ROUTED, seed=9, dtype="bfloat16", norm_jitter=0.1)
+    return d
+
+
+def test_routed_feed_forward_and_steps_that_cannot_be_replayed(routed_dir):
+    """A feed-forward with routing, and single decoded tokens of requests that take turns: the toy parts read the
+    step on the host, so such steps must not be recorded into a graph with one request's state slot in it."""
+    from atoma_infer_amd.cache import plan_cache
+    from atoma_infer_amd.models import load_model, random_model
+    w = plain_weights(routed_dir)
+    reqs = {n: random_tokens(ln, TOY_ROUTED["vocab"], 80 + i) for i, (n, ln) in enumerate([("a", 70), ("b", 41)])}
+    want = {n: toy_plain_forward(t, w, TOY_ROUTED) for n, t in reqs.items()}
+    turns = [([("a", 60), ("b", 32)], [])] + [([(n, 1)], []) for _ in range(8) for n in ("a", "b")] \
+        + [([("a", 2), ("b", 1)], ["a", "b"])]
+    model = load_model(routed_dir, "float32")
+    assert not model.spec.graph_safe()
+    plan = plan_cache(model.spec)
+    got, runner = _toy_run(model, plan, reqs, [([(n, len(t))], [n]) for n, t in reqs.items()], [8, 8])
+    _toy_check(got, want, "float32")
+    assert not runner.use_graphs
+    got, _ = _toy_run(model, plan, reqs, turns, [8, 8])
+    _toy_check(got, want, "float32")
+    # bfloat16: the same steps against whole prompts of the same engine
+    model = load_model(routed_dir, "bfloat16")
+    whole, _ = _toy_run(model, plan, reqs, [([(n, len(t))], [n]) for n, t in reqs.items()], [8, 8])
+    got, _ = _toy_run(model, plan, reqs, turns, [8, 8])
+    for key, row in got.items():
+        assert frob_err(row[None], whole[key][None]) < TOL_BF16, key
+    # the architecture this framework serves is made of parts that can be replayed
+    assert random_model(TINY_B, seed=1, dtype="bfloat16").spec.graph_safe()
 
 
 def test_toy_architecture_generates_through_the_engine(toy_dir):
