@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine at Llama-3.2-1B sizes with random weights, on one GPU.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--sizes 1b|3b|8b] [--layers N]
 
 A "step" is one decode step of the whole engine (scheduler, step function, sampler).  The default run has the
 layer sizes of Llama-3.2-1B (16 layers, width 2048, 32 heads over 8 KV heads of 64, feed-forward 8192, vocabulary
@@ -29,7 +29,14 @@ LLAMA_1B = {
                      "original_max_position_embeddings": 8192, "rope_type": "llama3"},
     "max_position_embeddings": 131072, "tie_word_embeddings": True,
 }
-FULL_LAYERS = 16
+# other members of the family, for measurements beside the default (``--sizes``): what differs from LLAMA_1B
+OTHER_SIZES = {
+    "3b": dict(hidden_size=3072, num_attention_heads=24, num_key_value_heads=8, intermediate_size=8192,
+               num_hidden_layers=28),
+    "8b": dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, intermediate_size=14336,
+               num_hidden_layers=32, tie_word_embeddings=False,
+               rope_scaling=dict(LLAMA_1B["rope_scaling"], factor=8.0)),
+}
 
 
 def log(msg):
@@ -109,7 +116,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--sizes", choices=["1b", "3b", "8b"], default="1b",
+                    help="layer sizes of Llama-3.2-1B (the default run), Llama-3.2-3B or Llama-3.1-8B")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (default: all)")
     ap.add_argument("--prompt-len", type=int, default=2048)
     ap.add_argument("--context", type=int, default=8192)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -130,7 +139,11 @@ def main() -> int:
     from atoma_infer_amd.cache import plan_cache
     from atoma_infer_amd.models import random_model
 
-    cfg = dict(LLAMA_1B, num_hidden_layers=args.layers)
+    base = dict(LLAMA_1B, **OTHER_SIZES.get(args.sizes, {}))
+    full_layers = base["num_hidden_layers"]
+    args.layers = args.layers or full_layers
+    cfg = dict(base, num_hidden_layers=args.layers)
+    name = {"1b": "Llama-3.2-1B", "3b": "Llama-3.2-3B", "8b": "Llama-3.1-8B"}[args.sizes]
     log(f"building the model ({args.layers} layers, random weights) ...")
     t0 = time.time()
     model = random_model(cfg, seed=0, dtype="bfloat16", stored="bfloat16")
@@ -167,16 +180,17 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * st / d, 1)
 
     line = {
-        "metric": "decode tok/s at batch 8 (Llama-3.2-1B sizes, 2048-token prompts); points: batch 1 and 64; "
-                  "prefill tok/s at 2048 tokens",
+        "metric": f"decode tok/s at batch {args.batch} ({name} sizes, {args.prompt_len}-token prompts); "
+                  "points: batch 1 and 64; prefill tok/s at 2048 tokens",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (uniform random token ids, random weights N(0, 0.02))",
-        "config": {"model": "Llama-3.2-1B sizes", "layers": args.layers, "layers_full": FULL_LAYERS,
+        "config": {"model": name + " sizes",
+                   "layers": args.layers, "layers_full": full_layers,
                    "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
                    "head_dim": hd, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
                    "global_batch": args.batch, "seq_len": args.prompt_len, "context": args.context,
-                   "mean_decode_context": round(mean_ctx, 1), "kv_block": 16, "tied_embeddings": True,
+                   "mean_decode_context": round(mean_ctx, 1), "kv_block": 16, "tied_embeddings": bool(base["tie_word_embeddings"]),
                    "parallelism": "single GPU"},
         "prefill": prefill, "roofline": roofline, "points": points,
     }
