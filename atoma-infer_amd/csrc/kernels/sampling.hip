@@ -1,4 +1,5 @@
-// Sampling from float32 logits, one block of 1024 threads per row:
+// Sampling from float32 logits, one block of 1024 threads per row (two walks over the row without a cut, five or
+// six with top-k or top-p):
 //   greedy (temperature <= 0): argmax, lowest index on ties;
 //   else weights w_i = exp((l_i - max) / T), optionally cut to the k largest and then to the smallest set of
 //   largest weights whose mass reaches top_p of the whole, ties towards the lower index; the token is the first
@@ -7,7 +8,7 @@
 // The reference samples on the host with candle's LogitsProcessor in the modes All / TopK / TopP / TopKThenTopP
 // (backends/vllm/src/llm_service.rs:346-372, model_executor.rs:231-235) and applies a repeat penalty to the
 // last repeat_last_n tokens first (model_executor.rs:211-225).
-// All reductions run in an order fixed by the vocabulary size alone, so a row's draw does not depend on the batch.
+// Masses are summed as integers (see fixed_of), so a row's draw depends on nothing but the row.
 #include "common.h"
 
 using namespace atoma;
@@ -41,26 +42,88 @@ __device__ ArgMax block_argmax(ArgMax a, ArgMax* scratch) {
   return r;
 }
 
-// sum of a float and of an int over the block, both in one pass
-__device__ void block_sum2(float& f, int& n, float* fs, int* ns) {
-  f = wave_sum(f);
+// Kept weights are summed as integers, in units of 2^-40 of the largest weight (which is 1): integer sums do not
+// depend on their order, so thresholds, kept mass and the draw are exact functions of the row, whatever the
+// number of threads or the order in which they add.
+typedef unsigned long long u64;
+// w * 2^40 cut to an integer, as hi * 2^20 + lo, in two exact steps of 20 bits (there is no single
+// float-to-64-bit instruction; sums of a few thousand hi or lo parts fit 32 bits)
+__device__ __forceinline__ void fixed_parts(float w, uint32_t& hi, uint32_t& lo) {
+  const float a = w * 1048576.0f;
+  hi = (uint32_t)a;
+  lo = (uint32_t)((a - (float)hi) * 1048576.0f);
+}
+__device__ __forceinline__ u64 fixed_of(float w) {
+  uint32_t hi, lo;
+  fixed_parts(w, hi, lo);
+  return ((u64)hi << 20) + lo;
+}
+
+constexpr int kBins = kSampThreads;             // one histogram bin per thread
+constexpr int kSlices = 8;                      // per wave, for the draw
+
+template <typename T> __device__ __forceinline__ T wave_total(T v) {
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) n += __shfl_xor(n, o, 64);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// inclusive prefix sums over the lanes of a wave
+template <typename T> __device__ __forceinline__ T wave_prefix(T v) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const T up = __shfl_up(v, o, 64);
+    if (lane >= o) v += up;
+  }
+  return v;
+}
+
+// f(value, index) for every element of x[0, n): groups of four neighbours per thread where the row allows
+// 16-byte loads
+template <typename F> __device__ __forceinline__ void sweep(const float* __restrict__ x, int n, F f) {
+  const int tid = threadIdx.x;
+  if ((((uintptr_t)x) & 15) == 0) {
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const int n4 = n >> 2;
+#pragma unroll 4
+    for (int i = tid; i < n4; i += kSampThreads) {
+      const float4 v = x4[i];
+      f(v.x, 4 * i);
+      f(v.y, 4 * i + 1);
+      f(v.z, 4 * i + 2);
+      f(v.w, 4 * i + 3);
+    }
+    for (int i = (n4 << 2) + tid; i < n; i += kSampThreads) f(x[i], i);
+  } else {
+    for (int i = tid; i < n; i += kSampThreads) f(x[i], i);
+  }
+}
+
+// The highest bin b whose suffix sum hist[b] + hist[b + 1] + ... reaches target (0 < target <= sum of all bins),
+// and what of target is left for bin b itself.  Thread t looks at bin t.  sel < 0 if no bin does.
+template <typename T>
+__device__ void select_bin(const T* hist, T target, int& sel, T& rest, T* wave_sums, int* sel_s, T* rest_s) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T mine = hist[tid];
+  T suffix = mine;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const T down = __shfl_down(suffix, o, 64);
+    if (lane + o < 64) suffix += down;
+  }
+  if (lane == 0) wave_sums[wave] = suffix;
+  if (tid == 0) *sel_s = -1;
   __syncthreads();
-  if (lane == 0) {
-    fs[wave] = f;
-    ns[wave] = n;
+  for (int w2 = wave + 1; w2 < kSampWaves; ++w2) suffix += wave_sums[w2];
+  if (suffix >= target && suffix - mine < target) {      // suffix sums fall with t: one bin at most
+    *sel_s = tid;
+    *rest_s = target - (suffix - mine);
   }
   __syncthreads();
-  float ft = 0.f;
-  int nt = 0;
-  for (int i = 0; i < kSampWaves; ++i) {
-    ft += fs[i];
-    nt += ns[i];
-  }
-  f = ft;
-  n = nt;
+  sel = *sel_s;
+  rest = sel >= 0 ? *rest_s : target;
+  __syncthreads();
 }
 
 __global__ void __launch_bounds__(kSampThreads)
@@ -68,32 +131,23 @@ sample_kernel(const float* __restrict__ logits, int ld, int vocab, const float* 
               const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
               float* __restrict__ weights, int32_t* __restrict__ out_token, float* __restrict__ out_logit) {
   __shared__ ArgMax am[kSampWaves];
-  __shared__ float fs[kSampWaves];
-  __shared__ int ns[kSampWaves];
-  __shared__ float scan_f[kSampThreads];
-  __shared__ int scan_n[kSampThreads];
-  __shared__ int chosen;
+  __shared__ uint32_t hist_k[kBins];       // top-k search: how many weights fall into each bin
+  __shared__ uint32_t hist_pn[kBins];      // top-p search: how many, and their mass
+  __shared__ u64 hist_pm[kBins];
+  __shared__ u64 wave_u64[kSampWaves];
+  __shared__ uint32_t wave_u32[kSampWaves];
+  __shared__ u64 slice_mass[kSampWaves * kSlices];
+  __shared__ uint32_t slice_rank[kSampWaves * kSlices];
+  __shared__ int sel_s;
+  __shared__ u64 rest_u64;
+  __shared__ uint32_t rest_u32;
 
-  const int row = blockIdx.x, tid = threadIdx.x;
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* lr = logits + (size_t)row * ld;
   float* w = weights + (size_t)row * vocab;
 
   ArgMax a = {-INFINITY, 0x7fffffff};
-  if ((vocab & 3) == 0 && (((uintptr_t)lr) & 15) == 0) {
-    // four values per load, several loads in flight
-    const float4* l4 = reinterpret_cast<const float4*>(lr);
-    const int n4 = vocab >> 2;
-#pragma unroll 4
-    for (int i = tid; i < n4; i += kSampThreads) {
-      const float4 v = l4[i];
-      a = better(a, ArgMax{v.x, 4 * i});
-      a = better(a, ArgMax{v.y, 4 * i + 1});
-      a = better(a, ArgMax{v.z, 4 * i + 2});
-      a = better(a, ArgMax{v.w, 4 * i + 3});
-    }
-  } else {
-    for (int i = tid; i < vocab; i += kSampThreads) a = better(a, ArgMax{lr[i], i});
-  }
+  sweep(lr, vocab, [&](float v, int i) { a = better(a, ArgMax{v, i}); });
   a = block_argmax(a, am);
   const float temp = temperature[row];
   if (!(temp > 0.f)) {
@@ -104,136 +158,308 @@ sample_kernel(const float* __restrict__ logits, int ld, int vocab, const float* 
     return;
   }
 
-  // weights and their total
-  const float inv_t = 1.0f / temp;
-  float total = 0.f;
-  int dummy = 0;
-  for (int i = tid; i < vocab; i += kSampThreads) {
-    const float wi = expf((lr[i] - a.v) * inv_t);
-    w[i] = wi;
-    total += wi;
-  }
-  block_sum2(total, dummy, fs, ns);
-  __syncthreads();  // w written by other threads is read below
-
-  // Threshold tau (as float bits; weights are non-negative so bit order is value order) and the number of
-  // weights equal to tau that are kept (those of lowest index).  Everything above tau is kept.
-  uint32_t tau = 0;            // keep all: w >= 0
-  int ties_kept = 0x7fffffff;  // all ties
   const int k = top_k[row];
   const float p = top_p[row];
-  if (k > 0 && k < vocab) {
-    uint32_t prefix = 0;
-    for (int bit = 30; bit >= 0; --bit) {
-      const uint32_t cand = prefix | (1u << bit);
-      int cnt = 0;
-      float f0 = 0.f;
-      for (int i = tid; i < vocab; i += kSampThreads) cnt += (__float_as_uint(w[i]) >= cand);
-      block_sum2(f0, cnt, fs, ns);
-      if (cnt >= k) prefix = cand;
-    }
-    int gt = 0;
-    float f0 = 0.f;
-    for (int i = tid; i < vocab; i += kSampThreads) gt += (__float_as_uint(w[i]) > prefix);
-    block_sum2(f0, gt, fs, ns);
-    tau = prefix;
-    ties_kept = k - gt;
-  }
-  if (p < 1.0f) {
-    const float need = p * total;
-    uint32_t prefix = 0;
-    for (int bit = 30; bit >= 0; --bit) {
-      const uint32_t cand = prefix | (1u << bit);
-      float mass = 0.f;
-      int n0 = 0;
-      for (int i = tid; i < vocab; i += kSampThreads) mass += (__float_as_uint(w[i]) >= cand) ? w[i] : 0.f;
-      block_sum2(mass, n0, fs, ns);
-      if (mass >= need) prefix = cand;
-    }
-    float mass_gt = 0.f;
-    int n_eq = 0;
-    for (int i = tid; i < vocab; i += kSampThreads) {
-      const uint32_t b = __float_as_uint(w[i]);
-      mass_gt += (b > prefix) ? w[i] : 0.f;
-      n_eq += (b == prefix);
-    }
-    block_sum2(mass_gt, n_eq, fs, ns);
-    const float tv = __uint_as_float(prefix);
-    int ties = n_eq;
-    if (tv > 0.f) {
-      ties = (int)ceilf((need - mass_gt) / tv);
-      if (ties < 1) ties = 1;
-      if (ties > n_eq) ties = n_eq;
-    }
-    // the tighter of the two cuts wins
-    if (prefix > tau || (prefix == tau && ties < ties_kept)) {
-      tau = prefix;
-      ties_kept = ties;
-    }
-  }
+  const bool cut_k = k > 0 && k < vocab, cut_p = p < 1.0f, cut = cut_k || cut_p;
 
-  // Each thread owns a contiguous span of the vocabulary; scan kept mass and tie counts over spans.
-  const int span = (vocab + kSampThreads - 1) / kSampThreads;
-  const int lo = tid * span, hi = (lo + span < vocab) ? lo + span : vocab;
-  int my_ties = 0;
-  for (int i = lo; i < hi; ++i) my_ties += (__float_as_uint(w[i]) == tau);
-  scan_n[tid] = my_ties;
-  __syncthreads();
-  if (tid == 0) {
-    int run = 0;
-    for (int i = 0; i < kSampThreads; ++i) {
-      const int c = scan_n[i];
-      scan_n[i] = run;
-      run += c;
+  // Each wave owns a contiguous stretch of the vocabulary, cut into kSlices slices of whole pieces of 256 values
+  // (four neighbours a lane, fetched four pieces at a time: a wave walks at the pace of its loads).
+  const int stretch = ((vocab + kSampWaves * 256 - 1) / (kSampWaves * 256)) * 256;
+  const int slice_len = ((stretch / 256 + kSlices - 1) / kSlices) * 256;
+  const int begin = wave * stretch, end = begin + stretch < vocab ? begin + stretch : vocab;
+  const bool vec_l = (((uintptr_t)lr) & 15) == 0, vec_w = (((uintptr_t)w) & 15) == 0;
+  // the lane's four values of the piece of x at `at`, up to `stop`; how many exist
+  auto piece = [&](const float* x, bool vec, int at, int stop, float* v) -> int {
+    const int i = at + lane * 4;
+    const int n = stop - i < 0 ? 0 : stop - i > 4 ? 4 : stop - i;
+    if (n == 4 && vec) {
+      const float4 q = *reinterpret_cast<const float4*>(x + i);
+      v[0] = q.x, v[1] = q.y, v[2] = q.z, v[3] = q.w;
+    } else {
+      for (int e = 0; e < 4; ++e) v[e] = e < n ? x[i + e] : 0.f;
     }
-  }
+    return n;
+  };
+  auto slice_range = [&](int sl, int& s_begin, int& s_end) {
+    s_begin = begin + sl * slice_len;
+    s_end = s_begin + slice_len < end ? s_begin + slice_len : end;
+  };
+
+  // Weights w = exp((l - max) / T) = 2^((l - max) * log2(e) / T), largest = 1: one multiply and the hardware's
+  // exp2.  The same walk fills what the next step needs: with a cut, the histograms of the first ten bits and the
+  // total; without, the kept mass of every slice (everything is kept).
+  hist_k[tid] = 0;
+  hist_pn[tid] = 0;
+  hist_pm[tid] = 0;
   __syncthreads();
-  int rank = scan_n[tid];
-  float my_mass = 0.f;
-  for (int i = lo; i < hi; ++i) {
-    const uint32_t b = __float_as_uint(w[i]);
-    const bool keep = b > tau || (b == tau && rank < ties_kept);
-    rank += (b == tau);
-    my_mass += keep ? w[i] : 0.f;
-  }
-  scan_f[tid] = my_mass;
-  if (tid == 0) chosen = -1;
-  __syncthreads();
-  if (tid == 0) {
-    float run = 0.f;
-    for (int i = 0; i < kSampThreads; ++i) {
-      const float c = scan_f[i];
-      scan_f[i] = run;
-      run += c;
-    }
-    fs[0] = run;  // kept mass
-  }
-  __syncthreads();
-  const float target = uniform[row] * fs[0];
-  const float before = scan_f[tid];
-  // the span that contains the target walks it; the last kept token catches a target at the very end
-  if (my_mass > 0.f && before <= target && (target < before + my_mass)) {
-    float run = before;
-    int r = scan_n[tid], pick = -1, last_kept = -1;
-    for (int i = lo; i < hi; ++i) {
-      const uint32_t b = __float_as_uint(w[i]);
-      const bool keep = b > tau || (b == tau && r < ties_kept);
-      r += (b == tau);
-      if (!keep) continue;
-      last_kept = i;
-      run += w[i];
-      if (run > target) {
-        pick = i;
-        break;
+  const float inv_t = 1.4426950408889634f / temp;
+  uint32_t total_hi = 0, total_lo = 0;
+  for (int sl = 0; sl < kSlices; ++sl) {
+    int s_begin, s_end;
+    slice_range(sl, s_begin, s_end);
+    uint32_t hi_sum = 0, lo_sum = 0;
+    for (int at0 = s_begin; at0 < s_end; at0 += 4 * 256) {
+      float vs[4][4];
+      int ns[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ns[j] = piece(lr, vec_l, at0 + j * 256, s_end, vs[j]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = at0 + j * 256 + lane * 4, n = ns[j];
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o[e] = __builtin_amdgcn_exp2f((vs[j][e] - a.v) * inv_t);
+          if (e >= n) continue;
+          uint32_t hi, lo;
+          fixed_parts(o[e], hi, lo);
+          hi_sum += hi;
+          lo_sum += lo;
+          if (cut) {
+            const uint32_t bin = (__float_as_uint(o[e]) >> 20) & (kBins - 1);
+            if (cut_k) atomicAdd(&hist_k[bin], 1u);
+            if (cut_p) {
+              atomicAdd(&hist_pn[bin], 1u);
+              atomicAdd(&hist_pm[bin], ((u64)hi << 20) + lo);
+            }
+          }
+        }
+        if (n == 4 && vec_w) {
+          *reinterpret_cast<float4*>(w + i) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+          for (int e = 0; e < n; ++e) w[i + e] = o[e];
+        }
       }
     }
-    if (pick < 0) pick = last_kept;
-    atomicMax(&chosen, pick);
+    if (!cut) {
+      const u64 mass = wave_total(((u64)hi_sum << 20) + lo_sum);
+      if (lane == 0) slice_mass[wave * kSlices + sl] = mass;
+    }
+    total_hi += hi_sum;
+    total_lo += lo_sum;
+  }
+  u64 total = 0;
+  if (cut_p) {
+    total = wave_total(((u64)total_hi << 20) + total_lo);
+    if (lane == 0) wave_u64[wave] = total;
+  }
+  __syncthreads();          // w and the histograms written by other threads are read below
+  if (cut_p) {
+    total = 0;
+    for (int i = 0; i < kSampWaves; ++i) total += wave_u64[i];
+    __syncthreads();
+  }
+
+  // The cut: a threshold tau (as float bits; weights are non-negative, so bit order is value order) above which
+  // everything is kept, and the number of weights equal to tau that are kept (those of lowest index).  Both
+  // searches walk down the bits of tau ten at a time: a histogram over the next ten bits of the weights that
+  // share the bits found so far, then the highest bin whose suffix reaches what is still wanted.  A weight is at
+  // most 1 = 0x3f800000, so 30 bits suffice.
+  uint32_t bits_k = 0, bits_p = 0;       // the bits of the two thresholds found so far
+  uint32_t want_k = cut_k ? (uint32_t)k : 0u, equal_k = 0, equal_p = 0;
+  u64 want_p = 0;
+  if (cut_p) {
+    const double need = ceil((double)p * (double)total);
+    want_p = need < 1.0 ? 1ull : (u64)need;
+    if (want_p > total) want_p = total;
+  }
+  if (cut) {
+#pragma unroll 1
+    for (int level = 0; level < 3; ++level) {
+      const int shift = 20 - 10 * level;
+      if (level > 0) {                     // (the first histograms were filled with the weights)
+        hist_k[tid] = 0;
+        hist_pn[tid] = 0;
+        hist_pm[tid] = 0;
+        __syncthreads();
+        sweep(w, vocab, [&](float v, int) {
+          const uint32_t b = __float_as_uint(v);
+          const uint32_t high = b >> (shift + 10), bin = (b >> shift) & (kBins - 1);
+          if (cut_k && high == bits_k) atomicAdd(&hist_k[bin], 1u);
+          if (cut_p && high == bits_p) {
+            atomicAdd(&hist_pn[bin], 1u);
+            atomicAdd(&hist_pm[bin], fixed_of(v));
+          }
+        });
+        __syncthreads();
+      }
+      int sel;
+      if (cut_k) {
+        select_bin<uint32_t>(hist_k, want_k, sel, want_k, wave_u32, &sel_s, &rest_u32);
+        if (sel < 0) sel = 0, want_k = 0x7fffffff;          // cannot happen: k < vocab weights exist
+        bits_k = (bits_k << 10) | (uint32_t)sel;
+        equal_k = hist_k[sel];
+      }
+      if (cut_p) {
+        select_bin<u64>(hist_pm, want_p, sel, want_p, wave_u64, &sel_s, &rest_u64);
+        if (sel < 0) sel = 0;                               // cannot happen: want_p <= total
+        bits_p = (bits_p << 10) | (uint32_t)sel;
+        equal_p = hist_pn[sel];
+      }
+      __syncthreads();
+    }
+  }
+  uint32_t tau = 0, n_equal = 0xffffffffu;
+  u64 ties_kept = ~0ull;                 // all of them
+  if (cut_k) {
+    tau = bits_k;
+    ties_kept = want_k;                  // what the weights above tau leave of k
+    n_equal = equal_k;
+  }
+  if (cut_p) {
+    // as many ties as it takes to reach the mass still wanted
+    const u64 each = fixed_of(__uint_as_float(bits_p));
+    u64 ties = each ? (want_p + each - 1) / each : (u64)equal_p;
+    if (ties < 1) ties = 1;
+    if (ties > equal_p) ties = equal_p;
+    if (!cut_k || bits_p > tau || (bits_p == tau && ties < ties_kept)) {     // the tighter of the two cuts wins
+      tau = bits_p;
+      ties_kept = ties;
+      n_equal = equal_p;
+    }
+  }
+  const bool all_ties = ties_kept >= (u64)n_equal;
+
+  // The draw: the first index, in vocabulary order, at which the running sum of kept weights exceeds
+  // u * (kept mass).  A tie's rank is the number of ties before it.  A walk over the weights leaves every slice's
+  // kept mass (and the rank at its start) in LDS; the slice that holds the target is then walked again with
+  // running sums over its lanes.
+  // the kept mass of the lane's values of one piece, in two parts; rank: ties before the lane's first value
+  auto lane_mass = [&](const float* v, int n, uint32_t rank, bool* keep, uint32_t& hi_sum, uint32_t& lo_sum) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t b = __float_as_uint(v[e]);
+      keep[e] = e < n && (b > tau || (b == tau && (all_ties || (u64)rank < ties_kept)));
+      if (e < n && b == tau) ++rank;
+      if (keep[e]) {
+        uint32_t hi, lo;
+        fixed_parts(v[e], hi, lo);
+        hi_sum += hi;
+        lo_sum += lo;
+      }
+    }
+  };
+  auto lane_ties = [&](const float* v, int n) -> uint32_t {
+    uint32_t ties = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ties += e < n && __float_as_uint(v[e]) == tau;
+    return ties;
+  };
+
+  if (cut) {
+    uint32_t rank_run = 0;               // ties before the piece at hand
+    if (!all_ties) {
+      uint32_t mine = 0;
+      for (int at0 = begin; at0 < end; at0 += 4 * 256) {
+        float vs[4][4];
+        int ns[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ns[j] = piece(w, vec_w, at0 + j * 256, end, vs[j]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mine += lane_ties(vs[j], ns[j]);
+      }
+      mine = wave_total(mine);
+      if (lane == 0) wave_u32[wave] = mine;
+      __syncthreads();
+      for (int i = 0; i < wave; ++i) rank_run += wave_u32[i];
+      __syncthreads();
+    }
+    for (int sl = 0; sl < kSlices; ++sl) {
+      int s_begin, s_end;
+      slice_range(sl, s_begin, s_end);
+      if (lane == 0) slice_rank[wave * kSlices + sl] = rank_run;
+      uint32_t hi_sum = 0, lo_sum = 0;
+      for (int at0 = s_begin; at0 < s_end; at0 += 4 * 256) {
+        float vs[4][4];
+        int ns[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ns[j] = piece(w, vec_w, at0 + j * 256, s_end, vs[j]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t rank = 0;
+          if (!all_ties) {
+            const uint32_t ties = lane_ties(vs[j], ns[j]);
+            const uint32_t incl = wave_prefix(ties);
+            rank = rank_run + incl - ties;
+            rank_run += __shfl(incl, 63, 64);
+          }
+          bool keep[4];
+          lane_mass(vs[j], ns[j], rank, keep, hi_sum, lo_sum);
+        }
+      }
+      const u64 mass = wave_total(((u64)hi_sum << 20) + lo_sum);
+      if (lane == 0) slice_mass[wave * kSlices + sl] = mass;
+    }
+  } else if (lane == 0) {
+    for (int sl = 0; sl < kSlices; ++sl) slice_rank[wave * kSlices + sl] = 0;
   }
   __syncthreads();
-  if (tid == 0) {
-    int c = chosen;
-    if (c < 0) c = a.i;  // rounding left the target beyond every span: fall back to the most likely token
+
+  // which slice holds the target: running sums over the slices, one slice a thread
+  constexpr int kAllSlices = kSampWaves * kSlices;
+  static_assert(kAllSlices <= kSampThreads && kAllSlices % 64 == 0, "one slice a thread");
+  const u64 mine = tid < kAllSlices ? slice_mass[tid] : 0;
+  const u64 incl = wave_prefix(mine);
+  if (lane == 63) wave_u64[wave] = incl;
+  if (tid == 0) sel_s = -1;
+  __syncthreads();
+  u64 before = incl - mine, kept = 0;
+  for (int i = 0; i < kAllSlices / 64; ++i) {
+    if (i < wave) before += wave_u64[i];
+    kept += wave_u64[i];
+  }
+  u64 target = (u64)((double)uniform[row] * (double)kept);
+  if (target >= kept) target = kept - 1;           // (kept >= 2^40: the largest weight is always kept)
+  if (tid < kAllSlices && before <= target && target < before + mine) {
+    sel_s = tid;
+    rest_u64 = before;
+  }
+  __syncthreads();
+  const int slice = sel_s;
+  if (slice < 0 || slice / kSlices != wave) return;         // (one slice does: kept > target)
+  u64 run = rest_u64;
+  uint32_t rank_at = slice_rank[slice];
+  int s_begin, s_end;
+  slice_range(slice % kSlices, s_begin, s_end);
+  int pick = -1;
+  for (int at = s_begin; at < s_end; at += 256) {
+    float v[4];
+    const int n = piece(w, vec_w, at, s_end, v);
+    uint32_t rank = 0;
+    if (!all_ties) {
+      const uint32_t ties = lane_ties(v, n);
+      const uint32_t ti = wave_prefix(ties);
+      rank = rank_at + ti - ties;
+      rank_at += __shfl(ti, 63, 64);
+    }
+    bool keep[4];
+    uint32_t hi_sum = 0, lo_sum = 0;
+    lane_mass(v, n, rank, keep, hi_sum, lo_sum);
+    const u64 lm = ((u64)hi_sum << 20) + lo_sum;
+    const u64 li = wave_prefix(lm);
+    const u64 whole = __shfl(li, 63, 64);
+    if (run + whole > target) {
+      const u64 ahead = __ballot(run + li > target);
+      const int first = __ffsll((long long)ahead) - 1;
+      int found = -1;
+      if (lane == first) {
+        u64 r = run + li - lm;
+        for (int e = 0; e < 4; ++e) {
+          if (!keep[e]) continue;
+          r += fixed_of(v[e]);
+          if (r > target) {
+            found = at + lane * 4 + e;
+            break;
+          }
+        }
+      }
+      pick = __shfl(found, first, 64);
+      break;
+    }
+    run += whole;
+  }
+  if (lane == 0) {
+    const int c = pick >= 0 ? pick : a.i;
     out_token[row] = c;
     out_logit[row] = lr[c];
   }

@@ -132,15 +132,20 @@ def test_eos_stops_and_too_long_is_ignored(model_dirs):
 # the sampling kernel against the plain sampling functions
 
 
-@pytest.mark.parametrize("vocab", [331, 1000, 5000])
+@pytest.mark.parametrize("vocab", [331, 1000, 5000, 50001, 128256])
 def test_sample_kernel(vocab):
+    """Rows of a batch against the plain distribution and draw; 50001 leaves all rows but the first unaligned, 128256
+    is a real vocabulary (every wave of the kernel has several slices of several pieces)."""
     from atoma_infer_amd.kernels import ops
     g = torch.Generator().manual_seed(vocab)
     rows = [(0.0, 0, 1.0), (0.7, 0, 1.0), (1.3, 5, 1.0), (0.7, 0, 0.6), (0.9, 20, 0.8), (0.5, 1, 1.0), (2.0, 0, 0.999)]
     logits = torch.randn(len(rows), vocab, generator=g) * 2.0
     logits[2, 10] = logits[2, 20] = logits[2].max() + 1.0        # ties at the top
+    dists = [None if t == 0.0 else plain_llama.sampling_distribution(logits[i], t, k, p)
+             for i, (t, k, p) in enumerate(rows)]
+    cdfs = [None if d is None else torch.cumsum(d.double(), 0) / d.double().sum() for d in dists]
+    dev = lambda x, dt: torch.tensor(x, dtype=dt, device="cuda:0")
     for u in (0.0, 0.013, 0.25, 0.5, 0.77, 0.999):
-        dev = lambda x, dt: torch.tensor(x, dtype=dt, device="cuda:0")
         tok, lg = ops.sample(logits.cuda(), dev([r[0] for r in rows], torch.float32),
                              dev([r[1] for r in rows], torch.int32), dev([r[2] for r in rows], torch.float32),
                              dev([u] * len(rows), torch.float32))
@@ -149,14 +154,35 @@ def test_sample_kernel(vocab):
             if t == 0.0:
                 assert tok[i] == int(torch.argmax(logits[i]))
                 continue
-            dist = plain_llama.sampling_distribution(logits[i], t, k, p)
-            want = plain_llama.draw(dist, u)
-            assert dist[tok[i]] > 0, f"row {i}: token {tok[i]} is outside the kept set"
+            want = plain_llama.draw(dists[i], u)
+            assert dists[i][tok[i]] > 0, f"row {i}: token {tok[i]} is outside the kept set"
             if tok[i] != want:
-                c = torch.cumsum(dist.double(), 0) / dist.double().sum()
                 lo, hi = sorted((tok[i], want))
-                assert abs(float(c[lo]) - u) < 1e-5 or abs(float(c[hi - 1]) - u) < 1e-5, (i, u, tok[i], want)
+                assert abs(float(cdfs[i][lo]) - u) < 1e-5 or abs(float(cdfs[i][hi - 1]) - u) < 1e-5, (i, u, tok[i], want)
             assert float(lg[i]) == float(logits[i, tok[i]])
+
+
+def test_sample_kernel_many_ties_in_a_large_vocabulary():
+    """Ties at the threshold that are only partly kept, spread over the stretches of several waves: the kept ones
+    are those of lowest index, and every kept token can be drawn."""
+    from atoma_infer_amd.kernels import ops
+    vocab = 40000
+    logits = torch.full((2, vocab), -3.0)
+    tied = list(range(5, vocab, 997))                   # 41 tied tokens across the vocabulary
+    logits[0, tied] = 2.0
+    logits[1, tied] = 2.0
+    logits[1, 123] = 4.0                                # one token above the ties
+    dev = lambda x, dt: torch.tensor(x, dtype=dt, device="cuda:0")
+    seen = [set(), set()]
+    n = 400
+    for i in range(n):
+        u = (i + 0.5) / n
+        tok, _ = ops.sample(logits.cuda(), dev([1.0, 1.0], torch.float32), dev([7, 12], torch.int32),
+                            dev([1.0, 1.0], torch.float32), dev([u, u], torch.float32))
+        for r, t in enumerate(tok.cpu().tolist()):
+            seen[r].add(t)
+    assert seen[0] == set(tied[:7])
+    assert seen[1] == {123} | set(tied[:11])
 
 
 def test_sample_kernel_kept_sets_and_ties():
