@@ -223,11 +223,12 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: 
     return out
 
 
-def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None):
+def sample_packed(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+                  uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per row of float32 ``logits`` [S, V]: argmax where temperature <= 0, else a draw (see sampling.hip).
 
-    Returns (tokens int32 [S], logits of the chosen tokens float32 [S]).
+    Returns one float32 tensor [2, S]: row 0 holds the tokens (int32 bits), row 1 the logits of the chosen tokens,
+    so that one copy brings both to the host.
     """
     _dev(logits, temperature, top_k, top_p, uniform)
     _need(logits.dim() == 2 and logits.dtype is torch.float32 and logits.stride(1) == 1, "logits must be float32 [S, V]")
@@ -239,11 +240,17 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
         workspace = torch.empty((s, v), dtype=torch.float32, device=logits.device)
     _need(workspace.dtype is torch.float32 and workspace.is_contiguous() and workspace.numel() >= s * v,
           "sample: workspace too small")
-    tok = torch.empty((s,), dtype=torch.int32, device=logits.device)
-    lg = torch.empty((s,), dtype=torch.float32, device=logits.device)
+    out = torch.empty((2, s), dtype=torch.float32, device=logits.device)
     _check(core().atoma_sample(_p(logits), logits.stride(0) if s > 1 else v, s, v, _p(temperature), _p(top_k),
-                               _p(top_p), _p(uniform), _p(workspace), _p(tok), _p(lg), _stream()), "sample")
-    return tok, lg
+                               _p(top_p), _p(uniform), _p(workspace), _p(out[0]), _p(out[1]), _stream()), "sample")
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None):
+    """``sample_packed`` as (tokens int32 [S], logits of the chosen tokens float32 [S])."""
+    out = sample_packed(logits, temperature, top_k, top_p, uniform, workspace)
+    return out[0].view(torch.int32), out[1]
 
 
 def repeat_penalty(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, penalty: torch.Tensor) -> None:

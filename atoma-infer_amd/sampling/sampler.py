@@ -75,10 +75,10 @@ class Sampler:
         if pen_rows:
             pen = torch.tensor([pen_rows, pen_toks], dtype=torch.int32).to(self.device)
             ops.repeat_penalty(logits, pen[0], pen[1], m[3])
-        tok, lg = ops.sample(logits, m[0], m[4].view(torch.int32), m[1], m[2])
+        out = ops.sample_packed(logits, m[0], m[4].view(torch.int32), m[1], m[2])
+        tok, lg = out[0].view(torch.int32), out[1]
         host = torch.empty((2, s), dtype=torch.float32, pin_memory=True)
-        host[0].copy_(tok.view(torch.float32), non_blocking=True)
-        host[1].copy_(lg, non_blocking=True)
+        host.copy_(out, non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
         pending = Pending(tok, lg, host, ev)
