@@ -53,7 +53,7 @@ def make_engine(model, batch, context, page=16):
                      validation=ValidationConfig(max_input_length=context - 1, max_total_tokens=context))
 
 
-def decode_run(model, batch, prompt_len, steps, warmup, context, seed=0):
+def decode_run(model, batch, prompt_len, steps, warmup, context, seed=0, sampling=None):
     """Prefill ``batch`` prompts (untimed), then time ``steps`` decode steps.  Returns (seconds, mean context)."""
     import torch
     from atoma_infer_amd.sampling import GenerateParameters
@@ -64,6 +64,10 @@ def decode_run(model, batch, prompt_len, steps, warmup, context, seed=0):
     prompt_steps = batch * (-(-prompt_len // max(2048, batch)))
     params = GenerateParameters(do_sample=False, max_new_tokens=steps + warmup + prompt_steps + 8,
                                 ignore_eos_token=True)
+    if sampling:        # (temperature, top_k, top_p): draw instead of the default argmax
+        params = GenerateParameters(do_sample=True, temperature=sampling[0], top_k=sampling[1] or None,
+                                    top_p=sampling[2] if sampling[2] < 1.0 else None,
+                                    random_seed=seed, max_new_tokens=params.max_new_tokens, ignore_eos_token=True)
     for _ in range(batch):
         eng.add_request(torch.randint(0, vocab, (prompt_len,), generator=g).tolist(), params)
     while any(r.in_prefill for r in eng.scheduler.running) or eng.scheduler.waiting:
@@ -123,6 +127,10 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=8192)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 runs")
+    ap.add_argument("--temperature", type=float, default=0.0,
+                    help="sample with this temperature (and --top-k, --top-p) instead of the default argmax")
+    ap.add_argument("--top-k", type=int, default=0)
+    ap.add_argument("--top-p", type=float, default=1.0)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
@@ -164,7 +172,9 @@ def main() -> int:
                "frac": round(pre_flops / pre_s / PEAK_FLOPS["bf16"], 4)}
 
     log(f"decode at batch {args.batch}: {args.warmup} warm-up + {args.steps} timed steps ...")
-    dt, mean_ctx = decode_run(model, args.batch, args.prompt_len, args.steps, args.warmup, args.context)
+    sampling = (args.temperature, args.top_k, args.top_p) if args.temperature > 0 else None
+    dt, mean_ctx = decode_run(model, args.batch, args.prompt_len, args.steps, args.warmup, args.context,
+                              sampling=sampling)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     step_bytes = model.weight_bytes() + kv_bytes_per_token * mean_ctx * args.batch
@@ -176,7 +186,7 @@ def main() -> int:
     if not args.no_points:
         for b, st in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
             log(f"decode at batch {b} ...")
-            d, _ = decode_run(model, b, args.prompt_len, st, min(args.warmup, 4), args.context)
+            d, _ = decode_run(model, b, args.prompt_len, st, min(args.warmup, 4), args.context, sampling=sampling)
             points[f"decode_b{b}"] = round(b * st / d, 1)
 
     line = {
@@ -190,7 +200,8 @@ def main() -> int:
                    "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
                    "head_dim": hd, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
                    "global_batch": args.batch, "seq_len": args.prompt_len, "context": args.context,
-                   "mean_decode_context": round(mean_ctx, 1), "kv_block": 16, "tied_embeddings": bool(base["tie_word_embeddings"]),
+                   "mean_decode_context": round(mean_ctx, 1), "kv_block": 16, "sampling": ("argmax" if not sampling else f"T={sampling[0]} top_k={sampling[1]} top_p={sampling[2]}"),
+                   "tied_embeddings": bool(base["tie_word_embeddings"]),
                    "parallelism": "single GPU"},
         "prefill": prefill, "roofline": roofline, "points": points,
     }
