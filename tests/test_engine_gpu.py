@@ -15,7 +15,7 @@ from util import (NORM_JITTER, TINY, TOL_BF16, TOL_F32, frob_err, make_model_dir
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-PAGE = {"A": 4, "B": 16, "C": 16, "D": 16}
+PAGE = {"A": 4, "B": 16, "C": 16, "D": 16, "E": 16}
 
 
 @pytest.fixture(scope="module")
@@ -97,7 +97,8 @@ def check_against_plain(model_dir, requests, got, dtype):
 
 
 def lengths(name):
-    return {"A": [100, 37, 64, 5], "B": [200, 1, 77, 130], "C": [150, 48, 97, 16], "D": [900, 300, 150, 40]}[name]
+    return {"A": [100, 37, 64, 5], "B": [200, 1, 77, 130], "C": [150, 48, 97, 16], "D": [900, 300, 150, 40],
+            "E": [600, 290, 33, 129]}[name]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -150,7 +151,8 @@ def test_mixed_batches_with_few_pages(model_dirs, name, dtype):
     pages freed by finished requests are used again at once."""
     vocab = TINY[name]["vocab_size"]
     lens = {"A": [60, 33, 47, 21, 58, 40, 9, 52], "B": [120, 1, 77, 90, 45, 130, 18, 66],
-            "C": [90, 48, 97, 16, 70, 33, 80, 25], "D": [700, 48, 97, 530, 70, 33, 80, 25]}[name]
+            "C": [90, 48, 97, 16, 70, 33, 80, 25], "D": [700, 48, 97, 530, 70, 33, 80, 25],
+            "E": [300, 48, 97, 610, 70, 33, 80, 25]}[name]
     requests = {f"r{i}": random_tokens(n, vocab, 300 + i) for i, n in enumerate(lens)}
     page = PAGE[name]
     rng = random.Random(5)

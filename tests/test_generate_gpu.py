@@ -467,7 +467,7 @@ def random_trace(rng, requests, max_live=4):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,seed", [("A", 0), ("B", 1), ("C", 2), ("D", 3), ("D", 4)])
+@pytest.mark.parametrize("name,seed", [("A", 0), ("B", 1), ("C", 2), ("D", 3), ("D", 4), ("E", 5)])
 def test_random_traces_replay_like_the_plain_model(model_dirs, tmp_path, name, seed, dtype):
     import io
     import random
@@ -475,7 +475,7 @@ def test_random_traces_replay_like_the_plain_model(model_dirs, tmp_path, name, s
     rng = random.Random(seed)
     cfg = TINY[name]
     vocab = cfg["vocab_size"]
-    longest = 400 if name == "D" else min(cfg["max_position_embeddings"], 120)
+    longest = 400 if name in ("D", "E") else min(cfg["max_position_embeddings"], 120)
     requests = {f"q{i}": random_tokens(rng.randint(1, longest), vocab, 900 * seed + i) for i in range(rng.randint(3, 7))}
     steps, peak = random_trace(rng, requests)
     runner = make_runner(model_dirs[name], dtype, peak)

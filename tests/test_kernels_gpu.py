@@ -466,7 +466,8 @@ def test_gemm_with_swiglu_epilogue(m, inter, k):
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 23, 40, 64])
-@pytest.mark.parametrize("nh,nkv,hd,k", [(8, 2, 64, 256), (3, 1, 16, 64), (32, 8, 64, 2048), (5, 5, 48, 96)])
+@pytest.mark.parametrize("nh,nkv,hd,k", [(8, 2, 64, 256), (3, 1, 16, 64), (32, 8, 64, 2048), (5, 5, 48, 96),
+                                         (24, 8, 128, 256), (32, 8, 128, 512), (3, 1, 128, 384)])
 def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
     """The q, k, v projection that rotates and stores in its epilogue against product, rotation and store done
     apart."""

@@ -42,8 +42,16 @@ TINY_D = {
                      "original_max_position_embeddings": 8192, "rope_type": "llama3"},
     "max_position_embeddings": 2048, "tie_word_embeddings": True,
 }
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
-NORM_JITTER = {"A": 0.0, "B": 0.1, "C": 0.1, "D": 0.1}
+# heads of 128 in groups of three over one KV head (the larger Llamas' head size, where the bfloat16 attention has
+# one wave per task only), an untied head, another eps and theta
+TINY_E = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 384, "intermediate_size": 528, "vocab_size": 777, "num_hidden_layers": 2,
+    "num_attention_heads": 3, "num_key_value_heads": 1, "rms_norm_eps": 3e-6, "rope_theta": 250000.0,
+    "max_position_embeddings": 1024, "tie_word_embeddings": False,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+NORM_JITTER = {"A": 0.0, "B": 0.1, "C": 0.1, "D": 0.1, "E": 0.1}
 
 
 def make_model_dir(path: str, cfg: dict, seed: int, dtype: str, norm_jitter: float = 0.0) -> str:
