@@ -385,7 +385,7 @@ extern "C" int atoma_rope_cache_write(void* qkv, int act_dtype, int row_stride, 
       ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0) {
     const int groups = (n_tokens + kRopeTokens - 1) / kRopeTokens;
     const int passes = (kRopeTokens * (nh + nkv) * (hd >> 4) + 255) / 256;      // of 256 threads over a block's items
-    int split = (512 + groups - 1) / groups;                                   // aim at 512 blocks
+    int split = (2048 + groups - 1) / groups;                                  // aim at 2048 blocks: eight a CU
     split = split > passes ? passes : split;
     hipLaunchKernelGGL(rope_cache_write_vec_kernel, dim3(groups, split), dim3(256), 0,
                        stream, (uint16_t*)qkv, row_stride, positions, cos_t, sin_t, (uint16_t*)kcache,
