@@ -8,23 +8,32 @@ using namespace atoma;
 
 // ---------------------------------------------------------------------------------------------
 // Embedding gather into the float32 residual stream: out[t, :] = table[token[t], :].
+// Tokens that the host has not seen (fed from the sampler on the device) are checked here: an id outside the table
+// reads nothing and leaves a row of NaN, which shows in that request's logits and in nobody else's.
 // Reference: models/src/llama.rs:470 (candle Embedding).
 template <typename TW>
 __global__ void embed_kernel(const int32_t* __restrict__ tokens, const TW* __restrict__ table,
-                             float* __restrict__ out, int width) {
+                             float* __restrict__ out, int width, int vocab) {
   const int t = blockIdx.x;
-  const size_t src = (size_t)tokens[t] * width, dst = (size_t)t * width;
+  const int token = tokens[t];
+  const size_t dst = (size_t)t * width;
+  if (token < 0 || token >= vocab) {
+    for (int i = threadIdx.x; i < width; i += blockDim.x) out[dst + i] = __int_as_float(0x7fc00000);
+    return;
+  }
+  const size_t src = (size_t)token * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) out[dst + i] = to_f32(table[src + i]);
 }
 
 extern "C" int atoma_embed(const int32_t* tokens, const void* table, int table_dtype, float* out, int n_tokens,
-                           int width, hipStream_t stream) {
+                           int width, int vocab, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   dim3 grid(n_tokens), block(256);
   if (table_dtype == kF32)
-    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, tokens, (const float*)table, out, width);
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, tokens, (const float*)table, out, width, vocab);
   else if (table_dtype == kBF16)
-    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, tokens, (const bf16_t*)table, out, width);
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, tokens, (const bf16_t*)table, out, width,
+                       vocab);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();

@@ -149,14 +149,13 @@ sample_kernel(const float* __restrict__ logits, int ld, int vocab, const float* 
   ArgMax a = {-INFINITY, 0x7fffffff};
   sweep(lr, vocab, [&](float v, int i) { a = better(a, ArgMax{v, i}); });
   a = block_argmax(a, am);
+  if ((unsigned)a.i >= (unsigned)vocab) a.i = 0;       // a row of NaN has no largest value: still name a token
   const float temp = temperature[row];
-  if (!(temp > 0.f)) {
-    if (tid == 0) {
-      out_token[row] = a.i;
-      out_logit[row] = a.v;
-    }
-    return;
+  if (tid == 0) {          // the answer of a greedy row, and of a row whose weights are no numbers
+    out_token[row] = a.i;
+    out_logit[row] = lr[a.i];
   }
+  if (!(temp > 0.f)) return;
 
   const int k = top_k[row];
   const float p = top_p[row];
@@ -408,6 +407,7 @@ sample_kernel(const float* __restrict__ logits, int ld, int vocab, const float* 
     if (i < wave) before += wave_u64[i];
     kept += wave_u64[i];
   }
+  if (kept == 0) return;                           // weights that are no numbers: the default answer stands
   u64 target = (u64)((double)uniform[row] * (double)kept);
   if (target >= kept) target = kept - 1;           // (kept >= 2^40: the largest weight is always kept)
   if (tid < kAllSlices && before <= target && target < before + mine) {

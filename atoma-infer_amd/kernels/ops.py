@@ -77,7 +77,7 @@ def core():
 # ------------------------------------------------------------------------------------------------------------
 
 def embed(tokens: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = table[tokens[t]] as float32.  The caller guarantees 0 <= token < table rows."""
+    """out[t] = table[tokens[t]] as float32; a token outside the table gives a row of NaN."""
     _dev(tokens, table)
     _i32(tokens, "tokens")
     _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, width]")
@@ -85,8 +85,8 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor]
     if out is None:
         out = torch.empty((n, width), dtype=torch.float32, device=table.device)
     _need(out.dtype is torch.float32 and out.is_contiguous() and tuple(out.shape) == (n, width), "embed: bad out")
-    _check(core().atoma_embed(_p(tokens), _p(table), _code(table, "embedding table"), _p(out), n, width, _stream()),
-           "embed")
+    _check(core().atoma_embed(_p(tokens), _p(table), _code(table, "embedding table"), _p(out), n, width,
+                              table.shape[0], _stream()), "embed")
     return out
 
 

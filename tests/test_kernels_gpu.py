@@ -563,3 +563,26 @@ def test_attention_whole_ranges_with_eight_waves(window):
         want = plain_attention(qq, ks[e], vs[e], s, scale, window, nh // nkv).reshape(nh * hd)
         err = (out[e].double().cpu() - want).abs().max() / want.abs().max()
         assert err < 2e-2, f"request {e} of length {s + 1}: {err:.3e}"
+
+
+def test_tokens_outside_the_table_and_rows_of_nan_do_no_harm():
+    """A sampled token reaches the next step without passing the host: the embedding checks it, and the sampler
+    names a token of the vocabulary whatever its logits hold."""
+    from atoma_infer_amd.kernels import ops
+    table = rnd(50, 24, dtype=torch.bfloat16, seed=1)
+    toks = torch.tensor([3, 50, -1, 2 ** 31 - 1, 49], dtype=torch.int32, device=DEV)
+    out = ops.embed(toks, table)
+    assert torch.equal(out[0], table[3].float()) and torch.equal(out[4], table[49].float())
+    assert bool(torch.isnan(out[1:4]).all())
+    logits = torch.randn(4, 1000, generator=torch.Generator().manual_seed(0)).to(DEV)
+    logits[1] = float("nan")
+    logits[2, 100:200] = float("nan")
+    logits[3] = float("-inf")
+    dev = lambda x, dt: torch.tensor(x, dtype=dt, device=DEV)
+    for temp, k, p in ((0.0, 0, 1.0), (0.8, 0, 1.0), (0.8, 20, 0.9)):
+        tok, _ = ops.sample(logits, dev([temp] * 4, torch.float32), dev([k] * 4, torch.int32),
+                            dev([p] * 4, torch.float32), dev([0.3] * 4, torch.float32))
+        tok = tok.cpu().tolist()
+        assert all(0 <= t < 1000 for t in tok), tok
+        if temp == 0.0:
+            assert tok[0] == int(torch.argmax(logits[0])) and tok[3] == 0
