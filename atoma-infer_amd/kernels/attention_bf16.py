@@ -52,10 +52,8 @@ def max_waves_for(hd: int) -> int:
 
 
 # (request, KV head) pairs from which on a decoded token's keys are not cut into chunks: measured on MI355X (256 CUs),
-# half as many pairs as CUs win already at contexts up to 4,096, three quarters at any context
+# half as many pairs as CUs win at contexts from 2,000 to 32,000 tokens; with 64 pairs chunks win at all of them
 WHOLE_MIN_PAIRS = 128
-WHOLE_MAX_KEYS = 4096
-WHOLE_MIN_PAIRS_LONG = 192
 
 
 def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = False) -> Tuple[int, int]:
@@ -71,8 +69,7 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = F
     decides is that of 256-key tasks over all KV heads; ``max_keys`` is rounded up to 256.
     """
     pairs = n_split * kv_heads
-    if whole_ok and (pairs >= max(WHOLE_MIN_PAIRS_LONG, WHOLE_MIN_PAIRS) or
-                     (pairs >= WHOLE_MIN_PAIRS and max_keys <= WHOLE_MAX_KEYS)):
+    if whole_ok and pairs >= WHOLE_MIN_PAIRS:     # at 2,000 as at 32,000 keys (measured from 128 pairs on)
         return 0, 8
     tasks = n_split * -(-max_keys // CHUNK) * kv_heads
     if tasks <= 160:

@@ -257,7 +257,6 @@ def test_decoding_with_whole_key_ranges(model_dirs, monkeypatch):
     threshold is lowered so that three requests do it: decoded through graphs, against the plain model."""
     from atoma_infer_amd.kernels import attention_bf16
     monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 2)
-    monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS_LONG", 2)
     name, dtype = "D", "bfloat16"
     vocab = TINY[name]["vocab_size"]
     requests = {"a": random_tokens(700, vocab, 31), "b": random_tokens(90, vocab, 32), "c": random_tokens(300, vocab, 33)}
