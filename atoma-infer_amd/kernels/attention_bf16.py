@@ -54,6 +54,9 @@ def max_waves_for(hd: int) -> int:
 # (request, KV head) pairs from which on a decoded token's keys are not cut into chunks: measured on MI355X (256 CUs),
 # half as many pairs as CUs win at contexts from 2,000 to 32,000 tokens; with 64 pairs chunks win at all of them
 WHOLE_MIN_PAIRS = 128
+# keys from which on the chunks of a decoded token are 512 keys long, walked by two waves (2 to 6 % quicker steps at
+# 16k to 32k tokens with 1 to 12 requests; no gain at 8k)
+LONG_KEYS = 16384
 
 
 def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = False) -> Tuple[int, int]:
@@ -65,8 +68,9 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = F
     A wave walks its keys one 32-key block after another, so few keys per wave shorten the chain when few requests
     decode, and long chunks save partial results (and time in the merging kernel) when many do.  Measured on
     MI355X with 2,000-token contexts and 8 KV heads: one or two requests want 128-key chunks, three to about
-    eleven 256-key chunks walked by two waves each, more requests 256-key chunks with a wave each.  The count that
-    decides is that of 256-key tasks over all KV heads; ``max_keys`` is rounded up to 256.
+    eleven 256-key chunks walked by two waves each, more requests 256-key chunks with a wave each, or 512-key
+    chunks walked by two waves from 16k keys on.  The count that decides is that of 256-key tasks over all KV
+    heads; ``max_keys`` is rounded up to 256.
     """
     pairs = n_split * kv_heads
     if whole_ok and pairs >= WHOLE_MIN_PAIRS:     # at 2,000 as at 32,000 keys (measured from 128 pairs on)
@@ -76,6 +80,8 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = F
         return 128, 1
     if tasks <= 800:
         return CHUNK, 2
+    if max_keys >= LONG_KEYS:
+        return 2 * CHUNK, 2     # long contexts: half as many partial results to write and to merge
     return CHUNK, 1
 
 
@@ -185,7 +191,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
             live = _live_pieces(rows, qt, min(qt, count - tok0))
             if do_split:
                 c_first, c_last = lo // chunk, (k_end - 1) // chunk
-                slots = bucket * (CHUNK // chunk) if bucket is not None else c_last + 1
+                slots = -(-(bucket * CHUNK) // chunk) if bucket is not None else c_last + 1
                 for row0 in live:
                     combine.append((e, tok0, qt, row0, 0, 0, n_part + c_first, c_last - c_first + 1) + tail)
                     for c in range(slots):
@@ -240,7 +246,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
         whole[..., 9] = 1
         whole[..., 10] = starts[:, None]
         return whole.reshape(-1, 12), (s * row_chunks, 0, 0, waves)
-    slots = bucket * (CHUNK // chunk)
+    slots = -(-(bucket * CHUNK) // chunk)
     c = np.arange(slots, dtype=np.int64)
     c_first, c_last = lo // chunk, (k_end - 1) // chunk
     valid = (c[None, :] >= c_first[:, None]) & (c[None, :] <= c_last[:, None])          # [s, slots]

@@ -82,6 +82,31 @@ def test_decode_builder_equals_the_general_one(seed):
     assert A.build_tasks(other, counts, group, window, bucket)[1] == mf
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_long_contexts(seed):
+    """Contexts of tens of thousands of keys: longer chunks, the same coverage, both builders alike."""
+    rng = np.random.default_rng(500 + seed)
+    s = int(rng.integers(1, 12))
+    group, window = int(rng.choice([1, 4, 8])), int(rng.choice([0, 0, 9000]))
+    starts = rng.integers(15000, 40000, size=s).astype(np.int32)
+    counts = np.ones(s, dtype=np.int32)
+    bucket = -(-int(starts.max() + 1) // 256)
+    fast, mf = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
+    slow, ms = A.build_tasks(starts, counts, group, window, bucket, vectorized=False, kv_heads=8, max_waves=8)
+    assert mf == ms
+    live = fast[:, 0] >= 0
+    assert np.array_equal(live, slow[:, 0] >= 0) and np.array_equal(fast[live], slow[live])
+    coverage(fast, mf, starts, counts, group, window)
+    if bucket * 256 >= A.LONG_KEYS and s * bucket * 8 > 800:
+        spans = fast[live][:, 5] - fast[live][:, 4]
+        assert int(spans.max()) == 512 and mf[3] == 2
+    # a portion of a prompt beside them
+    counts2 = counts.copy()
+    counts2[0] = 40
+    arr, meta = A.build_tasks(starts, counts2, group, window)
+    coverage(arr, meta, starts, counts2, group, window)
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_whole_ranges_for_many_decoding_requests(seed):
     """Enough (request, KV head) pairs to fill the GPU: a decoded token's keys are one task for eight waves, and

@@ -255,6 +255,9 @@ ATTN_CASES = [
     (8, 2, 64, 16, 0, [(0, 1100), (900, 150), (2047, 1)]),
     (4, 2, 32, 16, 800, [(0, 1300), (1200, 40)]),
     (4, 1, 128, 16, 0, [(4000, 70)]),
+    # decoded tokens with so many keys that their chunks are 512 keys long
+    (8, 8, 64, 16, 0, [(20000, 1), (16500, 1), (3, 2)]),
+    (4, 4, 128, 16, 9000, [(17000, 1), (30000, 1), (16385, 1)]),
 ]
 
 
