@@ -35,6 +35,7 @@ constexpr int DTILES = (HD + 31) / 32; // 32-row tiles of O^T
 constexpr int PAGE = 16;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kSlack = 8.0f;   // see the softmax in the kernel
+constexpr int kCUs = 256;        // MI355X
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -77,7 +78,7 @@ __device__ __forceinline__ bf16x8 pack8(const float* v) {
 //   4 x 2  prompts and mixed steps;
 //   1 x 8  decode steps of many requests: a task is all keys of a request's token, so nothing is left to the
 //          second kernel (there are enough requests and KV heads to fill the GPU without cutting keys into tasks).
-template <int TASKS, int KSPLIT>
+template <int TASKS, int KSPLIT, bool LATE = false>
 __global__ void __launch_bounds__(64 * TASKS * KSPLIT)
 attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
                       const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
@@ -192,8 +193,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   };
 
   // One block is in flight: the next block's loads are issued right after S^T (the values move aside first) when
-  // registers allow, else at the end of the block.
-  constexpr bool EARLY = HD <= 128;
+  // registers allow, else at the end of the block.  LATE asks for the end of the block as well: 25 registers fewer,
+  // which lets two workgroups of eight waves share a CU.
+  constexpr bool EARLY = HD <= 128 && !LATE;
   constexpr int STRIDE = 32 * KSPLIT;
   const int k_first = k_begin + 32 * part;
   bf16x8 kf[KSTEPS];
@@ -465,14 +467,21 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
   const Task* t = reinterpret_cast<const Task*>(tasks);
   // ksplit: waves that share a task's keys: 1, 2 (four tasks a workgroup) or 8 (one task a workgroup), the latter
   // two for head sizes whose merge fits in LDS
-#define ATOMA_ATTN(T, KS)                                                                                          \
-  hipLaunchKernelGGL((attention_mfma_kernel<T, KS>), dim3(((n_tasks + T - 1) / T) * nkv), dim3(64 * T * KS), 0,   \
+#define ATOMA_ATTN(T, KS, ...)                                                                                     \
+  hipLaunchKernelGGL((attention_mfma_kernel<T, KS, ##__VA_ARGS__>), dim3(((n_tasks + T - 1) / T) * nkv),          \
+                     dim3(64 * T * KS), 0,                                                                        \
                      stream, (const uint16_t*)q, q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,      \
                      (uint16_t*)out, out_stride, part_o, part_lse, t, n_tasks, block_tables, max_blocks, scale,   \
                      window, nh, nkv)
   if (ksplit == 1) ATOMA_ATTN(4, 1);
-  else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1));
-  else if (ksplit == 8 && kSplit8Fits) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1));
+  // (two waves a task: always the late loads, two workgroups to a CU; long prompts gain 9 %, short ones nothing)
+  else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1), true);
+  else if (ksplit == 8 && kSplit8Fits) {
+    // more workgroups than CUs: two of them to a CU finish sooner than two rounds of one (measured; with fewer,
+    // the loads in flight during the softmax count for more)
+    if ((long long)n_tasks * nkv > kCUs) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), true);
+    else ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1));
+  }
   else return ATOMA_ERR_SHAPE;
 #undef ATOMA_ATTN
   ATOMA_LAUNCH_CHECK();

@@ -541,14 +541,15 @@ def test_products_replay_in_graphs(m, n, k, cdt):
             torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("more", [30, 8])      # 320 and 144 workgroups: more and fewer than the GPU has CUs
 @pytest.mark.parametrize("window", [0, 200])
-def test_attention_whole_ranges_with_eight_waves(window):
+def test_attention_whole_ranges_with_eight_waves(window, more):
     """A decode step of many requests: every (request, KV head) pair is one task whose keys eight waves share and
     merge in LDS.  Lengths from one key to a few thousand, so that waves with nothing to do sit beside full ones."""
     from atoma_infer_amd.kernels import attention_bf16 as A
     nh, nkv, hd, page = 32, 8, 64, 16
     g = torch.Generator().manual_seed(7)
-    starts = [0, 1, 30, 31, 32, 255, 256, 257, 511, 1000] + torch.randint(0, 2500, (30,), generator=g).tolist()
+    starts = [0, 1, 30, 31, 32, 255, 256, 257, 511, 1000] + torch.randint(0, 2500, (more,), generator=g).tolist()
     counts = [1] * len(starts)
     lens = [s + 1 for s in starts]
     ks, vs, kc, vc, bt = paged_setup(lens, nkv, hd, page, torch.bfloat16, seed=3)
