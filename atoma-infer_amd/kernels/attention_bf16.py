@@ -67,8 +67,9 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = F
 
     A wave walks its keys one 32-key block after another, so few keys per wave shorten the chain when few requests
     decode, and long chunks save partial results (and time in the merging kernel) when many do.  Measured on
-    MI355X with 2,000-token contexts and 8 KV heads: one or two requests want 128-key chunks, three to about
-    eleven 256-key chunks walked by two waves each, more requests 256-key chunks with a wave each, or 512-key
+    MI355X with 2,000-token contexts and 8 KV heads: one or two requests want 128-key chunks, three to seven the
+    same walked by two waves each (up to 4,096 keys: beyond, the merge of twice as many partial results costs more),
+    up to about eleven 256-key chunks walked by two waves each, more requests 256-key chunks with a wave each, or 512-key
     chunks walked by two waves from 16k keys on.  The count that decides is that of 256-key tasks over all KV
     heads; ``max_keys`` is rounded up to 256.
     """
@@ -78,6 +79,8 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = F
     tasks = n_split * -(-max_keys // CHUNK) * kv_heads
     if tasks <= 160:
         return 128, 1
+    if tasks <= 540 and max_keys <= 4096:
+        return 128, 2           # three to seven requests at 2,000 tokens: 2 to 4 % quicker steps than 256-key chunks
     if tasks <= 800:
         return CHUNK, 2
     if max_keys >= LONG_KEYS:
