@@ -394,7 +394,7 @@ def test_text_in_and_out_with_a_tokenizer(model_dirs, tmp_path):
     request at the piece that equals one of them, ``truncate`` keeps the end of the prompt's text and
     ``return_full_text`` puts the prompt before the output."""
     import shutil
-    from tokenizers import Tokenizer, models, pre_tokenizers, decoders
+    from tokenizers import Tokenizer, models, pre_tokenizers
     from atoma_infer_amd.config import CacheConfig, SchedulerConfig
     from atoma_infer_amd.engine.engine import LlmEngine
     from atoma_infer_amd.sampling import GenerateParameters

@@ -4,7 +4,7 @@ encoding), whose run order names a layer twice and lets a layer read another lay
 written with random weights, built and stepped without a change to the framework's files."""
 import dataclasses
 import math
-from typing import Dict, List, Optional
+from typing import Dict, List
 
 import pytest
 import torch

@@ -3,7 +3,6 @@
 import itertools
 import random
 
-import pytest
 
 from atoma_infer_amd.cache import CacheManager, GroupGeometry
 from atoma_infer_amd.config import SchedulerConfig
