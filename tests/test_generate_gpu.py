@@ -34,7 +34,7 @@ def engine(model_dir, dtype, page, pages, **sched):
 
 
 def test_greedy_generation_tiny_a_workload(model_dirs):
-    """BASELINE's Tiny A workload: 2 prompts of 8 and 5 ids, 8 greedy steps each, float32, block size 4."""
+    """The tiny workload A: 2 prompts of 8 and 5 ids, 8 greedy steps each, float32, block size 4."""
     from atoma_infer_amd.sampling import GenerateParameters
     d = model_dirs["A"]
     w, cfg = plain_weights(d), plain_config(d)
@@ -54,7 +54,7 @@ def test_greedy_generation_tiny_a_workload(model_dirs):
 
 
 def test_tiny_b_workload_portions_beside_decodes_with_temperature(model_dirs):
-    """BASELINE's Tiny B workload: prompts of 37, 1 and 20 ids in 16-token portions alongside decodes, temperature
+    """The tiny workload B: prompts of 37, 1 and 20 ids in 16-token portions alongside decodes, temperature
     0.7 with a fixed seed.  The sampled tokens must be what the plain model and plain sampler give for the same
     uniform numbers, and must not depend on how requests were batched."""
     from atoma_infer_amd.sampling import GenerateParameters, uniform
