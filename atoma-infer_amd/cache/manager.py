@@ -89,6 +89,11 @@ class CacheManager:
         if h:
             self._lib.cm_destroy(h)
 
+    @property
+    def handle(self):
+        """The native manager, for other parts of the host library (the scheduler takes its pages from it)."""
+        return self._h
+
     # -- requests ------------------------------------------------------------------------------------
     def add(self, request: int) -> int:
         rc = self._lib.cm_add_request(self._h, request)

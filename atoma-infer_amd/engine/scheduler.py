@@ -17,19 +17,26 @@ returns to the *front* of the waiting queue and later prefills its prompt and th
 (scheduler.rs:650-690, 1778-1896).  If the request that cannot grow is the only one running, it is finished as
 "length_capped": nothing could be given back for it.
 
+The decisions are made in the host library (csrc/host/scheduler.cpp), next to the cache manager it draws pages
+from; this module keeps the ``Request`` objects, reports their counters before each plan and applies the plan's
+outcome to them.
+
 Differences from the reference, on purpose: portions of a prompt stay in the running queue until the prompt is
 done (the reference drops them, scheduler.rs:1313-1338), pages are given back when a request finishes (the
 reference frees only on abort and preemption), and there is no swap space.
 """
 from __future__ import annotations
 
+import ctypes
 import dataclasses
 import time
-from collections import deque
-from typing import Deque, List, Optional
+from typing import Dict, List, Optional
+
+import numpy as np
 
 from ..cache.manager import CacheManager
 from ..config.engine import SchedulerConfig
+from ..kernels.library import load_host_library
 from .request import Request, Status
 
 
@@ -57,40 +64,90 @@ class ScheduleOutput:
         return not self.entries
 
 
+class SchedulerError(RuntimeError):
+    pass
+
+
+_PREEMPTED, _IGNORED, _CAPPED, _ADMITTED, _WAITING, _RUNNING = range(6)
+_lib = None
+
+
+def _native():
+    global _lib
+    if _lib is None:
+        lib = load_host_library()
+        p, i, i64, f64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_double
+        lib.sc_create.restype = p
+        lib.sc_create.argtypes = [p, i, i, i, i, i, f64]
+        lib.sc_destroy.restype = None
+        lib.sc_destroy.argtypes = [p]
+        lib.sc_add.argtypes = [p, i64, f64, ctypes.c_int32]
+        lib.sc_remove.argtypes = [p, i64]
+        lib.sc_sync.argtypes = [p, i, p]
+        lib.sc_schedule.argtypes = [p, f64]
+        lib.sc_entries.argtypes = [p, p, i]
+        lib.sc_list.argtypes = [p, i, p, i]
+        for name in ("sc_num_waiting", "sc_num_running", "sc_num_preemptions", "sc_last_prompt_latency"):
+            getattr(lib, name).argtypes = [p]
+        lib.sc_num_preemptions.restype = i64
+        lib.sc_last_prompt_latency.restype = f64
+        _lib = lib
+    return _lib
+
+
 class Scheduler:
+    """``cache`` is a ``CacheManager`` or anything that forwards to one (``handle`` is what the native scheduler
+    draws pages from).  If it has ``adopted(request)`` and ``forgot(request)``, they are called for every request
+    that a plan registered with the manager or released from it, so that books kept beside the manager follow."""
+
     def __init__(self, config: SchedulerConfig, cache: CacheManager, clock=time.monotonic):
         config.validate()
         self.config, self.cache, self.clock = config, cache, clock
-        self.waiting: Deque[Request] = deque()
-        self.running: List[Request] = []
-        self.num_preemptions = 0
-        self.last_prompt_latency = 0.0
-        self._prev_prompt = False
-        self._prev_time = 0.0
+        self._lib = _native()
+        self._h = self._lib.sc_create(cache.handle, config.max_num_batched_tokens, config.max_num_sequences,
+                                      config.max_model_len, int(config.enable_chunked_prefill),
+                                      config.max_prefill_chunk, float(config.delay_factor))
+        if not self._h:
+            raise SchedulerError(f"the native scheduler refused {config}")
+        self._requests: Dict[int, Request] = {}
+        self._running: Dict[int, Request] = {}
+        self._adopted = getattr(cache, "adopted", None)
+        self._forgot = getattr(cache, "forgot", None)
+        self._ids = np.zeros(max(64, 4 * config.max_num_sequences), dtype=np.int64)
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.sc_destroy(h)
 
     # -- queue operations --------------------------------------------------------------------------------
     def add(self, request: Request) -> None:
+        if self._lib.sc_add(self._h, request.uid, float(request.metrics.arrival_time), request.length) != 0:
+            raise SchedulerError(f"request number {request.uid} is already queued")
         request.status = Status.WAITING
-        self.waiting.append(request)
+        self._requests[request.uid] = request
 
     def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self._requests)
 
     def num_unfinished(self) -> int:
-        return len(self.waiting) + len(self.running)
+        return len(self._requests)
+
+    def _take_out(self, r: Request, status: Status) -> None:
+        held = self._lib.sc_remove(self._h, r.uid)
+        if held < 0:
+            raise SchedulerError(f"request {r.request_id} is not queued")
+        del self._requests[r.uid]
+        self._running.pop(r.uid, None)
+        if held and self._forgot is not None:
+            self._forgot(r.uid)
+        r.status = status
 
     def abort(self, request_id: str) -> Optional[Request]:
         """Remove a request wherever it is; its pages go back (scheduler.rs:390-443)."""
-        for r in list(self.waiting):
+        for r in self._requests.values():
             if r.request_id == request_id:
-                self.waiting.remove(r)
-                r.status = Status.FINISHED_ABORTED
-                return r
-        for r in self.running:
-            if r.request_id == request_id:
-                self.running.remove(r)
-                self._release(r)
-                r.status = Status.FINISHED_ABORTED
+                self._take_out(r, Status.FINISHED_ABORTED)
                 return r
         return None
 
@@ -98,121 +155,76 @@ class Scheduler:
         """A request has produced its last token: give back what it holds.  It is usually running; it waits if it
         was preempted while that token was still on its way."""
         assert status.finished
-        if request.status is Status.RUNNING:
-            self.running.remove(request)
-        else:
-            self.waiting.remove(request)
-        self._release(request)
-        request.status = status
+        self._take_out(request, status)
 
-    def _release(self, r: Request) -> None:
-        if self.cache.has(r.uid):
-            self.cache.free(r.uid)
+    # -- inspection --------------------------------------------------------------------------------------
+    def _list(self, kind: int) -> List[Request]:
+        n = self._lib.sc_list(self._h, kind, self._ids.ctypes.data, self._ids.size)
+        if n > self._ids.size:
+            self._ids = np.zeros(2 * n, dtype=np.int64)
+            n = self._lib.sc_list(self._h, kind, self._ids.ctypes.data, self._ids.size)
+        return [self._requests[u] for u in self._ids[:n].tolist()]
+
+    @property
+    def waiting(self) -> List[Request]:
+        """The waiting queue from its head."""
+        return self._list(_WAITING)
+
+    @property
+    def running(self) -> List[Request]:
+        return self._list(_RUNNING)
+
+    @property
+    def num_preemptions(self) -> int:
+        return self._lib.sc_num_preemptions(self._h)
+
+    @property
+    def last_prompt_latency(self) -> float:
+        return self._lib.sc_last_prompt_latency(self._h)
 
     # -- one step's plan -----------------------------------------------------------------------------------
-    def _chunk(self, r: Request, budget: int) -> int:
-        n = min(r.num_uncomputed, budget)
-        if self.config.max_prefill_chunk > 0 and r.num_uncomputed > 1:
-            n = min(n, self.config.max_prefill_chunk)
-        if not self.config.enable_chunked_prefill and n < r.num_uncomputed:
-            return 0  # prompts are not cut: wait for a step with room for all of it
-        return n
-
-    def _preempt(self, victim: Request, out: ScheduleOutput) -> None:
-        self.running.remove(victim)
-        self._release(victim)
-        victim.num_computed = 0
-        victim.status = Status.WAITING
-        victim.metrics.num_preemptions += 1
-        self.waiting.appendleft(victim)
-        self.num_preemptions += 1
-        out.preempted.append(victim)
-        # a victim already planned into this step gives its place back
-        out.entries[:] = [e for e in out.entries if e.request is not victim]
-
-    def _passed_delay(self, now: float) -> bool:
-        """The reference's optional batching delay (scheduler.rs:2077-2097)."""
-        if self._prev_prompt:
-            self.last_prompt_latency = now - self._prev_time
-        self._prev_time, self._prev_prompt = now, False
-        if self.config.delay_factor > 0 and self.waiting:
-            earliest = min(r.metrics.arrival_time for r in self.waiting)
-            return (now - earliest) > self.config.delay_factor * self.last_prompt_latency or not self.running
-        return True
-
     def schedule(self) -> ScheduleOutput:
-        out = ScheduleOutput([], [], [], [])
-        cfg = self.config
         now = self.clock()
-        self.running.sort(key=lambda r: r.metrics.arrival_time)  # first come first served (policy.rs:56-61)
-
-        def used_tokens():
-            return sum(e.num_tokens for e in out.entries)
-
-        # 1 and 2: running requests, decodes before portions of prompts
-        live = [r for r in self.running if not r.frozen]
-        order = [r for r in live if not r.in_prefill] + [r for r in live if r.in_prefill]
-        if len(order) <= cfg.max_num_sequences and len(order) <= cfg.max_num_batched_tokens and \
-                all(r.num_uncomputed == 1 for r in order):
-            # the common step: everything running decodes one token and fits both budgets; pages are taken
-            # request by request, and the general path below takes over at the first that finds none
-            done = 0
-            for r in order:
-                if not self.cache.can_reserve(r.uid, r.num_computed + 1):
-                    break
-                self.cache.reserve(r.uid, r.num_computed + 1)
-                out.entries.append(ScheduledEntry(r, 1, r.num_computed, True))
-                done += 1
-            order = order[done:]
-        for r in order:
-            if r.status is not Status.RUNNING:
-                continue  # preempted while serving an earlier request
-            if len(out.entries) >= cfg.max_num_sequences:
-                break
-            n = self._chunk(r, cfg.max_num_batched_tokens - used_tokens())
-            if n <= 0:
-                continue
-            while not self.cache.can_reserve(r.uid, r.num_computed + n):
-                # the latest arrival that is not just waiting for its last token (that one frees its pages soon)
-                victim = next((v for v in reversed(self.running) if not v.frozen), r)
-                if victim is r and len(self.running) == 1:
-                    # nothing else to give back: the pool cannot hold this request any longer
-                    self.running.remove(r)
-                    self._release(r)
-                    r.status = Status.FINISHED_LENGTH_CAPPED
-                    out.capped.append(r)
-                    break
-                self._preempt(victim, out)
-                if victim is r:
-                    break
-            if r.status is not Status.RUNNING:
-                continue
-            self.cache.reserve(r.uid, r.num_computed + n)
-            out.entries.append(ScheduledEntry(r, n, r.num_computed, r.num_computed + n == r.length))
-
-        # 3: admissions, unless something was preempted in this step (its pages are meant for the running ones)
-        if not out.preempted and self._passed_delay(now):
-            while self.waiting:
-                r = self.waiting[0]
-                if r.length > cfg.max_model_len or not self.cache.fits_at_all(r.length):
-                    self.waiting.popleft()
-                    r.status = Status.FINISHED_IGNORED
-                    out.ignored.append(r)
-                    continue
-                if len(out.entries) >= cfg.max_num_sequences or len(self.running) >= cfg.max_num_sequences:
-                    break
-                n = self._chunk(r, cfg.max_num_batched_tokens - used_tokens())
-                if n <= 0:
-                    break
-                if self.cache.num_free_slots() == 0 or not self.cache.can_reserve(-1, n):
-                    break  # later: the head of the queue blocks those behind it
-                self.waiting.popleft()
-                self.cache.add(r.uid)
-                self.cache.reserve(r.uid, n)
-                r.status = Status.RUNNING
-                if r.metrics.first_scheduled_time is None:
-                    r.metrics.first_scheduled_time = now
-                self.running.append(r)
-                out.entries.append(ScheduledEntry(r, n, 0, n == r.length))
-                self._prev_prompt = True
+        lib, h = self._lib, self._h
+        if self._running:
+            rows = np.array([x for r in self._running.values()
+                             for x in (r.uid, r.length, r.num_computed, r.num_sampled, r.frozen)], dtype=np.int64)
+            if lib.sc_sync(h, len(self._running), rows.ctypes.data) != 0:
+                raise SchedulerError("a running request is unknown to the native scheduler")
+        n = lib.sc_schedule(h, float(now))
+        if n < 0:
+            raise SchedulerError("the cache manager refused pages it had just promised")
+        out = ScheduleOutput([], [], [], [])
+        # releases first: a request's number leaves the books beside the manager before anything else happens
+        for r in self._list(_PREEMPTED):
+            del self._running[r.uid]
+            r.num_computed = 0
+            r.status = Status.WAITING
+            r.metrics.num_preemptions += 1
+            out.preempted.append(r)
+            if self._forgot is not None:
+                self._forgot(r.uid)
+        for r in self._list(_CAPPED):
+            del self._running[r.uid]
+            del self._requests[r.uid]
+            r.status = Status.FINISHED_LENGTH_CAPPED
+            out.capped.append(r)
+            if self._forgot is not None:
+                self._forgot(r.uid)
+        for r in self._list(_IGNORED):
+            del self._requests[r.uid]
+            r.status = Status.FINISHED_IGNORED
+            out.ignored.append(r)
+        for r in self._list(_ADMITTED):
+            self._running[r.uid] = r
+            r.status = Status.RUNNING
+            if r.metrics.first_scheduled_time is None:
+                r.metrics.first_scheduled_time = now
+            if self._adopted is not None:
+                self._adopted(r.uid)
+        if n:
+            rows = np.empty((n, 4), dtype=np.int64)
+            lib.sc_entries(h, rows.ctypes.data, n)
+            reqs = self._requests
+            out.entries = [ScheduledEntry(reqs[u], k, s, bool(d)) for u, k, s, d in rows.tolist()]
         return out

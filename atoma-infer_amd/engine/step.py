@@ -123,21 +123,18 @@ class _Graph:
 class RunnerCache:
     """The cache manager as the scheduler sees it, with the runner's own books kept in step.
 
-    Same methods as ``CacheManager`` (has, add, free, can_reserve, reserve, fits_at_all, num_free_slots,
-    num_free_pages), so the scheduler runs against either.
+    Everything is forwarded to the ``CacheManager``; ``adopted`` and ``forgot`` are what the scheduler calls after
+    it has registered a request with the manager, or released one from it, by itself.
     """
 
     def __init__(self, runner: "ModelRunner"):
         self._runner, self._mgr = runner, runner.manager
 
-    def has(self, request: int) -> bool:
-        return self._runner.has_request(request)
+    def adopted(self, request: int) -> None:
+        self._runner.adopt_request(request)
 
-    def add(self, request: int) -> int:
-        return self._runner.add_request(request)
-
-    def free(self, request: int) -> None:
-        self._runner.free_request(request)
+    def forgot(self, request: int) -> None:
+        self._runner.forget_request(request)
 
     def __getattr__(self, name):
         return getattr(self._mgr, name)
@@ -165,10 +162,15 @@ class ModelRunner:
     # -- requests ------------------------------------------------------------------------------------
     def add_request(self, request: int) -> int:
         slot = self.manager.add(request)
+        self.adopt_request(request)
+        return slot
+
+    def adopt_request(self, request: int) -> None:
+        """Open the books for a request that the manager already knows: nothing computed, state cleared."""
+        slot = self.manager.state_slot(request)
         self._computed[request] = 0
         for st in self.pool.states.values():
             st[slot].zero_()
-        return slot
 
     def has_request(self, request: int) -> bool:
         return request in self._computed
@@ -178,6 +180,10 @@ class ModelRunner:
 
     def free_request(self, request: int) -> None:
         self.manager.free(request)
+        self.forget_request(request)
+
+    def forget_request(self, request: int) -> None:
+        """Close the books of a request that the manager has already released."""
         del self._computed[request]
 
     def reset_request(self, request: int) -> None:

@@ -186,3 +186,135 @@ def test_max_prefill_chunk_caps_portions():
         sizes.append(out.entries[0].num_tokens)
         run_step(s, out)
     assert sizes == [16, 16, 5]
+
+
+def test_delay_factor_holds_admissions_back_while_something_runs():
+    """backends/vllm/src/scheduler.rs:2077-2097: after a step with a prompt, a waiting request is admitted only
+    once it has waited longer than delay_factor times that step's duration, or when nothing runs."""
+    now = [0.0]
+    cache = CacheManager([GroupGeometry(4, 64)], 8)
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=64, max_num_sequences=8, max_model_len=256,
+                                  delay_factor=2.0), cache, clock=lambda: now[0])
+    a = make_request(0, 10)
+    a.metrics.arrival_time = 0.0
+    s.add(a)
+    out = s.schedule()                       # nothing runs: admitted at once
+    assert [e.request.uid for e in out.entries] == [0]
+    run_step(s, out)
+    now[0] = 1.0                             # the prompt step took 1.0
+    b = make_request(1, 10)
+    b.metrics.arrival_time = 1.0
+    s.add(b)
+    out = s.schedule()
+    assert s.last_prompt_latency == 1.0
+    assert [e.request.uid for e in out.entries] == [0]          # b has waited 0 < 2 * 1.0
+    run_step(s, out)
+    now[0] = 2.5
+    out = s.schedule()
+    assert [e.request.uid for e in out.entries] == [0]          # 1.5 < 2.0
+    run_step(s, out)
+    now[0] = 3.5
+    out = s.schedule()
+    assert [e.request.uid for e in out.entries] == [0, 1]       # 2.5 > 2.0
+
+
+class _Limits:
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+
+
+def _random_world(seed):
+    """The same random traffic through the native scheduler and the plain one; every plan must be the same.
+
+    The engine's pipelining is played too: a sampled token is pending for one step, a request whose last token is
+    pending is frozen, and a request may end (or be aborted) while it waits after a preemption."""
+    from plain_scheduler import PlainPages, PlainRequest, PlainScheduler
+    rng = random.Random(seed)
+    page, pages, slots = rng.choice([1, 3, 4, 16]), rng.randint(3, 40), rng.randint(1, 6)
+    lim = _Limits(max_tokens=rng.randint(4, 48), max_requests=rng.randint(1, 6), max_model_len=rng.randint(30, 120),
+                  cut=rng.random() < 0.8, max_portion=rng.choice([0, 0, 5, 16]),
+                  delay_factor=rng.choice([0.0, 0.0, 0.5, 3.0]))
+    if not lim.cut:
+        lim.max_tokens = max(lim.max_tokens, lim.max_model_len)      # the configuration demands it
+    lim.max_tokens = max(lim.max_tokens, lim.max_requests)
+    now = [0.0]
+    cache = CacheManager([GroupGeometry(page, pages)], slots)
+    native = Scheduler(SchedulerConfig(max_num_batched_tokens=lim.max_tokens, max_num_sequences=lim.max_requests,
+                                       max_model_len=lim.max_model_len, enable_chunked_prefill=lim.cut,
+                                       max_prefill_chunk=lim.max_portion, delay_factor=lim.delay_factor),
+                       cache, clock=lambda: now[0])
+    plain_pages = PlainPages(page, pages, slots)
+    plain = PlainScheduler(lim, plain_pages)
+    mine, theirs, uid = {}, {}, 0
+    pending_mine, pending_theirs = [], []
+    plans = preemptions = 0
+    for step in range(rng.randint(40, 160)):
+        now[0] += rng.choice([0.1, 0.5, 2.0])
+        for _ in range(rng.choice([0, 0, 1, 1, 2, 4])):
+            n, max_new = rng.choice([1, 2, 7, 20, 45, 130]), rng.choice([1, 2, 5, 30])
+            a = make_request(uid, n, max_new=max_new)
+            a.metrics.arrival_time = now[0]
+            b = PlainRequest(uid, n, now[0], max_new)
+            native.add(a)
+            plain.add(b)
+            mine[uid], theirs[uid] = a, b
+            uid += 1
+        if mine and rng.random() < 0.05:
+            u = rng.choice(sorted(mine))
+            assert native.abort(f"r{u}") is mine.pop(u)
+            plain.take_out(theirs.pop(u), "aborted")
+        out_a, out_b = native.schedule(), plain.schedule(now[0])
+        plans += 1
+        preemptions += len(out_b.preempted)
+        assert [(e.request.uid, e.num_tokens, e.start, e.do_sample) for e in out_a.entries] == \
+            [(r.uid, n, st, sm) for r, n, st, sm in out_b.entries], (seed, step)
+        for name in ("preempted", "ignored", "capped"):
+            assert [r.uid for r in getattr(out_a, name)] == [r.uid for r in getattr(out_b, name)], (seed, step, name)
+        assert [r.uid for r in native.waiting] == [r.uid for r in plain.waiting], (seed, step)
+        assert sorted(r.uid for r in native.running) == sorted(r.uid for r in plain.running), (seed, step)
+        assert cache.num_free_pages() == plain_pages.free_pages() and \
+            cache.num_free_slots() == plain_pages.num_free_slots(), (seed, step)
+        assert out_a.num_tokens <= lim.max_tokens and len(out_a.entries) <= lim.max_requests
+        cache.check()
+        for r in out_a.ignored + out_a.capped:
+            mine.pop(r.uid), theirs.pop(r.uid)
+        for r in out_a.preempted:
+            assert r.num_computed == 0 and r.status is Status.WAITING
+        # the tokens of the step before reach the host: requests may end on them, also while they wait
+        for a in pending_mine:
+            a.pending -= 1
+            if a.uid in mine:
+                a.output_ids.append(7)
+                if len(a.output_ids) >= a.plan.max_new_tokens or a.length > lim.max_model_len:
+                    native.finish(mine.pop(a.uid), Status.FINISHED_LENGTH_CAPPED)
+        for b in pending_theirs:
+            b.pending -= 1
+            if b.uid in theirs:
+                b.outputs += 1
+                if b.outputs >= b.max_new or b.length > lim.max_model_len:
+                    plain.take_out(theirs.pop(b.uid), "capped")
+        # this step runs: tokens are computed, sampled tokens are pending until the next step
+        pending_mine, pending_theirs = [], []
+        for e in out_a.entries:
+            a = e.request
+            a.num_computed += e.num_tokens
+            if e.do_sample:
+                a.pending += 1
+                a.frozen = a.num_sampled >= a.plan.max_new_tokens or a.length > lim.max_model_len
+                pending_mine.append(a)
+        for b, n, _, sample in out_b.entries:
+            b.num_computed += n
+            if sample:
+                b.pending += 1
+                b.frozen = b.num_sampled >= b.max_new or b.length > lim.max_model_len
+                pending_theirs.append(b)
+    assert native.num_preemptions == plain.num_preemptions
+    return plans, preemptions
+
+
+def test_native_scheduler_decides_like_the_plain_one_under_random_traffic():
+    plans = preemptions = 0
+    for seed in range(60):
+        p, q = _random_world(seed)
+        plans, preemptions = plans + p, preemptions + q
+    assert plans > 3000 and preemptions > 50      # the traffic did drive pages out
