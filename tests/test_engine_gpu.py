@@ -267,3 +267,41 @@ def test_decoding_with_whole_key_ranges(model_dirs, monkeypatch):
     g = runner._graphs.get((3, 3))
     assert g is not None and g.graph is not None, "the decode steps were meant to replay as a graph"
     assert attention_bf16.chunk_for(3, 700, 2, whole_ok=True) == (0, 8)
+
+
+LLAMA_1B_LAYERS = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": 2048, "intermediate_size": 8192,
+    "vocab_size": 128256, "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192, "rope_type": "llama3"},
+    "max_position_embeddings": 131072, "tie_word_embeddings": True,
+}
+
+
+# the widths of Llama 3.1 8B (heads of 128, where the bfloat16 attention has one wave per task only) with one layer,
+# an untied head and a smaller vocabulary that is no multiple of anything
+LLAMA_8B_LAYER = dict(LLAMA_1B_LAYERS, hidden_size=4096, intermediate_size=14336, vocab_size=32003,
+                      num_hidden_layers=1, tie_word_embeddings=False)
+
+
+@pytest.mark.parametrize("cfg", [LLAMA_1B_LAYERS, LLAMA_8B_LAYER], ids=["1b", "8b"])
+def test_layers_of_serving_size_in_mixed_steps(tmp_path, cfg):
+    """Layers with the sizes of Llama 3.2 1B (and its whole vocabulary) and of Llama 3.1 8B: at these widths the
+    products take other plans (wider waves, K split over the grid, the library from 65 rows on) than any tiny
+    configuration reaches."""
+    model_dir = make_model_dir(str(tmp_path / "m"), cfg, seed=3, dtype="bfloat16", norm_jitter=0.1)
+    vocab = cfg["vocab_size"]
+    requests = {"a": random_tokens(300, vocab, 1), "b": random_tokens(90, vocab, 2), "c": random_tokens(33, vocab, 3)}
+    steps = [([("a", 200)], []), ([("a", 37), ("b", 50)], []), ([("a", 2), ("b", 1), ("c", 30)], [])]
+    steps += [([("a", 1), ("b", 1), ("c", 1)], [])] * 3
+    steps += [([("a", 58), ("b", 36)], ["a", "b", "c"])]
+    for dtype in DTYPES:
+        runner = make_runner(model_dir, dtype, 16, 40)
+        got = run_schedule(runner, requests, steps)
+        assert len(got) == 300 + 90 + 33
+        check_against_plain(model_dir, requests, got, dtype)
+        assert runner.manager.num_free_pages() == 40
+        del runner
+        torch.cuda.empty_cache()
+    _plain_cache.clear()
