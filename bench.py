@@ -61,7 +61,8 @@ def decode_run(model, batch, prompt_len, steps, warmup, context, seed=0, samplin
     g = torch.Generator().manual_seed(seed)
     vocab = model.vocab_size
     # requests that finish their prompt early decode while the others are still in theirs
-    prompt_steps = batch * (-(-prompt_len // max(2048, batch)))
+    # (the decoded tokens share the step's budget with the prompts, hence the factor of two)
+    prompt_steps = 2 * batch * (-(-prompt_len // max(2048, batch)))
     params = GenerateParameters(do_sample=False, max_new_tokens=steps + warmup + prompt_steps + 8,
                                 ignore_eos_token=True)
     if sampling:        # (temperature, top_k, top_p): draw instead of the default argmax
@@ -138,7 +139,7 @@ def main() -> int:
     if int(os.environ.get("WORLD_SIZE", "1")) > 1:
         print("bench.py: started with WORLD_SIZE > 1; this engine runs on one GPU", flush=True)
         return 2
-    if args.prompt_len + args.steps + args.warmup + args.batch * (-(-args.prompt_len // 2048)) + 8 > args.context:
+    if args.prompt_len + args.steps + args.warmup + 2 * args.batch * (-(-args.prompt_len // 2048)) + 8 > args.context:
         print("bench.py: prompt + steps exceed the context", file=sys.stderr)
         return 1
 
