@@ -318,3 +318,46 @@ def test_native_scheduler_decides_like_the_plain_one_under_random_traffic():
         p, q = _random_world(seed)
         plans, preemptions = plans + p, preemptions + q
     assert plans > 3000 and preemptions > 50      # the traffic did drive pages out
+
+
+def test_the_native_scheduler_refuses_what_does_not_fit_its_books():
+    import pytest
+    from atoma_infer_amd.engine.scheduler import SchedulerError
+    s, cache = make_scheduler()
+    a = make_request(0, 5)
+    s.add(a)
+    with pytest.raises(SchedulerError):
+        s.add(make_request(0, 9))                      # the number is taken
+    stranger = make_request(77, 5)
+    with pytest.raises(SchedulerError):
+        s.finish(stranger, Status.FINISHED_STOPPED)    # never queued
+    out = s.schedule()
+    assert [e.request.uid for e in out.entries] == [0] and s.num_unfinished() == 1
+    # the runner's books are told of every request the scheduler registers or releases by itself
+    calls = []
+
+    class Books:
+        def __init__(self, mgr):
+            self._mgr = mgr
+
+        def adopted(self, uid):
+            calls.append(("adopted", uid, self._mgr.state_slot(uid)))
+
+        def forgot(self, uid):
+            calls.append(("forgot", uid, self._mgr.has(uid)))
+
+        def __getattr__(self, name):
+            return getattr(self._mgr, name)
+
+    mgr = CacheManager([GroupGeometry(4, 4)], 4)
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=64, max_num_sequences=4, max_model_len=64), Books(mgr))
+    a, b = make_request(0, 7, max_new=6), make_request(1, 7, max_new=6)
+    s.add(a)
+    s.add(b)
+    run_step(s, s.schedule())
+    run_step(s, s.schedule())
+    out = s.schedule()                                 # b is preempted: the pool is full
+    assert [r.uid for r in out.preempted] == [1]
+    s.abort("r0")
+    assert calls == [("adopted", 0, 0), ("adopted", 1, 1), ("forgot", 1, False), ("forgot", 0, False)]
+    mgr.check()
