@@ -584,3 +584,156 @@ def test_toy_architecture_generates_through_the_engine(toy_dir):
                     scheduler=SchedulerConfig(max_num_batched_tokens=8, max_num_sequences=2, max_model_len=64))
     outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=5, ignore_eos_token=True))
     assert [o.inference_outputs[0].token_ids for o in outs] == want
+
+
+# ----------------------------------------------------------------------------------------------------------
+# a second toy architecture: another norm and another arrangement of a block
+
+
+def _parallel_parts():
+    """A norm that subtracts the mean and has a bias, and a block whose mixer and feed-forward both read the same
+    normed input and whose outputs are added to the residual stream together."""
+    from atoma_infer_amd.parts import Block, Norm, WeightSpec, register_block, register_norm
+
+    class ShiftScaleNorm(Norm):
+        def __init__(self, width: int, eps: float):
+            self.width, self.eps = width, eps
+
+        def weight_specs(self):
+            return {"weight": WeightSpec((self.width,), "norm"), "bias": WeightSpec((self.width,))}
+
+        def load(self, get, device, act_dtype):
+            self.weight, self.bias = get("weight").to(device).float(), get("bias").to(device).float()
+            self.act_dtype = act_dtype
+
+        def add_norm(self, resid, delta, rows=None):
+            if delta is not None:
+                delta = delta.float().sum(0) if delta.dim() == 3 else delta.float()
+            if rows is None:
+                if delta is not None:
+                    resid += delta
+                x = resid
+            else:
+                sel = rows.long()
+                x = resid[sel] if delta is None else resid[sel] + delta[sel]
+            mu = x.mean(-1, keepdim=True)
+            var = ((x - mu) ** 2).mean(-1, keepdim=True)
+            return ((x - mu) * torch.rsqrt(var + self.eps) * self.weight + self.bias).to(self.act_dtype)
+
+    class ParallelBlock(Block):
+        def __init__(self, norm, mixer, feed_forward):
+            self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
+
+        def _children(self):
+            return (("norm", self.norm), ("mixer", self.mixer), ("ffn", self.feed_forward))
+
+        def weight_specs(self):
+            return {f"{n}.{k}": ws for n, part in self._children() for k, ws in part.weight_specs().items()}
+
+        def load(self, get, device, act_dtype):
+            for n, part in self._children():
+                part.load(lambda rel, _n=n: get(f"{_n}.{rel}"), device, act_dtype)
+
+        def forward(self, resid, delta, ctx, cache):
+            x = self.norm.add_norm(resid, delta)
+            outs = [self.mixer.forward(x, ctx, cache), self.feed_forward.forward(x, ctx)]
+            # either may come as float32 planes of a split product; the next norm sums whatever it is given
+            return torch.stack([o.float().sum(0) if o.dim() == 3 else o.float() for o in outs])
+
+    register_norm("toy_shift_scale", ShiftScaleNorm, replace=True)
+    register_block("toy_parallel", ParallelBlock, replace=True)
+
+
+def _parallel_architecture():
+    from atoma_infer_amd.config import ModelConfig, key, register_architecture
+    from atoma_infer_amd.config.base import as_float, as_positive_int
+    from atoma_infer_amd.models import ModelSpec
+    from atoma_infer_amd.parts import OutputHead, TokenEmbedding, make_part
+
+    @dataclasses.dataclass(frozen=True)
+    class ParallelConfig(ModelConfig):
+        architectures = ("ToyParallelForCausalLM",)
+        width: int = key(convert=as_positive_int)
+        vocab: int = key(convert=as_positive_int)
+        heads: int = key(convert=as_positive_int)
+        kv_heads: int = key(convert=as_positive_int)
+        inter: int = key(convert=as_positive_int)
+        depth: int = key(convert=as_positive_int)
+        eps: float = key(convert=as_float)
+        max_positions: int = key(convert=as_positive_int)
+
+        def to_dict(self):
+            d = {f.name: getattr(self, f.name) for f in dataclasses.fields(self)}
+            d["architectures"] = ["ToyParallelForCausalLM"]
+            return d
+
+    def build(cfg: ParallelConfig) -> ModelSpec:
+        hd = cfg.width // cfg.heads
+        norm = lambda: make_part("norm", "toy_shift_scale", width=cfg.width, eps=cfg.eps)
+        layers = []
+        for i in range(cfg.depth):
+            pos = make_part("position", "rotary", head_size=hd, theta=10000.0, max_positions=cfg.max_positions)
+            mixer = make_part("mixer", "attention", width=cfg.width, num_heads=cfg.heads, num_kv_heads=cfg.kv_heads,
+                              head_size=hd, position=pos)
+            ffn = make_part("feed_forward", "swiglu", width=cfg.width, intermediate=cfg.inter)
+            layers.append((f"par.layers.{i}", make_part("block", "toy_parallel", norm=norm(), mixer=mixer,
+                                                        feed_forward=ffn)))
+        return ModelSpec(width=cfg.width, vocab_size=cfg.vocab, max_positions=cfg.max_positions,
+                         embedding=("par.embed", TokenEmbedding(cfg.vocab, cfg.width)), layers=layers,
+                         final_norm=("par.final_norm", norm()), head=("par.head", OutputHead(cfg.width, cfg.vocab)))
+
+    register_architecture("ToyParallelForCausalLM", ParallelConfig, build, replace=True)
+
+
+TOY_PARALLEL = {"architectures": ["ToyParallelForCausalLM"], "width": 96, "vocab": 173, "heads": 6, "kv_heads": 3,
+                "inter": 136, "depth": 3, "eps": 1e-4, "max_positions": 256}
+
+
+def parallel_plain_forward(tokens: List[int], w: Dict[str, torch.Tensor], cfg: dict) -> torch.Tensor:
+    H, nh, nkv = cfg["width"], cfg["heads"], cfg["kv_heads"]
+    hd, t = H // nh, len(tokens)
+
+    def norm(x, p):
+        mu = x.mean(-1, keepdim=True)
+        return (x - mu) / torch.sqrt(((x - mu) ** 2).mean(-1, keepdim=True) + cfg["eps"]) * w[p + "weight"] + w[p + "bias"]
+
+    c, s = P.rope_tables({"hidden_size": H, "num_attention_heads": nh, "rope_theta": 10000.0}, torch.arange(t))
+    x = w["par.embed.weight"][torch.tensor(tokens)]
+    for i in range(cfg["depth"]):
+        p = f"par.layers.{i}."
+        h = norm(x, p + "norm.")
+        q = P.apply_rope((h @ w[p + "mixer.q_proj.weight"].T).view(t, nh, hd), c, s)
+        k = P.apply_rope((h @ w[p + "mixer.k_proj.weight"].T).view(t, nkv, hd), c, s)
+        v = (h @ w[p + "mixer.v_proj.weight"].T).view(t, nkv, hd)
+        kk, vv = k.repeat_interleave(nh // nkv, 1), v.repeat_interleave(nh // nkv, 1)
+        o = P.attention_scores_softmax_pv(q.transpose(0, 1), kk.transpose(0, 1), vv.transpose(0, 1),
+                                          1 / math.sqrt(hd), True, None)
+        x = x + o.transpose(0, 1).reshape(t, H) @ w[p + "mixer.o_proj.weight"].T + P.swiglu_mlp(h, w, p + "ffn.")
+    return norm(x, "par.final_norm.") @ w["par.head.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_another_norm_and_another_block_arrangement(tmp_path, dtype):
+    """Registered here, built from config.json, loaded, stepped in portions beside decoded tokens: nothing in the
+    framework's files knows of them."""
+    from atoma_infer_amd.cache import plan_cache
+    from atoma_infer_amd.config import unregister_architecture
+    from atoma_infer_amd.models import load_model
+    from atoma_infer_amd.weights import write_random_model
+    _parallel_parts()
+    _parallel_architecture()
+    try:
+        d = write_random_model(str(tmp_path / "par"), TOY_PARALLEL, seed=4, dtype="bfloat16", norm_jitter=0.1)
+        model = load_model(d, dtype)
+        assert not model.spec.graph_safe()          # the toy parts do not say they can be replayed
+        plan = plan_cache(model.spec)
+        w = plain_weights(d)
+        reqs = {n: random_tokens(ln, TOY_PARALLEL["vocab"], 30 + i) for i, (n, ln) in enumerate([("a", 100), ("b", 37)])}
+        want = {n: parallel_plain_forward(t, w, TOY_PARALLEL) for n, t in reqs.items()}
+        sched = [([("a", 64)], []), ([("a", 3), ("b", 30)], []), ([("a", 1), ("b", 1)], []), ([("b", 2), ("a", 1)], []),
+                 ([("a", 31), ("b", 4)], ["a", "b"])]
+        got, runner = _toy_run(model, plan, reqs, sched, [10])
+        _toy_check(got, want, dtype)
+        assert runner.manager.num_free_pages(0) == 10
+    finally:
+        unregister_architecture("ToyParallelForCausalLM")
