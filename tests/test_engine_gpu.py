@@ -305,3 +305,46 @@ def test_layers_of_serving_size_in_mixed_steps(tmp_path, cfg):
         del runner
         torch.cuda.empty_cache()
     _plain_cache.clear()
+
+
+def test_decode_graphs_with_library_products_inside(tmp_path):
+    """With more than 64 decoding requests the linears of a step are the library's, inside the recorded graph.
+    Every replay is compared with the same step run eagerly, with eager work and a synchronisation between
+    replays: a library call that clears memory through a node of its own would show here after the first replay."""
+    from atoma_infer_amd.engine import StepEntry
+    model_dir = make_model_dir(str(tmp_path / "m"), LLAMA_1B_LAYERS, seed=5, dtype="bfloat16", norm_jitter=0.1)
+    vocab, n_req = LLAMA_1B_LAYERS["vocab_size"], 70
+    toks = [random_tokens(22 + (i % 9) + 14, vocab, 200 + i) for i in range(n_req + 1)]
+    graphed = make_runner(model_dir, "bfloat16", 16, 4 * (n_req + 1), slots=n_req + 1)
+    eager = make_runner(model_dir, "bfloat16", 16, 4 * (n_req + 1), slots=n_req + 1)
+    eager.use_graphs = False
+    for rn in (graphed, eager):
+        for i in range(n_req + 1):
+            rn.add_request(i)
+
+    def both(entries):
+        outs = []
+        for rn in (graphed, eager):
+            batch = [StepEntry(r, toks[r][rn.computed_len(r):rn.computed_len(r) + n], rn.computed_len(r), [n - 1])
+                     for r, n in entries]
+            outs.append(rn.step(batch).clone())
+        return outs
+
+    g, e = both([(r, len(toks[r]) - 14) for r in range(n_req)])          # the prompts, one step
+    assert torch.equal(g, e)
+    for step in range(12):
+        g, e = both([(r, 1) for r in range(n_req)])
+        assert torch.equal(g, e), f"decode step {step}"
+        assert bool(torch.isfinite(g).all())
+        if step in (3, 7):
+            g, e = both([(n_req, 9)])                                      # eager work between replays
+            assert torch.equal(g, e)
+        if step == 5:
+            torch.cuda.synchronize()
+    key = (n_req, 1)
+    assert key in graphed._graphs and graphed._graphs[key].graph is not None and not eager._graphs
+    # and the last replay against the plain model, for a few of the requests
+    last = {r: graphed.computed_len(r) - 1 for r in (0, 33, 69)}
+    got = {(f"r{r}", p): g[r].cpu() for r, p in last.items()}
+    check_against_plain(model_dir, {f"r{r}": toks[r] for r in last}, got, "bfloat16")
+    _plain_cache.clear()
