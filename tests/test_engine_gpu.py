@@ -348,3 +348,40 @@ def test_decode_graphs_with_library_products_inside(tmp_path):
     got = {(f"r{r}", p): g[r].cpu() for r, p in last.items()}
     check_against_plain(model_dir, {f"r{r}": toks[r] for r in last}, got, "bfloat16")
     _plain_cache.clear()
+
+
+def test_decode_graphs_are_dropped_and_recorded_again(model_dirs, monkeypatch):
+    """Only so many graphs are kept; the one unused longest goes.  With room for two, steps of one to four requests
+    take turns, so that graphs are dropped while the step before may still run, and recorded anew."""
+    from atoma_infer_amd.engine import StepEntry, step as step_module
+    monkeypatch.setattr(step_module, "MAX_GRAPHS", 2)
+    name, dtype = "B", "bfloat16"
+    vocab = TINY[name]["vocab_size"]
+    toks = [random_tokens(120, vocab, 300 + i) for i in range(4)]
+    graphed = make_runner(model_dirs[name], dtype, PAGE[name], 40)
+    eager = make_runner(model_dirs[name], dtype, PAGE[name], 40)
+    eager.use_graphs = False
+    for rn in (graphed, eager):
+        for i in range(4):
+            rn.add_request(i)
+
+    def both(entries):
+        outs = []
+        for rn in (graphed, eager):
+            batch = [StepEntry(r, toks[r][rn.computed_len(r):rn.computed_len(r) + n], rn.computed_len(r), [n - 1])
+                     for r, n in entries]
+            outs.append(rn.step(batch).clone())
+        return outs
+
+    g, e = both([(r, 20 + r) for r in range(4)])
+    assert torch.equal(g, e)
+    recorded = set()
+    for step in range(48):
+        n = [1, 2, 3, 4, 2, 1, 4, 3][step % 8] if step % 3 else 2
+        g, e = both([(r, 1) for r in range(n)])
+        assert torch.equal(g, e), f"step {step} with {n} requests"
+        assert len(graphed._graphs) <= 2
+        recorded |= {k for k, v in graphed._graphs.items() if v.graph is not None}
+    assert len(recorded) >= 2          # graphs were recorded, dropped and recorded again along the way
+    got = {("r0", graphed.computed_len(0) - 1): g[0].cpu()}
+    check_against_plain(model_dirs[name], {"r0": toks[0]}, got, dtype)
