@@ -88,7 +88,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int slot = wave % TASKS, part = wave / TASKS;   // which of the workgroup's tasks, which share of its keys
   // workgroups are numbered with the KV head running fastest: neighbours read the same block tables and finish
-  // together, and the longest tasks (which come first) start first
+  // together, and the longest tasks (which come first) start first.  The GPU deals workgroups to its eight XCDs in
+  // turn, so with eight KV heads (or a multiple) all tiles of a prompt that read one head's keys and values run on
+  // one XCD and find them in its L2.
   const int kvh = blockIdx.x % nkv;
   const int ti = (blockIdx.x / nkv) * TASKS + slot;
   // with KSPLIT > 1 every wave must reach the barrier below: a wave without work runs an empty range
