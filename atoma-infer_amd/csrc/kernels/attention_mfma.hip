@@ -90,7 +90,8 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   // workgroups are numbered with the KV head running fastest: neighbours read the same block tables and finish
   // together, and the longest tasks (which come first) start first.  The GPU deals workgroups to its eight XCDs in
   // turn, so with eight KV heads (or a multiple) all tiles of a prompt that read one head's keys and values run on
-  // one XCD and find them in its L2.
+  // one XCD and find them in its L2 (with the KV head running slowest a prompt of 2,048 tokens takes 48 us instead
+  // of 37, a portion of 2,048 tokens behind 14,336 others 373 instead of 359; from 30,000 keys on it is all one).
   const int kvh = blockIdx.x % nkv;
   const int ti = (blockIdx.x / nkv) * TASKS + slot;
   // with KSPLIT > 1 every wave must reach the barrier below: a wave without work runs an empty range
