@@ -385,3 +385,54 @@ def test_decode_graphs_are_dropped_and_recorded_again(model_dirs, monkeypatch):
     assert len(recorded) >= 2          # graphs were recorded, dropped and recorded again along the way
     got = {("r0", graphed.computed_len(0) - 1): g[0].cpu()}
     check_against_plain(model_dirs[name], {"r0": toks[0]}, got, dtype)
+
+
+def _random_configuration(rng):
+    """Every size drawn: head size in steps of 16, any number of heads and groups, widths and a vocabulary that
+    are no powers of two (the feed-forward width sometimes no multiple of 8), one to three layers."""
+    hd = rng.choice([16, 32, 48, 64, 80, 96, 128, 256])
+    nkv = rng.choice([1, 2, 3, 5])
+    nh = nkv * rng.choice([1, 2, 3, 4, 7])
+    while nh * hd > 1536:
+        nh = max(nh // 2, 1)
+    if nh % nkv:
+        nkv = 1
+    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": nh * hd,
+           "intermediate_size": rng.choice([rng.randint(8, 700), 8 * rng.randint(2, 90), 32 * rng.randint(1, 24)]),
+           "vocab_size": rng.randint(50, 3000), "num_hidden_layers": rng.randint(1, 3),
+           "num_attention_heads": nh, "num_key_value_heads": nkv, "rms_norm_eps": rng.choice([1e-5, 1e-6, 3e-6]),
+           "rope_theta": rng.choice([10000.0, 500000.0]), "max_position_embeddings": 1024,
+           "tie_word_embeddings": rng.random() < 0.5}
+    if rng.random() < 0.5:
+        cfg["rope_scaling"] = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                               "original_max_position_embeddings": 64, "rope_type": "llama3"}
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations_step_like_the_plain_model(tmp_path, seed):
+    rng = random.Random(7000 + seed)
+    cfg = _random_configuration(rng)
+    model_dir = make_model_dir(str(tmp_path / "m"), cfg, seed=seed, dtype="bfloat16", norm_jitter=0.1)
+    vocab = cfg["vocab_size"]
+    la, lb, lc = rng.randint(150, 400), rng.randint(20, 200), rng.randint(2, 70)
+    requests = {"a": random_tokens(la, vocab, 1), "b": random_tokens(lb, vocab, 2), "c": random_tokens(lc, vocab, 3)}
+    first = rng.randint(1, la - 40)
+    steps, left = [([("a", first)], [])], {"a": la - first, "b": lb, "c": lc}
+    while any(left.values()):
+        entries = []
+        for k in ("a", "b", "c"):
+            if left[k] and rng.random() < 0.8:
+                n = min(left[k], rng.choice([1, 1, 1, 2, 3, 17, 40, 70, 130]))
+                entries.append((k, n))
+                left[k] -= n
+        if entries:
+            rng.shuffle(entries)
+            steps.append((entries, []))
+    pages = sum(-(-len(v) // 16) for v in requests.values()) + 2
+    for dtype in DTYPES:
+        runner = make_runner(model_dir, dtype, 16, pages)
+        got = run_schedule(runner, requests, steps)
+        check_against_plain(model_dir, requests, got, dtype)
+        del runner
+    _plain_cache.clear()
