@@ -53,6 +53,24 @@ def test_greedy_generation_tiny_a_workload(model_dirs):
     assert [o.inference_outputs[0].token_ids for o in outs2] == want
 
 
+def test_engine_with_every_option_at_its_default(model_dirs):
+    """No option given: the pool is sized from the memory that is free, capped at what the scheduler's limits can
+    ever use, and generation is that of the plain model."""
+    from atoma_infer_amd.engine.engine import LlmEngine
+    from atoma_infer_amd.sampling import GenerateParameters
+    d = model_dirs["C"]
+    w, cfg = plain_weights(d), plain_config(d)
+    prompts = [random_tokens(40, TINY["C"]["vocab_size"], 5), random_tokens(3, TINY["C"]["vocab_size"], 6)]
+    want = [plain_llama.greedy_generate(p, 6, w, cfg) for p in prompts]
+    eng = LlmEngine(d, "float32")
+    sched, mgr = eng.scheduler_config, eng.runner.manager
+    assert sched.max_model_len == TINY["C"]["max_position_embeddings"]        # the model's own limit caps the default
+    assert mgr.num_pages() == sched.max_num_sequences * -(-sched.max_model_len // eng.cache_config.block_size)
+    outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=6, ignore_eos_token=True))
+    assert [o.inference_outputs[0].token_ids for o in outs] == want
+    assert mgr.num_free_pages() == mgr.num_pages()
+
+
 def test_tiny_b_workload_portions_beside_decodes_with_temperature(model_dirs):
     """The tiny workload B: prompts of 37, 1 and 20 ids in 16-token portions alongside decodes, temperature
     0.7 with a fixed seed.  The sampled tokens must be what the plain model and plain sampler give for the same
