@@ -50,9 +50,9 @@ _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
 _module_locks: Dict[str, threading.Lock] = {}
 
-# head sizes whose attention module the build check compiles ahead of time; any other multiple of 16 up to 256
-# is compiled when a model with that head size is first used
-STANDARD_HEAD_SIZES = (16, 32, 48, 64, 80, 96, 128, 256)
+# head sizes whose attention module the build check compiles ahead of time: every one the kernel takes (a few
+# seconds each); a model compiles only its own when it is first used and no built module is there
+STANDARD_HEAD_SIZES = tuple(range(16, 257, 16))
 
 
 def _lock_for(name: str) -> threading.Lock:

@@ -291,6 +291,32 @@ def test_paged_attention(nh, nkv, hd, page, window, entries, kind):
         row += c
 
 
+@pytest.mark.parametrize("hd", list(range(16, 257, 16)))
+def test_attention_at_every_head_size(hd):
+    """Every multiple of 16 up to 256, with grouped heads: a prompt of several tiles, a portion behind a prefix,
+    and decoded tokens whose keys are cut into chunks and merged."""
+    from atoma_infer_amd.kernels import attention_bf16
+    nh, nkv, page = 6, 2, 16
+    entries = [(0, 70), (300, 9), (700, 1), (129, 1), (15, 1)]
+    starts, counts = [s for s, _ in entries], [c for _, c in entries]
+    ks, vs, kc, vc, bt = paged_setup([s + c for s, c in entries], nkv, hd, page, torch.bfloat16, seed=hd)
+    t = sum(counts)
+    g = torch.Generator().manual_seed(hd)
+    qkv = (torch.randn(t, (nh + 2 * nkv) * hd, generator=g) * 1.5).bfloat16().to(DEV)
+    out = torch.full((t, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    scale = 1.0 / math.sqrt(hd)
+    assert attention_bf16.try_attention(qkv, kc, vc, out, FakeCtx(starts, counts), FakeCache(bt, page), scale, 0,
+                                        nh, nkv, hd)
+    row = 0
+    for e, (s, c) in enumerate(entries):
+        q = qkv[row:row + c, : nh * hd].cpu().view(c, nh, hd)
+        want = plain_attention(q, ks[e], vs[e], s, scale, 0, nh // nkv).reshape(c, nh * hd)
+        got = out[row:row + c].double().cpu()
+        err = (got - want).abs().max() / want.abs().max()
+        assert err < 2e-2, f"head size {hd}, entry {e} ({s}, {c}): {err:.3e}"
+        row += c
+
+
 STAND_OUT = [
     # (window, [(start, count)], key that gets the large score)
     (0, [(699, 1)], 0), (0, [(699, 1)], 15), (0, [(699, 1)], 16), (0, [(699, 1)], 127), (0, [(699, 1)], 128),
