@@ -291,12 +291,17 @@ def test_paged_attention(nh, nkv, hd, page, window, entries, kind):
         row += c
 
 
-@pytest.mark.parametrize("hd", list(range(16, 257, 16)))
-def test_attention_at_every_head_size(hd):
-    """Every multiple of 16 up to 256, with grouped heads: a prompt of several tiles, a portion behind a prefix,
-    and decoded tokens whose keys are cut into chunks and merged."""
+HEADS_AND_SIZES = [(6, 2, hd) for hd in range(16, 257, 16)] + [
+    # groups of 1, 7, 32, 33 and 40 heads to a KV head (more than 32 take several pieces of rows), many KV heads
+    (5, 5, 64), (7, 1, 32), (64, 2, 64), (33, 1, 32), (40, 1, 64), (80, 2, 16), (24, 24, 48), (9, 3, 128)]
+
+
+@pytest.mark.parametrize("nh,nkv,hd", HEADS_AND_SIZES)
+def test_attention_at_every_head_size_and_grouping(nh, nkv, hd):
+    """Every multiple of 16 up to 256, and groups of any size: a prompt of several tiles, a portion behind a
+    prefix, and decoded tokens whose keys are cut into chunks and merged."""
     from atoma_infer_amd.kernels import attention_bf16
-    nh, nkv, page = 6, 2, 16
+    page = 16
     entries = [(0, 70), (300, 9), (700, 1), (129, 1), (15, 1)]
     starts, counts = [s for s, _ in entries], [c for _, c in entries]
     ks, vs, kc, vc, bt = paged_setup([s + c for s, c in entries], nkv, hd, page, torch.bfloat16, seed=hd)
@@ -616,3 +621,40 @@ def test_tokens_outside_the_table_and_rows_of_nan_do_no_harm():
         assert all(0 <= t < 1000 for t in tok), tok
         if temp == 0.0:
             assert tok[0] == int(torch.argmax(logits[0])) and tok[3] == 0
+
+
+@pytest.mark.parametrize("whole", [False, True])
+@pytest.mark.parametrize("nh,nkv,hd", [(40, 1, 64), (33, 1, 32), (6, 2, 112), (64, 2, 64), (3, 3, 208)])
+def test_decode_plans_with_large_groups(nh, nkv, hd, whole, monkeypatch):
+    """The task lists of decode steps as the engine builds them (every request owns its bucket's chunk slots), for
+    groups of more than 32 heads, which take several pieces of rows: chunks merged by the second kernel, and whole
+    key ranges walked by eight waves."""
+    import numpy as np
+    from atoma_infer_amd.kernels import attention_bf16
+    if whole:
+        if attention_bf16.max_waves_for(hd) < 8:
+            pytest.skip("eight waves a task do not fit this head size")
+        monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 2)
+    group, page = nh // nkv, 16
+    starts = [700, 129, 15, 256, 511]
+    counts = [1] * len(starts)
+    ks, vs, kc, vc, bt = paged_setup([s + 1 for s in starts], nkv, hd, page, torch.bfloat16, seed=hd + nh)
+    t = len(starts)
+    g = torch.Generator().manual_seed(3)
+    qkv = (torch.randn(t, (nh + 2 * nkv) * hd, generator=g) * 1.5).bfloat16().to(DEV)
+    out = torch.full((t, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ctx = FakeCtx(starts, counts)
+    arr, meta = attention_bf16.build_tasks(np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32),
+                                           group, 0, 3, kv_heads=nkv, max_waves=attention_bf16.max_waves_for(hd))
+    assert (meta[1] == 0) == whole                       # no merge records with whole ranges
+    ctx.plans = {attention_bf16.plan_key(group, 0, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
+    scale = 1.0 / math.sqrt(hd)
+    # the block tables of a bucket of three cover 768 keys
+    wide = torch.zeros((t, 3 * 256 // page), dtype=torch.int32, device=DEV)
+    wide[:, : bt.shape[1]] = bt
+    assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, FakeCache(wide, page), scale, 0, nh, nkv, hd)
+    for e, s in enumerate(starts):
+        q = qkv[e:e + 1, : nh * hd].cpu().view(1, nh, hd)
+        want = plain_attention(q, ks[e], vs[e], s, scale, 0, group).reshape(1, nh * hd)
+        err = (out[e:e + 1].double().cpu() - want).abs().max() / want.abs().max()
+        assert err < 2e-2, f"request {e} at {s}: {err:.3e}"
