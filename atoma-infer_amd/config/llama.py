@@ -69,6 +69,10 @@ class LlamaConfig(ModelConfig):
     eos_token_id: Tuple[int, ...] = key(default=(), convert=_eos)
     rope_scaling: Optional[RopeScaling] = key(default=None, convert=RopeScaling.from_json)
     tie_word_embeddings: bool = key(default=False, convert=as_bool)
+    # attention over the last N keys only (none: all keys).  The reference's models report it to the engine through
+    # ``sliding_window()`` (backends/vllm/src/model_executor.rs:116-140; none for Llama) and its ``[cache]``
+    # section has the same option (backends/vllm/src/config.rs:137-159), which the engine writes in here.
+    sliding_window: Optional[int] = key(default=None, convert=as_positive_int)
     # Keys the reference does not read.  They are accepted only with the value
     # that the reference's code fixes, so that a checkpoint which needs another
     # value is refused instead of being run wrongly.
@@ -133,4 +137,6 @@ class LlamaConfig(ModelConfig):
             d["eos_token_id"] = self.eos_token_id[0] if len(self.eos_token_id) == 1 else list(self.eos_token_id)
         if self.rope_scaling is not None:
             d["rope_scaling"] = self.rope_scaling.to_dict()
+        if self.sliding_window is not None:
+            d["sliding_window"] = self.sliding_window
         return d

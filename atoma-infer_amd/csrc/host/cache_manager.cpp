@@ -108,11 +108,15 @@ int cm_can_reserve(void* h, int64_t id, int64_t new_len) {
   return 1;
 }
 
-// 1 if a request of new_len tokens could ever be held, with every page free.
+// 1 if a request of new_len tokens could ever be held, with every page free.  A group with a window gives pages
+// back as the request moves on: it must hold the window and the page that the next token opens.
 int cm_fits_at_all(void* h, int64_t new_len) {
   Manager* m = static_cast<Manager*>(h);
-  for (const Group& g : m->groups)
-    if (blocks_for(g, new_len) > g.num_pages) return 0;
+  for (const Group& g : m->groups) {
+    int64_t need = blocks_for(g, new_len);
+    if (g.window > 0 && blocks_for(g, g.window) + 1 < need) need = blocks_for(g, g.window) + 1;
+    if (need > g.num_pages) return 0;
+  }
   return 1;
 }
 

@@ -9,8 +9,8 @@
 //      blocks those behind it (scheduler.rs:897-1016).
 // Pages are reserved for what a step adds.  When they run out for a running request, the running request that
 // arrived last is preempted by recomputation (scheduler.rs:650-690, 1778-1896): what it holds goes back and it
-// returns to the front of the waiting queue.  A request that cannot grow while it runs alone is finished
-// ("capped").  A waiting request longer than the model length, or than the whole pool, is dropped ("ignored").
+// returns to the front of the waiting queue.  A request that runs alone tries shorter portions, and is finished
+// ("capped") when not even one token finds a page.  A waiting request longer than the model length, or than the whole pool, is dropped ("ignored").
 //
 // The scheduler keeps four counters per request (tokens held, tokens computed, tokens sampled, frozen); whoever
 // runs the steps reports them before each plan.  It calls the cache manager of the same library directly and lists
@@ -137,7 +137,7 @@ struct Sched {
       Req& r = reqs[order[i]];
       if (!r.running) continue;  // preempted while serving an earlier request
       if ((int)entries.size() >= max_seqs) break;
-      const int n = chunk(r, max_tokens - used_tokens());
+      int n = chunk(r, max_tokens - used_tokens());
       if (n <= 0) continue;
       while (!cm_can_reserve(cm, r.uid, r.computed + n)) {
         // the latest arrival that is not just waiting for its last token (that one frees its pages soon)
@@ -148,7 +148,12 @@ struct Sched {
             break;
           }
         if (victim == &r && running.size() == 1) {
-          // nothing else to give back: the pool cannot hold this request any longer
+          // nothing else to give back: a shorter portion may still find its pages (with a window of keys, pages
+          // come back as the request moves on); if one token finds none, the pool cannot hold this request
+          if (n > 1 && chunked) {
+            n /= 2;
+            continue;
+          }
           drop_running(r.uid);
           release(r.uid);
           r.running = false;

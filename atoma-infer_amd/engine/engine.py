@@ -40,8 +40,14 @@ class LlmEngine:
     def __init__(self, model: Union[str, Model], dtype: str = "bfloat16", *, cache: Optional[CacheConfig] = None,
                  scheduler: Optional[SchedulerConfig] = None, validation: Optional[ValidationConfig] = None,
                  device: str = "cuda:0"):
-        self.model = load_model(model, parse_dtype(dtype), device) if isinstance(model, str) else model
         self.cache_config = cache or CacheConfig()
+        window = self.cache_config.sliding_window
+        if isinstance(model, str):
+            self.model = load_model(model, parse_dtype(dtype), device, sliding_window=window)
+        else:
+            self.model = model
+            if window is not None and getattr(model.config, "sliding_window", None) != window:
+                raise ValueError("[cache] sliding_window differs from that of the model given; load the model with it")
         self.scheduler_config = scheduler or SchedulerConfig()
         self.validation = validation or ValidationConfig()
         self.cache_config.validate()

@@ -14,8 +14,9 @@ Each call of ``schedule`` plans one step under a token budget (``max_num_batched
 Pages are reserved for what a step adds, not for the whole prompt up front.  **When pages run out** for a running
 request, the running request that arrived last is preempted by recomputation: its pages are given back, it
 returns to the *front* of the waiting queue and later prefills its prompt and the tokens it had generated
-(scheduler.rs:650-690, 1778-1896).  If the request that cannot grow is the only one running, it is finished as
-"length_capped": nothing could be given back for it.
+(scheduler.rs:650-690, 1778-1896).  If the request that cannot grow is the only one running, it takes portions half
+as long (with a window of keys, pages come back as it moves on); when not even one token finds a page it is
+finished as "length_capped": nothing could be given back for it.
 
 The decisions are made in the host library (csrc/host/scheduler.cpp), next to the cache manager it draws pages
 from; this module keeps the ``Request`` objects, reports their counters before each plan and applies the plan's

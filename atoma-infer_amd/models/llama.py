@@ -23,7 +23,8 @@ def build_llama(cfg: LlamaConfig) -> ModelSpec:
         position = make_part("position", "rotary", head_size=hd, theta=cfg.rope_theta,
                              max_positions=cfg.max_position_embeddings, scaling=scaling)
         mixer = make_part("mixer", "attention", width=cfg.hidden_size, num_heads=cfg.num_attention_heads,
-                          num_kv_heads=cfg.num_key_value_heads, head_size=hd, position=position)
+                          num_kv_heads=cfg.num_key_value_heads, head_size=hd, position=position,
+                          window=cfg.sliding_window)
         ffn = make_part("feed_forward", "swiglu", width=cfg.hidden_size, intermediate=cfg.intermediate_size)
         block = make_part("block", "pre_norm",
                           norm1=make_part("norm", "rmsnorm", width=cfg.hidden_size, eps=cfg.rms_norm_eps),

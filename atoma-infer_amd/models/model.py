@@ -48,11 +48,13 @@ class Model:
         return spec.head[1].forward(x)
 
 
-def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") -> Model:
+def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0",
+               sliding_window: Optional[int] = None) -> Model:
     """Build the model that ``model_dir/config.json`` names and bind ``model_dir``'s weights to it.
 
     ``dtype`` is the activation and cache dtype: "bfloat16" runs the serving kernels, "float32" everything in
-    true 32-bit arithmetic.  Weights stay as stored (bfloat16 or float32) in both.
+    true 32-bit arithmetic.  Weights stay as stored (bfloat16 or float32) in both.  ``sliding_window`` overrides
+    what config.json says of it (the engine's ``[cache]`` option).
     """
     if dtype not in _ACT:
         raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}")
@@ -60,6 +62,10 @@ def load_model(model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0") 
     if dev.type != "cuda" or not torch.cuda.is_available():
         raise RuntimeError("this engine runs on a GPU only (device 'cuda:N'); no GPU is visible")
     arch, cfg = load_model_config(model_dir)
+    if sliding_window is not None:
+        if not any(f.name == "sliding_window" for f in dataclasses.fields(cfg)):
+            raise ValueError(f"the configuration of {arch.name} has no sliding_window to set")
+        cfg = dataclasses.replace(cfg, sliding_window=int(sliding_window))
     spec = arch.build(cfg)
     load_into(spec, model_dir, dev, _ACT[dtype])
     return Model(arch, cfg, spec, dev, _ACT[dtype])

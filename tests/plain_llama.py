@@ -147,10 +147,13 @@ def swiglu_mlp(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str) -> torc
 
 
 def block(x: torch.Tensor, w: Dict[str, torch.Tensor], i: int, cfg: dict, positions: torch.Tensor) -> torch.Tensor:
-    """Pre-norm block with two residual sums (models/src/llama.rs:393-410)."""
+    """Pre-norm block with two residual sums (models/src/llama.rs:393-410).  A ``sliding_window`` in ``cfg`` (the
+    reference's models report one through ``sliding_window()``, backends/vllm/src/model_executor.rs:116-140, and
+    hand it to the attention kernel as its left window) limits every layer's attention to that many keys."""
     p = f"model.layers.{i}."
     eps = cfg["rms_norm_eps"]
-    h = x + self_attention(rms_norm(x, w[p + "input_layernorm.weight"], eps), w, p + "self_attn.", cfg, positions)
+    h = x + self_attention(rms_norm(x, w[p + "input_layernorm.weight"], eps), w, p + "self_attn.", cfg, positions,
+                           window=cfg.get("sliding_window"))
     return h + swiglu_mlp(rms_norm(h, w[p + "post_attention_layernorm.weight"], eps), w, p + "mlp.")
 
 

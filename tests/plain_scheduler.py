@@ -10,8 +10,8 @@ counted by ``PlainPages`` (one group of pages, no window).  The policy is the re
 3. waiting requests in order, while budget, pages and slots last; the head of the queue blocks those behind it.
 
 When pages run out for a running request, the running request that arrived last (and is not frozen) is preempted:
-its pages go back, it returns to the front of the waiting queue with nothing computed.  A request that cannot grow
-while it runs alone is capped.  A waiting request longer than the model length or the pool is ignored.
+its pages go back, it returns to the front of the waiting queue with nothing computed.  A request that runs alone
+tries portions half as long, and is capped when not even one token finds a page.  A waiting request longer than the model length or the pool is ignored.
 """
 from collections import deque
 
@@ -161,6 +161,9 @@ class PlainScheduler:
             while not self.pages.can_reserve(r.uid, r.num_computed + n):
                 victim = next((v for v in reversed(self.running) if not v.frozen), r)
                 if victim is r and len(self.running) == 1:
+                    if n > 1 and lim.cut:
+                        n //= 2           # alone: a shorter portion may still find its pages
+                        continue
                     self.running.remove(r)
                     self._release(r)
                     r.status = "capped"

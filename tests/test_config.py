@@ -28,6 +28,15 @@ def test_llama_reads_every_key():
         == (8.0, 1.0, 4.0, 64, "llama3")
     again = LlamaConfig.from_dict(cfg.to_dict())
     assert again == cfg
+    # an optional window of keys: none unless given, kept through to_dict, and its layers' cache plan has it
+    assert cfg.sliding_window is None and "sliding_window" not in cfg.to_dict()
+    windowed = LlamaConfig.from_dict(dict(TINY_B, sliding_window=48))
+    assert windowed.sliding_window == 48 and LlamaConfig.from_dict(windowed.to_dict()) == windowed
+    from atoma_infer_amd.cache import plan_cache
+    arch = resolve_architecture(windowed.to_dict())
+    assert [g.spec.window for g in plan_cache(arch.build(windowed)).groups] == [48]
+    with pytest.raises(ConfigError):
+        LlamaConfig.from_dict(dict(TINY_B, sliding_window=0))
 
 
 def test_one_error_lists_every_fault():

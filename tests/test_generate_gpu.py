@@ -71,6 +71,42 @@ def test_engine_with_every_option_at_its_default(model_dirs):
     assert mgr.num_free_pages() == mgr.num_pages()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cache_option_sliding_window(model_dirs, dtype):
+    """``[cache] sliding_window``: every layer attends the last N keys only, and pages that the window has passed
+    go back while the request runs, so a pool far smaller than the sequences serves them."""
+    from atoma_infer_amd.config import CacheConfig, SchedulerConfig
+    from atoma_infer_amd.engine.engine import LlmEngine
+    from atoma_infer_amd.sampling import GenerateParameters
+    d, window = model_dirs["C"], 40
+    w, cfg = plain_weights(d), dict(plain_config(d), sliding_window=window)
+    vocab = TINY["C"]["vocab_size"]
+    prompts = [random_tokens(200, vocab, 11), random_tokens(90, vocab, 12)]
+    eng = LlmEngine(d, dtype, cache=CacheConfig(block_size=16, num_gpu_blocks_override=12, sliding_window=window),
+                    scheduler=SchedulerConfig(max_num_batched_tokens=32, max_num_sequences=2, max_model_len=400))
+    assert eng.model.config.sliding_window == window
+    outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=30, ignore_eos_token=True))
+    assert eng.stats["preemptions"] == 0          # 230 and 120 tokens would need 23 pages without the window
+    assert eng.runner.manager.num_free_pages() == 12
+    for p, o in zip(prompts, outs):
+        got = o.inference_outputs[0].token_ids
+        if dtype == "float32":
+            assert got == plain_llama.greedy_generate(p, 30, w, cfg)
+        else:
+            # bfloat16 may turn a near tie: every token must be among the plain model's best few given the same past
+            seq = list(p)
+            for tok in got:
+                logits = plain_llama.forward(seq, w, cfg)[-1]
+                assert logits[tok] >= logits.max() - 0.05 * (logits.max() - logits.min())
+                seq.append(tok)
+    # all keys again without the option: other tokens (the window does change what is computed)
+    full = LlmEngine(d, "float32", cache=CacheConfig(block_size=16, num_gpu_blocks_override=40),
+                     scheduler=SchedulerConfig(max_num_batched_tokens=32, max_num_sequences=2, max_model_len=400))
+    outs_full = full.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=30, ignore_eos_token=True))
+    assert [o.inference_outputs[0].token_ids for o in outs_full] == \
+        [plain_llama.greedy_generate(p, 30, w, plain_config(d)) for p in prompts]
+
+
 def test_tiny_b_workload_portions_beside_decodes_with_temperature(model_dirs):
     """The tiny workload B: prompts of 37, 1 and 20 ids in 16-token portions alongside decodes, temperature
     0.7 with a fixed seed.  The sampled tokens must be what the plain model and plain sampler give for the same

@@ -161,6 +161,66 @@ def test_a_request_that_outgrows_the_pool_alone_is_capped():
     assert cache.num_free_pages() == 2 and not s.has_unfinished()
 
 
+def test_a_request_alone_takes_shorter_portions_before_it_gives_up():
+    cache2 = CacheManager([GroupGeometry(4, 5)], 8)
+    s2 = Scheduler(SchedulerConfig(max_num_batched_tokens=64, max_num_sequences=8, max_model_len=256), cache2)
+    blocker, c = make_request(5, 4, max_new=30), make_request(6, 16)
+    s2.add(blocker)
+    run_step(s2, s2.schedule())                 # blocker holds 1 page (4 tokens) and will need a 2nd
+    s2.add(c)
+    out = s2.schedule()                         # blocker decodes (page 2), c's 16 tokens need 4 pages, 3 are free
+    assert [(e.request.uid, e.num_tokens) for e in out.entries] == [(5, 1)]      # the head of the queue waits
+    s2.finish(blocker, Status.FINISHED_STOPPED)
+    out = s2.schedule()
+    assert [(e.request.uid, e.num_tokens) for e in out.entries] == [(6, 16)]
+    run_step(s2, out)
+    # alone with 4 of 5 pages: decoding goes on until the pool is full, then it is capped, not preempted
+    for _ in range(8):
+        out = s2.schedule()
+        if out.capped:
+            break
+        assert [(e.request.uid, e.num_tokens) for e in out.entries] == [(6, 1)]
+        run_step(s2, out)
+    assert [r.uid for r in out.capped] == [6] and c.num_computed == 20
+    # a running request whose next portion does not fit while it is alone takes half of it, and half again
+    cache3 = CacheManager([GroupGeometry(4, 6)], 8)
+    s3 = Scheduler(SchedulerConfig(max_num_batched_tokens=8, max_num_sequences=8, max_model_len=256,
+                                   max_prefill_chunk=0), cache3)
+    d = make_request(7, 23)                     # 6 pages in all: fits at all
+    s3.add(d)
+    for want in (8, 8):
+        out = s3.schedule()
+        assert [(e.request.uid, e.num_tokens) for e in out.entries] == [(7, want)]
+        run_step(s3, out)
+    hog = cache3._lib.cm_add_request(cache3.handle, 99)       # someone else takes the last two pages but one
+    assert hog >= 0
+    cache3.reserve(99, 4)
+    out = s3.schedule()                         # 7 tokens left need 2 pages, 1 is free: 7 // 2 = 3 fit
+    assert [(e.request.uid, e.num_tokens, e.do_sample) for e in out.entries] == [(7, 3, False)]
+    cache3.check()
+
+
+def test_a_window_of_keys_lets_long_requests_into_a_small_pool():
+    """A group that keeps a window gives pages back as a request moves on (cache_manager.cpp): the pool must hold
+    the window and one page more, not the whole request."""
+    cache = CacheManager([GroupGeometry(4, 5, window=10)], 4)
+    assert cache.fits_at_all(1000) and not CacheManager([GroupGeometry(4, 3, window=10)], 4).fits_at_all(1000)
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=8, max_num_sequences=4, max_model_len=2000), cache)
+    a = make_request(0, 100, max_new=4)
+    s.add(a)
+    steps = 0
+    while s.has_unfinished():
+        out = s.schedule()
+        assert not out.ignored and not out.capped and out.entries
+        for e in out.entries:
+            cache.release_behind(e.request.uid, e.request.num_computed + e.num_tokens)    # as the runner does
+        run_step(s, out)
+        cache.check()
+        steps += 1
+        assert steps < 200
+    assert len(a.output_ids) == 4 and cache.num_free_pages() == 5
+
+
 def test_abort_frees_and_unchunked_prompts_wait_for_room():
     s, cache = make_scheduler(pages=128, page=4, max_num_batched_tokens=256, max_model_len=256,
                               enable_chunked_prefill=False)
