@@ -54,3 +54,5 @@ def test_library_thresholds():
     assert not wins(64, 3072, 2048, torch.bfloat16) and wins(65, 3072, 2048, torch.bfloat16)
     assert wins(33, 16384, 2048, torch.bfloat16) and not wins(32, 16384, 2048, torch.bfloat16)
     assert wins(17, 128256, 2048, torch.float32) == gemm_bf16._MM_OUT_DTYPE and not wins(16, 128256, 2048, torch.float32)
+    # the head: eight waves splitting K up to 8 rows, then 64 rows of W a wave and four waves splitting K
+    assert [gemm_bf16._plan(m, 128256, 2048, False) for m in (8, 9, 16)] == [(2, 8, 1), (4, 4, 1), (4, 4, 1)]
