@@ -104,6 +104,15 @@ def _live_pieces(rows: int, qt: int, live_tokens: int):
     return out
 
 
+def _chunk_slots(bucket: int, chunk: int, window: int) -> int:
+    """Partial results that a decoded token of a graph's bucket owns: one per chunk of the bucket's keys, or, with
+    a window, per chunk that a window can touch wherever it lies (its first chunk is then slot 0)."""
+    slots = -(-(bucket * CHUNK) // chunk)
+    if window > 0:
+        slots = min(slots, -(-window // chunk) + 1)
+    return slots
+
+
 _NULL_TASK = np.asarray((-1, 0, 1, 0, 0, 0, -1, 0, 0, 0, 0, 0), dtype=np.int32)
 
 
@@ -174,6 +183,8 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     chunk, waves = CHUNK, 1
     if split_entries:
         most = bucket * CHUNK if bucket is not None else max(int(starts[e]) + int(counts[e]) for e in split_entries)
+        if bucket is not None and window > 0:
+            most = min(most, window + CHUNK)
         chunk, waves = chunk_for(len(split_entries), most, kv_heads)
         waves = min(waves, max_waves)
     for e in range(len(starts)):
@@ -194,12 +205,14 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
             live = _live_pieces(rows, qt, min(qt, count - tok0))
             if do_split:
                 c_first, c_last = lo // chunk, (k_end - 1) // chunk
-                slots = -(-(bucket * CHUNK) // chunk) if bucket is not None else c_last + 1
+                # slot j holds chunk c_first + j
+                slots = _chunk_slots(bucket, chunk, window) if bucket is not None else c_last - c_first + 1
                 for row0 in live:
-                    combine.append((e, tok0, qt, row0, 0, 0, n_part + c_first, c_last - c_first + 1) + tail)
-                    for c in range(slots):
-                        if c_first <= c <= c_last:
-                            split.append((e, tok0, qt, row0, c * chunk, min((c + 1) * chunk, k_end), n_part + c, 0) + tail)
+                    combine.append((e, tok0, qt, row0, 0, 0, n_part, c_last - c_first + 1) + tail)
+                    for j in range(slots):
+                        c = c_first + j
+                        if c <= c_last:
+                            split.append((e, tok0, qt, row0, c * chunk, min((c + 1) * chunk, k_end), n_part + j, 0) + tail)
                         elif bucket is not None:
                             split.append(null)
                     n_part += slots
@@ -235,7 +248,8 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     lo = np.maximum(0, starts - window + 1) if window > 0 else np.zeros(s, dtype=np.int64)
     row_chunks = -(-group // 32)
     # the bucket, not the step's longest request, decides between whole ranges and chunks: a graph holds one of them
-    chunk, waves = chunk_for(s, bucket * CHUNK, kv_heads, whole_ok=max_waves >= 8)
+    keys = bucket * CHUNK if window <= 0 else min(bucket * CHUNK, window + CHUNK)      # what a token can see
+    chunk, waves = chunk_for(s, keys, kv_heads, whole_ok=max_waves >= 8)
     waves = min(waves, max_waves)
     if chunk == 0:
         whole = np.zeros((s, row_chunks, 12), dtype=np.int32)
@@ -249,10 +263,11 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
         whole[..., 9] = 1
         whole[..., 10] = starts[:, None]
         return whole.reshape(-1, 12), (s * row_chunks, 0, 0, waves)
-    slots = -(-(bucket * CHUNK) // chunk)
-    c = np.arange(slots, dtype=np.int64)
+    slots = _chunk_slots(bucket, chunk, window)
+    j = np.arange(slots, dtype=np.int64)
     c_first, c_last = lo // chunk, (k_end - 1) // chunk
-    valid = (c[None, :] >= c_first[:, None]) & (c[None, :] <= c_last[:, None])          # [s, slots]
+    c = c_first[:, None] + j[None, :]                          # [s, slots]: slot j holds chunk c_first + j
+    valid = c <= c_last[:, None]
     main = np.zeros((s, row_chunks, slots, 12), dtype=np.int32)
     e = np.arange(s, dtype=np.int64)
     rc = np.arange(row_chunks, dtype=np.int64)
@@ -260,9 +275,9 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     main[..., 0] = np.where(v, e[:, None, None], -1)
     main[..., 2] = 1
     main[..., 3] = np.where(v, 32 * rc[None, :, None], 0)
-    main[..., 4] = np.where(v, (c * chunk)[None, None, :], 0)
+    main[..., 4] = np.where(v, (c * chunk)[:, None, :], 0)
     main[..., 5] = np.where(v, np.minimum((c + 1) * chunk, k_end[:, None])[:, None, :], 0)
-    part = (e[:, None, None] * row_chunks + rc[None, :, None]) * slots + c[None, None, :]
+    part = (e[:, None, None] * row_chunks + rc[None, :, None]) * slots + j[None, None, :]
     main[..., 6] = np.where(v, part, -1)
     main[..., 8] = np.where(v, e[:, None, None], 0)
     main[..., 9] = np.where(v, 1, 0)
@@ -277,7 +292,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     comb[..., 0] = e[:, None]
     comb[..., 2] = 1
     comb[..., 3] = 32 * rc[None, :]
-    comb[..., 6] = (e[:, None] * row_chunks + rc[None, :]) * slots + c_first[:, None]
+    comb[..., 6] = (e[:, None] * row_chunks + rc[None, :]) * slots
     comb[..., 7] = (c_last - c_first + 1)[:, None]
     comb[..., 8] = e[:, None]
     comb[..., 9] = 1

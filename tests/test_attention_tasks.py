@@ -97,7 +97,8 @@ def test_long_contexts(seed):
     live = fast[:, 0] >= 0
     assert np.array_equal(live, slow[:, 0] >= 0) and np.array_equal(fast[live], slow[live])
     coverage(fast, mf, starts, counts, group, window)
-    if bucket * 256 >= A.LONG_KEYS and s * bucket * 8 > 800:
+    seen = min(bucket * 256, window + 256) if window else bucket * 256       # keys a token can see
+    if seen >= A.LONG_KEYS and s * -(-seen // 256) * 8 > 800:
         spans = fast[live][:, 5] - fast[live][:, 4]
         assert int(spans.max()) == 512 and mf[3] == 2
     # a portion of a prompt beside them
@@ -143,3 +144,17 @@ def test_tile_builder_equals_the_general_one(seed):
     assert live(fast, mf) == live(slow, ms)
     assert np.array_equal(fast[mf[0]:], slow[ms[0]:])
     coverage(fast, mf, starts, counts, group, window)
+
+
+def test_a_window_far_into_a_context_owns_few_slots():
+    """A decoded token behind a window sees a few chunks wherever it stands: its request owns slots for those,
+    not for every chunk of its context."""
+    starts = np.asarray([100_000, 70_001, 5], dtype=np.int32)
+    counts = np.ones(3, dtype=np.int32)
+    bucket = -(-100_001 // 256)
+    for builder in (True, False):
+        arr, meta = A.build_tasks(starts, counts, 4, 1000, bucket, vectorized=builder, kv_heads=8, max_waves=2)
+        coverage(arr, meta, starts, counts, 4, 1000)
+        assert meta[2] <= 3 * (1000 // 128 + 2) and meta[0] <= meta[2] + 3
+    without, meta_all = A.build_tasks(starts, counts, 4, 0, bucket, kv_heads=8, max_waves=2)
+    assert meta_all[2] > 500

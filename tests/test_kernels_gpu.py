@@ -658,3 +658,33 @@ def test_decode_plans_with_large_groups(nh, nkv, hd, whole, monkeypatch):
         want = plain_attention(q, ks[e], vs[e], s, scale, 0, group).reshape(1, nh * hd)
         err = (out[e:e + 1].double().cpu() - want).abs().max() / want.abs().max()
         assert err < 2e-2, f"request {e} at {s}: {err:.3e}"
+
+
+@pytest.mark.parametrize("window", [64, 200, 1000])
+def test_decode_plans_behind_a_window(window):
+    """Decoded tokens far behind a window, planned as the engine plans them: their requests own slots only for the
+    chunks a window can touch, the first of which is wherever the window begins."""
+    import numpy as np
+    from atoma_infer_amd.kernels import attention_bf16
+    nh, nkv, hd, page = 8, 2, 64, 16
+    starts = [1500, 700, 300, 129, 5]
+    counts = [1] * len(starts)
+    ks, vs, kc, vc, bt = paged_setup([s + 1 for s in starts], nkv, hd, page, torch.bfloat16, seed=window)
+    t = len(starts)
+    g = torch.Generator().manual_seed(4)
+    qkv = (torch.randn(t, (nh + 2 * nkv) * hd, generator=g) * 1.5).bfloat16().to(DEV)
+    out = torch.full((t, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ctx = FakeCtx(starts, counts)
+    bucket = -(-(max(starts) + 1) // 256)
+    arr, meta = attention_bf16.build_tasks(np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32),
+                                           nh // nkv, window, bucket, kv_heads=nkv,
+                                           max_waves=attention_bf16.max_waves_for(hd))
+    assert 0 < meta[2] <= t * (window // 128 + 2)
+    ctx.plans = {attention_bf16.plan_key(nh // nkv, window, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
+    scale = 1.0 / math.sqrt(hd)
+    assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, FakeCache(bt, page), scale, window, nh, nkv, hd)
+    for e, s0 in enumerate(starts):
+        q = qkv[e:e + 1, : nh * hd].cpu().view(1, nh, hd)
+        want = plain_attention(q, ks[e], vs[e], s0, scale, window, nh // nkv).reshape(1, nh * hd)
+        err = (out[e:e + 1].double().cpu() - want).abs().max() / want.abs().max()
+        assert err < 2e-2, f"request {e} at {s0}: {err:.3e}"
