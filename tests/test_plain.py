@@ -121,6 +121,43 @@ def test_llama3_frequency_scaling_branches():
     assert torch.allclose(base, torch.tensor([500000.0 ** (-i / 32) for i in range(0, 32, 2)]), rtol=1e-5)
 
 
+def _one_frequency_cfg(wavelen, **scaling):
+    """A configuration whose second inverse frequency has the given wavelength: head size 4, so the frequencies are
+    1 and theta^(-1/2), and theta = (wavelen / 2 pi)^2."""
+    return {"hidden_size": 4, "num_attention_heads": 1, "rope_theta": (wavelen / (2 * math.pi)) ** 2,
+            "rope_scaling": dict({"rope_type": "llama3"}, **scaling)}
+
+
+def test_llama3_blend_by_hand_and_at_the_edges_of_its_band():
+    """models/src/llama.rs:177-182: smooth = (orig / wavelen - low) / (high - low), and the blended frequency is
+    (1 - smooth) * f / factor + smooth * f.  With orig 64, low 1, high 4, factor 8 a wavelength of 32 gives
+    smooth = (2 - 1) / 3 = 1/3 and f * (2/3 / 8 + 1/3) = f * 5/12 (swapping smooth and 1 - smooth gives f * 17/24).
+    The blend is continuous with its neighbours: towards wavelength orig / high it tends to f, towards orig / low
+    to f / factor (:173-176); a frequency placed just inside either edge must lie within a fraction of a percent of
+    the branch outside it, and a swapped blend is off by the factor there."""
+    sc = dict(original_max_position_embeddings=64, low_freq_factor=1.0, high_freq_factor=4.0, factor=8.0)
+    f = 2 * math.pi / 32
+    inv = P.rope_inv_freq(_one_frequency_cfg(32.0, **sc))
+    assert math.isclose(float(inv[0]), 1.0, rel_tol=1e-6)                  # wavelength 6.28 < 16: untouched
+    assert math.isclose(float(inv[1]), f * 5 / 12, rel_tol=1e-5)
+    assert math.isclose(float(inv[1]), 0.0818123, rel_tol=1e-5)
+    # the two edges, from inside and from outside the band; other constants than above, none of them 1
+    sc = dict(original_max_position_embeddings=96, low_freq_factor=1.5, high_freq_factor=6.0, factor=5.0)
+    high_wl, low_wl = 96 / 6.0, 96 / 1.5
+    for wl, want_ratio in ((high_wl * (1 - 5e-4), 1.0), (high_wl * (1 + 5e-4), 1.0),
+                           (low_wl * (1 - 5e-4), 1 / 5.0), (low_wl * (1 + 5e-4), 1 / 5.0)):
+        inv = P.rope_inv_freq(_one_frequency_cfg(wl, **sc))
+        assert math.isclose(float(inv[1]) / (2 * math.pi / wl), want_ratio, rel_tol=5e-3), (wl, float(inv[1]))
+    # and halfway in terms of orig / wavelen (here 3.75, smooth 1/2) the two branches weigh the same
+    wl = 96 / 3.75
+    inv = P.rope_inv_freq(_one_frequency_cfg(wl, **sc))
+    assert math.isclose(float(inv[1]) / (2 * math.pi / wl), 0.5 * (1 + 1 / 5.0), rel_tol=1e-5)
+    # a quarter of the way (orig / wavelen = 2.625, smooth 1/4): 3/4 of f / factor and 1/4 of f
+    wl = 96 / 2.625
+    inv = P.rope_inv_freq(_one_frequency_cfg(wl, **sc))
+    assert math.isclose(float(inv[1]) / (2 * math.pi / wl), 0.75 / 5.0 + 0.25, rel_tol=1e-5)
+
+
 def test_rms_norm_and_swiglu_reduce_to_library_routines():
     g = torch.Generator().manual_seed(2)
     x, w = torch.randn(4, 96, generator=g), torch.randn(96, generator=g)
