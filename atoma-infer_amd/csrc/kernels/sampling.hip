@@ -496,3 +496,68 @@ extern "C" int atoma_repeat_penalty(float* logits, int ld, const int32_t* rows, 
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
+
+// ---- sampling without a workspace argument and without any allocation (declared in sample_static.h) ----------
+// The weights exp((l - max) / T) of all rows, which atoma_sample keeps in the caller's workspace, live here in an
+// array of the code object.  Every device that loads this library holds its own copy at its own address until the
+// process ends; host code may not use the array's name as an address, so the address is asked for once per device
+// and kept.  All calls on one device share the array: two that overlap in time (two streams, two threads) race.
+// Nothing in it has to start at zero: a sampled row writes all of its weights before it reads any of them.
+#include "sample_static.h"
+#include <mutex>
+
+static __device__ __align__(256) float scratch[ATOMA_SAMPLE_STATIC_MAX_FLOATS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+float* scratch_of_device[kMaxDevices] = {};       // device address of `scratch` on each device, once known
+
+// the address of the current device's copy of `scratch`; a HIP error code (positive) through rc otherwise
+float* scratch_address(int& rc) {
+  rc = 0;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    rc = (int)e;
+    return nullptr;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    rc = ATOMA_ERR_SHAPE;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(scratch_mutex);
+  if (scratch_of_device[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      rc = e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+      return nullptr;
+    }
+    scratch_of_device[dev] = static_cast<float*>(p);
+  }
+  return scratch_of_device[dev];
+}
+}  // namespace
+
+extern "C" int atoma_sample_static_init(void) {
+  int rc;
+  scratch_address(rc);
+  return rc;
+}
+
+extern "C" int atoma_sample_static(const float* logits, int ld, int n_rows, int vocab, const float* temperature,
+                                   const int32_t* top_k, const float* top_p, const float* uniform,
+                                   int32_t* out_token, float* out_logit, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (vocab <= 0 || ld < vocab) return ATOMA_ERR_SHAPE;
+  if ((unsigned long long)n_rows * (unsigned long long)vocab > (unsigned long long)ATOMA_SAMPLE_STATIC_MAX_FLOATS)
+    return ATOMA_ERR_TOO_LARGE;
+  int rc;
+  float* weights = scratch_address(rc);
+  if (weights == nullptr) return rc;
+  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(kSampThreads), 0, stream, logits, ld, vocab, temperature, top_k,
+                     top_p, uniform, weights, out_token, out_logit);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
