@@ -43,7 +43,7 @@ def _host():
         lib.cm_destroy.restype = None
         for name in ("cm_add_request", "cm_free", "cm_state_slot"):
             getattr(lib, name).argtypes = [ctypes.c_void_p, ctypes.c_int64]
-        for name in ("cm_can_reserve", "cm_reserve", "cm_release_behind"):
+        for name in ("cm_can_reserve", "cm_reserve", "cm_release_behind", "cm_can_admit"):
             getattr(lib, name).argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64]
         lib.cm_fits_at_all.argtypes = [ctypes.c_void_p, ctypes.c_int64]
         lib.cm_reserved_len.argtypes = [ctypes.c_void_p, ctypes.c_int64]
@@ -118,6 +118,11 @@ class CacheManager:
     def fits_at_all(self, length: int) -> bool:
         """Whether a request of ``length`` tokens could be held with every page free."""
         return bool(self._lib.cm_fits_at_all(self._h, length))
+
+    def can_admit(self, total: int, first: int) -> bool:
+        """Whether a new request of ``total`` tokens may start with a portion of ``first``: pages for the portion
+        and, in groups with a window, room for the window (and one page) of the newcomer and of everyone held."""
+        return bool(self._lib.cm_can_admit(self._h, total, first))
 
     def reserve(self, request: int, length: int) -> None:
         rc = self._lib.cm_reserve(self._h, request, length)

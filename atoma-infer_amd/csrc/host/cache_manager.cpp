@@ -51,6 +51,9 @@ int64_t pages_needed(const Manager& m, const Request* r, size_t gi, int64_t new_
   return want > have ? want - have : 0;
 }
 
+// pages of request r in group gi that are still held (table entries that a window has not released)
+int64_t live_pages(const Request& r, size_t gi) { return (int64_t)r.tables[gi].size() - r.first_live[gi]; }
+
 }  // namespace
 
 extern "C" {
@@ -118,6 +121,37 @@ int cm_fits_at_all(void* h, int64_t new_len) {
     if (need > g.num_pages) return 0;
   }
   return 1;
+}
+
+// 1 if a new request of total_len tokens may start with a first portion of first_len tokens.  Beside the pages of
+// that portion, a group with a window must have room for what the newcomer and every request already held will
+// need once they have moved on: the window and the page that the next token opens, each.  Without that, a request
+// admitted into pages that the others are about to ask for is preempted again at once, step after step.
+int cm_can_admit(void* h, int64_t total_len, int64_t first_len) {
+  Manager* m = static_cast<Manager*>(h);
+  if (m->free_slots.empty() || first_len > total_len) return 0;
+  for (size_t gi = 0; gi < m->groups.size(); ++gi) {
+    const Group& g = m->groups[gi];
+    int64_t need = blocks_for(g, first_len);
+    if (g.window > 0) {
+      const int64_t steady = blocks_for(g, g.window) + 1;
+      const int64_t own = blocks_for(g, total_len) < steady ? blocks_for(g, total_len) : steady;
+      if (own > need) need = own;
+      for (const auto& kv : m->requests) {
+        const int64_t lack = steady - live_pages(kv.second, gi);
+        if (lack > 0) need += lack;
+      }
+    }
+    if (need > (int64_t)g.free_list.size()) return 0;
+  }
+  return 1;
+}
+
+// 1 if some group keeps a window only.
+int cm_has_window(void* h) {
+  for (const Group& g : static_cast<Manager*>(h)->groups)
+    if (g.window > 0) return 1;
+  return 0;
 }
 
 // Makes every group cover positions [0, new_len).  All groups or none.

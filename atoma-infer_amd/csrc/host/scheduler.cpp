@@ -10,7 +10,10 @@
 // Pages are reserved for what a step adds.  When they run out for a running request, the running request that
 // arrived last is preempted by recomputation (scheduler.rs:650-690, 1778-1896): what it holds goes back and it
 // returns to the front of the waiting queue.  A request that runs alone tries shorter portions, and is finished
-// ("capped") when not even one token finds a page.  A waiting request longer than the model length, or than the whole pool, is dropped ("ignored").
+// ("capped") when not even one token finds a page.  A waiting request longer than the model length, or than the whole
+// pool, is dropped ("ignored").  With a window of keys (pages come back as a request moves on) portions are
+// shortened before anything is preempted, the first portion of a request that finds the pool idle is shortened until
+// it fits, and a request is admitted only if the window of every request already there still finds its pages.
 //
 // The scheduler keeps four counters per request (tokens held, tokens computed, tokens sampled, frozen); whoever
 // runs the steps reports them before each plan.  It calls the cache manager of the same library directly and lists
@@ -48,6 +51,7 @@ struct Entry {
 struct Sched {
   void* cm = nullptr;
   int max_tokens = 0, max_seqs = 0, max_model_len = 0, chunked = 1, max_chunk = 0;
+  bool windowed = false;  // some cache group keeps a window of keys only
   double delay_factor = 0.0;
   std::deque<int64_t> waiting;
   std::vector<int64_t> running;
@@ -137,7 +141,8 @@ struct Sched {
       Req& r = reqs[order[i]];
       if (!r.running) continue;  // preempted while serving an earlier request
       if ((int)entries.size() >= max_seqs) break;
-      int n = chunk(r, max_tokens - used_tokens());
+      const int n_whole = chunk(r, max_tokens - used_tokens());
+      int n = n_whole;
       if (n <= 0) continue;
       while (!cm_can_reserve(cm, r.uid, r.computed + n)) {
         // the latest arrival that is not just waiting for its last token (that one frees its pages soon)
@@ -147,13 +152,16 @@ struct Sched {
             victim = &reqs[*it];
             break;
           }
-        if (victim == &r && running.size() == 1) {
-          // nothing else to give back: a shorter portion may still find its pages (with a window of keys, pages
-          // come back as the request moves on); if one token finds none, the pool cannot hold this request
-          if (n > 1 && chunked) {
-            n /= 2;
-            continue;
-          }
+        const bool alone = victim == &r && running.size() == 1;
+        // A shorter portion may still find its pages: when nothing else could give any back, and, with a window
+        // of keys, always (pages come back as the request moves on, so a portion too long for what is free now
+        // is no reason to throw away what another request has computed).
+        if (n > 1 && chunked && (alone || windowed)) {
+          n /= 2;
+          continue;
+        }
+        if (alone) {
+          // not even one token finds a page: the pool cannot hold this request
           drop_running(r.uid);
           release(r.uid);
           r.running = false;
@@ -162,6 +170,7 @@ struct Sched {
         }
         preempt(*victim);
         if (victim == &r) break;
+        n = n_whole;      // what came back may hold the whole portion
       }
       if (!r.running) continue;
       if (cm_reserve(cm, r.uid, r.computed + n) != 0) return -1;
@@ -178,9 +187,18 @@ struct Sched {
           continue;
         }
         if ((int)entries.size() >= max_seqs || (int)running.size() >= max_seqs) break;
-        const int n = chunk(r, max_tokens - used_tokens());
-        if (n <= 0) break;
-        if (cm_num_free_slots(cm) == 0 || !cm_can_reserve(cm, -1, n)) break;  // later
+        int n = chunk(r, max_tokens - used_tokens());
+        if (n <= 0 || cm_num_free_slots(cm) == 0) break;
+        // If nothing holds pages, waiting frees none: only a shorter first portion helps (a prompt longer than
+        // the pool gets in through a window of keys); when one token finds no page the request can never run.
+        const bool pool_is_idle = cm_num_requests(cm) == 0;
+        while (n > 1 && chunked && pool_is_idle && !cm_can_admit(cm, r.length, n)) n /= 2;
+        if (!cm_can_admit(cm, r.length, n)) {
+          if (!pool_is_idle) break;  // later
+          waiting.pop_front();
+          ignored.push_back(r.uid);
+          continue;
+        }
         waiting.pop_front();
         if (cm_add_request(cm, r.uid) < 0) return -1;
         if (cm_reserve(cm, r.uid, n) != 0) return -1;
@@ -218,6 +236,7 @@ void* sc_create(void* cache_manager, int max_tokens, int max_seqs, int max_model
   s->chunked = chunked;
   s->max_chunk = max_chunk;
   s->delay_factor = delay_factor;
+  s->windowed = cm_has_window(cache_manager) != 0;
   return s;
 }
 

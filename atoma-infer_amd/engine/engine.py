@@ -167,6 +167,10 @@ class LlmEngine:
         launched = None
         if not plan.empty:
             launched = self._launch(plan)
+        elif self._in_flight is None and not (finished or plan.preempted) and self.scheduler.has_unfinished():
+            # nothing runs, nothing is on its way, nothing left the queue: the next plan would be the same
+            raise RuntimeError(f"the scheduler plans nothing although {self.scheduler.num_unfinished()} request(s) "
+                               f"wait: its limits admit none of them")
         if self._in_flight is not None:
             finished += self._resolve(self._in_flight)
         self._in_flight = launched

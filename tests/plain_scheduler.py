@@ -1,7 +1,7 @@
 """The scheduler's policy written out plainly, to compare the native scheduler's decisions with.
 
 It shares nothing with the product: requests are ``PlainRequest`` objects, statuses are strings, and pages are
-counted by ``PlainPages`` (one group of pages, no window).  The policy is the reference's chunked one
+counted by ``PlainPages`` (one group of pages, with or without a window of keys).  The policy is the reference's chunked one
 (backends/vllm/src/scheduler.rs:1257-1379 with the budget of :40-149, admissions :897-1016, recompute-preemption
 :650-690 and :1778-1896, the optional delay :2077-2097, first come first served policy.rs:56-61):
 
@@ -11,7 +11,10 @@ counted by ``PlainPages`` (one group of pages, no window).  The policy is the re
 
 When pages run out for a running request, the running request that arrived last (and is not frozen) is preempted:
 its pages go back, it returns to the front of the waiting queue with nothing computed.  A request that runs alone
-tries portions half as long, and is capped when not even one token finds a page.  A waiting request longer than the model length or the pool is ignored.
+tries portions half as long, and is capped when not even one token finds a page.  A waiting request longer than
+the model length or the pool is ignored.  With a window of keys portions are shortened before anything is
+preempted, a first portion that finds the pool idle is shortened until it fits, and a newcomer must leave room for
+the window (and one page) of everyone already there.
 """
 from collections import deque
 
@@ -44,17 +47,22 @@ class PlainRequest:
 
 
 class PlainPages:
-    """How many pages each request holds; pages are not told apart."""
+    """How many pages each request holds; pages are not told apart.  With ``window`` W a request needs the pages
+    that hold its last W tokens only: ``release_behind`` gives back those wholly below ``computed - W + 1``."""
 
-    def __init__(self, page_size, num_pages, slots):
-        self.page_size, self.num_pages, self.slots = page_size, num_pages, slots
-        self.held = {}
+    def __init__(self, page_size, num_pages, slots, window=0):
+        self.page_size, self.num_pages, self.slots, self.window = page_size, num_pages, slots, window
+        self.held = {}          # uid -> pages ever taken (the length of its table)
+        self.released = {}      # uid -> how many of them went back behind the window
 
     def _pages(self, length):
         return -(-length // self.page_size)
 
+    def _live(self, uid):
+        return self.held[uid] - self.released[uid]
+
     def free_pages(self):
-        return self.num_pages - sum(self.held.values())
+        return self.num_pages - sum(self._live(u) for u in self.held)
 
     def has(self, uid):
         return uid in self.held
@@ -62,24 +70,49 @@ class PlainPages:
     def num_free_slots(self):
         return self.slots - len(self.held)
 
+    def idle(self):
+        return not self.held
+
     def fits_at_all(self, length):
-        return self._pages(length) <= self.num_pages
+        need = self._pages(length)
+        if self.window:
+            need = min(need, self._pages(self.window) + 1)
+        return need <= self.num_pages
 
     def can_reserve(self, uid, length):
         if uid not in self.held and self.num_free_slots() == 0:
             return False
         return max(0, self._pages(length) - self.held.get(uid, 0)) <= self.free_pages()
 
+    def can_admit(self, total, first):
+        """A newcomer's first portion, and with a window also what it and everyone already there will need once
+        they have moved on: the window and one page each."""
+        if self.num_free_slots() == 0:
+            return False
+        need = self._pages(first)
+        if self.window:
+            steady = self._pages(self.window) + 1
+            need = max(need, min(self._pages(total), steady))
+            need += sum(max(0, steady - self._live(u)) for u in self.held)
+        return need <= self.free_pages()
+
     def add(self, uid):
         assert uid not in self.held and self.num_free_slots() > 0
         self.held[uid] = 0
+        self.released[uid] = 0
 
     def reserve(self, uid, length):
         assert self.can_reserve(uid, length)
         self.held[uid] = max(self.held[uid], self._pages(length))
 
+    def release_behind(self, uid, computed):
+        if self.window and computed - self.window + 1 > 0:
+            dead = min((computed - self.window + 1) // self.page_size, self.held[uid])
+            self.released[uid] = max(self.released[uid], dead)
+
     def free(self, uid):
         del self.held[uid]
+        del self.released[uid]
 
 
 class PlainOutput:
@@ -155,15 +188,16 @@ class PlainScheduler:
                 continue      # preempted for an earlier request of this step
             if len(out.entries) >= lim.max_requests:
                 break
-            n = self._portion(r, lim.max_tokens - used())
+            n = whole = self._portion(r, lim.max_tokens - used())
             if n <= 0:
                 continue
             while not self.pages.can_reserve(r.uid, r.num_computed + n):
                 victim = next((v for v in reversed(self.running) if not v.frozen), r)
-                if victim is r and len(self.running) == 1:
-                    if n > 1 and lim.cut:
-                        n //= 2           # alone: a shorter portion may still find its pages
-                        continue
+                alone = victim is r and len(self.running) == 1
+                if n > 1 and lim.cut and (alone or self.pages.window):
+                    n //= 2           # a shorter portion may still find its pages
+                    continue
+                if alone:
                     self.running.remove(r)
                     self._release(r)
                     r.status = "capped"
@@ -172,6 +206,7 @@ class PlainScheduler:
                 self._preempt(victim, out)
                 if victim is r:
                     break
+                n = whole
             if r.status != "running":
                 continue
             self.pages.reserve(r.uid, r.num_computed + n)
@@ -188,10 +223,18 @@ class PlainScheduler:
                 if len(out.entries) >= lim.max_requests or len(self.running) >= lim.max_requests:
                     break
                 n = self._portion(r, lim.max_tokens - used())
-                if n <= 0:
+                if n <= 0 or self.pages.num_free_slots() == 0:
                     break
-                if self.pages.num_free_slots() == 0 or not self.pages.can_reserve(-1, n):
-                    break
+                idle = self.pages.idle()
+                while n > 1 and lim.cut and idle and not self.pages.can_admit(r.length, n):
+                    n //= 2           # nothing holds pages: only a shorter first portion helps
+                if not self.pages.can_admit(r.length, n):
+                    if not idle:
+                        break
+                    self.waiting.popleft()
+                    r.status = "ignored"
+                    out.ignored.append(r)
+                    continue
                 self.waiting.popleft()
                 self.pages.add(r.uid)
                 self.pages.reserve(r.uid, n)

@@ -199,3 +199,25 @@ def test_tile_layout_is_a_permutation_and_serves_the_mfma_lanes(page, head):
             for hg in (0, 1):
                 slots = [int(vi[d, hg * 4 + i]) for i in range(4)] + [int(vi[d, 8 + hg * 4 + i]) for i in range(4)]
                 assert slots == list(range(slots[0], slots[0] + 8)) and slots[0] % 8 == 0
+
+
+def test_admission_with_a_window_counts_what_everyone_will_need():
+    """Without a window, admission asks for the first portion's pages only.  With one, also for the window and a
+    page of the newcomer and for what every request already held still lacks of its own."""
+    m = CacheManager([GroupGeometry(4, 8)], 4)
+    assert m.can_admit(100, 32) and not m.can_admit(100, 33)
+    w = CacheManager([GroupGeometry(4, 8, window=10)], 4)           # a request in full swing needs 3 + 1 pages
+    assert w.can_admit(100, 32) and not w.can_admit(100, 33)         # the first portion, all of it, at once
+    w.add(1)
+    w.reserve(1, 4)                                                  # holds 1 page, lacks 3 of its 4
+    assert w.can_admit(100, 4)                                       # 4 (own) + 3 (lacking) <= 7 free
+    w.add(2)
+    w.reserve(2, 4)                                                  # 6 free; those there lack 3 each
+    assert not w.can_admit(100, 4)                                   # 4 + 6 > 6
+    assert not w.can_admit(4, 4)                                     # even a one-page request: 1 + 6 > 6
+    w.reserve(1, 16)
+    w.reserve(2, 12)                                                 # 1 free; they lack 0 and 1
+    assert not w.can_admit(4, 4)
+    w.free(2)
+    assert w.can_admit(100, 4) and w.can_admit(100, 16) and not w.can_admit(100, 17)
+    w.check()

@@ -221,6 +221,62 @@ def test_a_window_of_keys_lets_long_requests_into_a_small_pool():
     assert len(a.output_ids) == 4 and cache.num_free_pages() == 5
 
 
+def _run_windowed(cache, s, reqs, limit=400):
+    steps = preempted = 0
+    while s.has_unfinished():
+        out = s.schedule()
+        assert out.entries or out.ignored or out.capped or out.preempted, "an empty plan: nothing would ever change"
+        preempted += len(out.preempted)
+        for e in out.entries:
+            cache.release_behind(e.request.uid, e.request.num_computed + e.num_tokens)    # as the runner does
+        run_step(s, out)
+        cache.check()
+        steps += 1
+        assert steps < limit
+    return steps, preempted
+
+
+def test_a_first_portion_longer_than_the_pool_is_shortened_not_waited_for():
+    """A prompt of 100 tokens, a token budget of 64, a pool of 20 tokens that keeps a window of 10: the first
+    portion must shrink to what the idle pool holds (waiting frees nothing), and the request runs to its end."""
+    cache = CacheManager([GroupGeometry(4, 5, window=10)], 4)
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=64, max_num_sequences=4, max_model_len=2000), cache)
+    a = make_request(0, 100, max_new=4)
+    s.add(a)
+    out = s.schedule()
+    assert [(e.request.uid, e.num_tokens) for e in out.entries] == [(0, 16)]      # 64 -> 32 -> 16 tokens = 4 pages
+    for e in out.entries:
+        cache.release_behind(e.request.uid, e.num_tokens)
+    run_step(s, out)
+    _run_windowed(cache, s, [a])
+    assert len(a.output_ids) == 4 and cache.num_free_pages() == 5 and a.status.finished
+
+
+def test_an_uncut_prompt_longer_than_a_windowed_pool_is_ignored():
+    cache = CacheManager([GroupGeometry(4, 5, window=10)], 4)
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=2000, max_num_sequences=4, max_model_len=2000,
+                                  enable_chunked_prefill=False), cache)
+    a, b = make_request(0, 100), make_request(1, 12, max_new=3)
+    s.add(a)
+    s.add(b)
+    out = s.schedule()
+    assert [r.uid for r in out.ignored] == [0] and [e.request.uid for e in out.entries] == [1]
+
+
+def test_admission_into_a_windowed_pool_leaves_room_for_those_already_there():
+    """Two long requests and a pool that holds the window (and one page) of two requests but not of three: the
+    third waits until one of the others is done instead of being admitted and preempted over and over."""
+    cache = CacheManager([GroupGeometry(4, 9, window=10)], 4)         # steady need: 3 + 1 pages a request
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=8, max_num_sequences=4, max_model_len=2000), cache)
+    reqs = [make_request(i, 40, max_new=30) for i in range(3)]
+    for r in reqs:
+        s.add(r)
+    out = s.schedule()
+    assert [e.request.uid for e in out.entries] == [0]                 # 8 tokens of budget: one portion
+    steps, preempted = _run_windowed(cache, s, reqs)
+    assert preempted == 0 and all(len(r.output_ids) == 30 for r in reqs) and cache.num_free_pages() == 9
+
+
 def test_abort_frees_and_unchunked_prompts_wait_for_room():
     s, cache = make_scheduler(pages=128, page=4, max_num_batched_tokens=256, max_model_len=256,
                               enable_chunked_prefill=False)
@@ -298,12 +354,13 @@ def _random_world(seed):
         lim.max_tokens = max(lim.max_tokens, lim.max_model_len)      # the configuration demands it
     lim.max_tokens = max(lim.max_tokens, lim.max_requests)
     now = [0.0]
-    cache = CacheManager([GroupGeometry(page, pages)], slots)
+    window = rng.choice([0, 0, 5, 12, 33])
+    cache = CacheManager([GroupGeometry(page, pages, window=window or None)], slots)
     native = Scheduler(SchedulerConfig(max_num_batched_tokens=lim.max_tokens, max_num_sequences=lim.max_requests,
                                        max_model_len=lim.max_model_len, enable_chunked_prefill=lim.cut,
                                        max_prefill_chunk=lim.max_portion, delay_factor=lim.delay_factor),
                        cache, clock=lambda: now[0])
-    plain_pages = PlainPages(page, pages, slots)
+    plain_pages = PlainPages(page, pages, slots, window)
     plain = PlainScheduler(lim, plain_pages)
     mine, theirs, uid = {}, {}, 0
     pending_mine, pending_theirs = [], []
@@ -358,12 +415,14 @@ def _random_world(seed):
         for e in out_a.entries:
             a = e.request
             a.num_computed += e.num_tokens
+            cache.release_behind(a.uid, a.num_computed)          # as the runner does after a step
             if e.do_sample:
                 a.pending += 1
                 a.frozen = a.num_sampled >= a.plan.max_new_tokens or a.length > lim.max_model_len
                 pending_mine.append(a)
         for b, n, _, sample in out_b.entries:
             b.num_computed += n
+            plain_pages.release_behind(b.uid, b.num_computed)
             if sample:
                 b.pending += 1
                 b.frozen = b.num_sampled >= b.max_new or b.length > lim.max_model_len
