@@ -127,12 +127,16 @@ _MM_OUT_DTYPE = _probe_mm_out_dtype()
 
 
 def try_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None,
-               ) -> Optional[torch.Tensor]:
-    """x [M, K] @ w [N, K]^T if a fast kernel takes the shape, else None (the caller falls back to float32 FMAs)."""
+               library_only: bool = False) -> Optional[torch.Tensor]:
+    """x [M, K] @ w [N, K]^T if a fast kernel takes the shape, else None (the caller falls back to float32 FMAs).
+    ``library_only``: None also where the library would not be the choice."""
     m, n = x.shape[0], w.shape[0]
     k = x.shape[1]
     ok = skinny_ok(x, w)
-    if not (ok and _library_wins(m, n, k, out_dtype)) and ok and (m <= SKINNY_MAX_M or out_dtype is torch.float32):
+    if library_only:
+        if not (_MM_OUT_DTYPE and out_dtype is torch.float32 and m > LIBRARY_MIN_M_WIDE):
+            return None
+    elif not (ok and _library_wins(m, n, k, out_dtype)) and ok and (m <= SKINNY_MAX_M or out_dtype is torch.float32):
         if out is None:
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
         for lo in range(0, m, SKINNY_MAX_M):

@@ -40,4 +40,9 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         y = gemm_bf16.linear_planes(x, w)
         if y is not None:
             return y
+        # many rows: the library's product, its float32 sums handed to the residual stream unrounded, as the
+        # planes of the few-row kernel are
+        y = gemm_bf16.try_linear(x, w, torch.float32, library_only=True)
+        if y is not None:
+            return y
     return linear(x, w)

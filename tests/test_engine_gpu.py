@@ -307,6 +307,86 @@ def test_layers_of_serving_size_in_mixed_steps(tmp_path, cfg):
     _plain_cache.clear()
 
 
+def _four_schedules(requests, rng):
+    """For requests r0..: each alone and whole; most of r0 in one step and its last 32 tokens one by one; r0 in portions
+    of changing size down to two tokens; all mixed, up to four live, portions beside decoded tokens."""
+    names = list(requests)
+    whole = [([(r, len(requests[r]))], [r]) for r in names]
+    n0 = len(requests[names[0]])
+    last32 = [([(names[0], n0 - 32)], [])] + [([(names[0], 1)], [])] * 31 + [([(names[0], 1)], [names[0]])]
+    sizes, left, cycle, i = [], n0, [17, 2, 31, 3, 16, 2, 5, 33, 1, 4], 0
+    while left:
+        sizes.append(min(cycle[i % len(cycle)], left))
+        left -= sizes[-1]
+        i += 1
+    portions = [([(names[0], k)], [names[0]] if j == len(sizes) - 1 else []) for j, k in enumerate(sizes)]
+    mixed, waiting, live, done = [], list(names), [], {r: 0 for r in names}
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            left = len(requests[r]) - done[r]
+            n = 1 if left <= 6 else min(rng.choice([2, 3, 5, 8, 13, 24]), left - 6)
+            if rng.random() < 0.15 and len(live) > 1:
+                continue
+            entries.append((r, n))
+            done[r] += n
+            if done[r] == len(requests[r]):
+                end.append(r)
+        if entries:
+            rng.shuffle(entries)
+            mixed.append((entries, end))
+            live = [r for r in live if r not in end]
+    return {"whole": whole, "last 32 one by one": last32, "portions": portions, "mixed": mixed}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_checkpoint_stored_in_float32(tmp_path, dtype):
+    """Tensors stored in 32 bits stay float32 on the device whatever the activation dtype is: the four schedules at
+    Tiny B from such a file, against the plain model on the same float32 numbers."""
+    name = "B"
+    model_dir = make_model_dir(str(tmp_path / "m"), TINY[name], seed=17, dtype="float32", norm_jitter=NORM_JITTER[name])
+    vocab = TINY[name]["vocab_size"]
+    lens = [120, 1, 77, 90, 45, 18]
+    requests = {f"r{i}": random_tokens(n, vocab, 500 + i) for i, n in enumerate(lens)}
+    need = sum(sorted(-(-n // 16) for n in lens)[-4:])
+    for kind, steps in _four_schedules(requests, random.Random(2)).items():
+        runner = make_runner(model_dir, dtype, 16, need, slots=4)
+        stored = {w.dtype for _, blk in runner.model.spec.layers for w in (blk.mixer.w_qkv, blk.mixer.w_o)}
+        assert stored == {torch.float32}, stored
+        got = run_schedule(runner, requests, steps)
+        check_against_plain(model_dir, requests, got, dtype)
+        assert runner.manager.num_free_pages(0) == need, kind
+    _plain_cache.clear()
+
+
+def test_all_sixteen_layers_of_llama_1b_size(tmp_path):
+    """The whole Llama 3.2 1B shape (16 layers, the full vocabulary, tied head, llama3 scaling with its own
+    constants) against the plain model (models/src/llama.rs:456-478): a prompt in uneven portions, three live
+    requests, a fourth that takes over the pages of the first, float32 and bfloat16."""
+    cfg = dict(LLAMA_1B_LAYERS, num_hidden_layers=16)
+    model_dir = make_model_dir(str(tmp_path / "m"), cfg, seed=9, dtype="bfloat16", norm_jitter=0.1)
+    vocab = cfg["vocab_size"]
+    requests = {"a": random_tokens(150, vocab, 1), "b": random_tokens(72, vocab, 2), "c": random_tokens(33, vocab, 3),
+                "d": random_tokens(90, vocab, 4)}
+    steps = [([("a", 93)], []), ([("a", 37), ("b", 50)], []), ([("a", 2), ("b", 1), ("c", 30)], [])]
+    steps += [([("a", 1), ("b", 1), ("c", 1)], [])] * 3
+    steps += [([("a", 15), ("b", 16)], ["a", "c"])]
+    steps += [([("d", 67), ("b", 1)], []), ([("d", 2)], []), ([("d", 21), ("b", 1)], ["b", "d"])]
+    pages = 10 + 5 + 3 + 1             # a, b, c and one to spare: d (6 pages) must take what a gave back
+    for dtype in DTYPES:
+        runner = make_runner(model_dir, dtype, 16, pages, slots=3)
+        got = run_schedule(runner, requests, steps)
+        assert len(got) == sum(len(v) for v in requests.values())
+        worst = check_against_plain(model_dir, requests, got, dtype)
+        print(f"16 layers, {dtype}: worst error {worst:.3e}", flush=True)
+        assert runner.manager.num_free_pages() == pages
+        del runner
+        torch.cuda.empty_cache()
+    _plain_cache.clear()
+
+
 def test_decode_graphs_with_library_products_inside(tmp_path):
     """With more than 64 decoding requests the linears of a step are the library's, inside the recorded graph.
     Every replay is compared with the same step run eagerly, with eager work and a synchronisation between

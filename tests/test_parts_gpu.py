@@ -740,8 +740,9 @@ def test_another_norm_and_another_block_arrangement(tmp_path, dtype):
 
 
 def test_toy_state_survives_preemption(toy_dir):
-    """Three requests in a pool that holds two: one is preempted and computed again later.  Its mixer state must
-    start from zero then (the slot it gets may have been another request's), or its tokens change."""
+    """Three requests in a pool that holds less than two at their full length (the window group admits only what
+    it can carry, so the squeeze must come from growth): one is preempted and computed again later.  Its mixer state
+    must start from zero then (the slot it gets may have been another request's), or its tokens change."""
     from atoma_infer_amd.config import CacheConfig, SchedulerConfig
     from atoma_infer_amd.engine.engine import LlmEngine
     from atoma_infer_amd.sampling import GenerateParameters
@@ -753,7 +754,7 @@ def test_toy_state_survives_preemption(toy_dir):
         for _ in range(20):
             seq.append(int(torch.argmax(toy_plain_forward(seq, w, TOY)[-1])))
         want.append(seq[len(p):])
-    eng = LlmEngine(toy_dir, "float32", cache=CacheConfig(block_size=16, num_gpu_blocks_override=7),
+    eng = LlmEngine(toy_dir, "float32", cache=CacheConfig(block_size=16, num_gpu_blocks_override=5),
                     scheduler=SchedulerConfig(max_num_batched_tokens=32, max_num_sequences=3, max_model_len=64))
     outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=20, ignore_eos_token=True))
     assert eng.stats["preemptions"] > 0

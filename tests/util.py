@@ -92,3 +92,20 @@ TOL_BF16 = 2e-2
 def random_tokens(n: int, vocab: int, seed: int) -> List[int]:
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def check_greedy_tokens(prompt: List[int], tokens: List[int], chosen_logits: List[float], w, cfg, tol: float) -> None:
+    """Greedy tokens of an engine whose logits carry rounding noise, against the plain model run on the sequence the
+    engine produced: at every step the logit the engine reports for its token must be the plain one within ``tol``
+    of the row's largest magnitude, and the token must be the plain argmax up to twice that (a flipped argmax
+    between two nearly equal logits is rounding; a token from a wrong row of logits is not)."""
+    import plain_llama
+    rows = plain_llama.forward(list(prompt) + list(tokens), w, cfg)[len(prompt) - 1:-1]
+    assert len(tokens) == len(chosen_logits) == rows.shape[0]
+    for step, (tok, lg) in enumerate(zip(tokens, chosen_logits)):
+        row = rows[step]
+        scale = float(row.abs().max())
+        assert abs(float(row[tok]) - lg) <= tol * scale, \
+            f"step {step}: the engine's logit {lg:.5f} of token {tok} is not the plain model's {float(row[tok]):.5f}"
+        assert float(row.max() - row[tok]) <= 2 * tol * scale, \
+            f"step {step}: token {tok} is no argmax of the plain model ({float(row[tok]):.5f} < {float(row.max()):.5f})"
