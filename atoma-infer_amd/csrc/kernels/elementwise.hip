@@ -6,6 +6,27 @@
 
 using namespace atoma;
 
+// four neighbouring values at a time
+struct f4 { float v[4]; };
+__device__ __forceinline__ f4 load4(const float* p) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  return f4{{t.x, t.y, t.z, t.w}};
+}
+__device__ __forceinline__ f4 load4(const bf16_t* p) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  return f4{{bf16_bits_to_f32((uint16_t)(t.x & 0xffff)), bf16_bits_to_f32((uint16_t)(t.x >> 16)),
+             bf16_bits_to_f32((uint16_t)(t.y & 0xffff)), bf16_bits_to_f32((uint16_t)(t.y >> 16))}};
+}
+__device__ __forceinline__ void store4(float* p, const f4& a) {
+  *reinterpret_cast<float4*>(p) = make_float4(a.v[0], a.v[1], a.v[2], a.v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const f4& a) {
+  uint2 t;
+  t.x = (uint32_t)f32_to_bf16_bits(a.v[0]) | ((uint32_t)f32_to_bf16_bits(a.v[1]) << 16);
+  t.y = (uint32_t)f32_to_bf16_bits(a.v[2]) | ((uint32_t)f32_to_bf16_bits(a.v[3]) << 16);
+  *reinterpret_cast<uint2*>(p) = t;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Embedding gather into the float32 residual stream: out[t, :] = table[token[t], :].
 // Tokens that the host has not seen (fed from the sampler on the device) are checked here: an id outside the table
@@ -36,6 +57,112 @@ extern "C" int atoma_embed(const int32_t* tokens, const void* table, int table_d
                        vocab);
   else
     return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A norm begun by the kernel that makes the residual row and finished by the product that reads it (decode steps of
+// at most 16 rows; the products are in gemm_bf16.hip).  "Begun" is: u = residual * norm weight, as bfloat16, and the
+// row's sum of squares in shares ss [parts][16]; "finished" is the division by sqrt(sum / width + eps).
+
+// Embedding gather with the first norm begun: resid [T][width] float32, u [T][width] bfloat16, ss [1][16].
+// One block of 256 threads per row, 16 blocks: those beyond T only clear their share.  Four columns a thread at a
+// time where the row allows 8- and 16-byte accesses (VEC), one otherwise.
+template <typename TW, typename TG, bool VEC>
+__global__ void __launch_bounds__(256)
+embed_begin_norm_kernel(const int32_t* __restrict__ tokens, const TW* __restrict__ table, float* __restrict__ resid,
+                        const TG* __restrict__ gamma, bf16_t* __restrict__ u, float* __restrict__ ss, int n_tokens,
+                        int width, int vocab) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  if (t >= n_tokens) {
+    if (threadIdx.x == 0) ss[t] = 0.f;
+    return;
+  }
+  const int token = tokens[t];
+  const bool ok = token >= 0 && token < vocab;
+  const size_t dst = (size_t)t * width, src = (size_t)(ok ? token : 0) * width;
+  const float nan = __int_as_float(0x7fc00000);
+  float sq = 0.f;
+  if (VEC) {
+    for (int i = 4 * threadIdx.x; i < width; i += 1024) {
+      f4 v = load4(table + src + i);
+      const f4 g = load4(gamma + i);
+      f4 o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (!ok) v.v[j] = nan;
+        o.v[j] = v.v[j] * g.v[j];
+        sq += v.v[j] * v.v[j];
+      }
+      store4(resid + dst + i, v);
+      store4(u + dst + i, o);
+    }
+  } else {
+    for (int i = threadIdx.x; i < width; i += 256) {
+      const float v = ok ? to_f32(table[src + i]) : nan;
+      resid[dst + i] = v;
+      u[dst + i] = from_f32<bf16_t>(v * to_f32(gamma[i]));
+      sq += v * v;
+    }
+  }
+  sq = block_sum<4>(sq, scratch);
+  if (threadIdx.x == 0) ss[t] = sq;
+}
+
+extern "C" int atoma_embed_begin_norm(const int32_t* tokens, const void* table, int table_dtype, float* resid,
+                                      const void* gamma, int gamma_dtype, void* u, float* ss, int n_tokens, int width,
+                                      int vocab, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (n_tokens > 16) return ATOMA_ERR_SHAPE;
+  const bool vec = width % 4 == 0 && (((uintptr_t)table | (uintptr_t)gamma | (uintptr_t)resid | (uintptr_t)u) & 15) == 0;
+#define ATOMA_EBN(TW, TG)                                                                                           \
+  do {                                                                                                              \
+    if (vec)                                                                                                        \
+      hipLaunchKernelGGL((embed_begin_norm_kernel<TW, TG, true>), dim3(16), dim3(256), 0, stream, tokens,           \
+                         (const TW*)table, resid, (const TG*)gamma, (bf16_t*)u, ss, n_tokens, width, vocab);        \
+    else                                                                                                            \
+      hipLaunchKernelGGL((embed_begin_norm_kernel<TW, TG, false>), dim3(16), dim3(256), 0, stream, tokens,          \
+                         (const TW*)table, resid, (const TG*)gamma, (bf16_t*)u, ss, n_tokens, width, vocab);        \
+  } while (0)
+  if (table_dtype == kF32 && gamma_dtype == kF32) ATOMA_EBN(float, float);
+  else if (table_dtype == kF32 && gamma_dtype == kBF16) ATOMA_EBN(float, bf16_t);
+  else if (table_dtype == kBF16 && gamma_dtype == kF32) ATOMA_EBN(bf16_t, float);
+  else if (table_dtype == kBF16 && gamma_dtype == kBF16) ATOMA_EBN(bf16_t, bf16_t);
+  else return ATOMA_ERR_DTYPE;
+#undef ATOMA_EBN
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// out [T][width] = u [T][width] / sqrt(sum_p ss[p][row] / width + eps), both bfloat16: the finished norm as a tensor,
+// for a reader that cannot finish it itself.  The shares are added in the order the products add them.
+__global__ void __launch_bounds__(256)
+finish_norm_kernel(const uint16_t* __restrict__ u, const float* __restrict__ ss, int parts, float eps,
+                   uint16_t* __restrict__ out, int width) {
+  __shared__ float scale_s;
+  const int t = blockIdx.x;
+  if (threadIdx.x < 64) {
+    const int kg = threadIdx.x >> 4;
+    float s = 0.f;
+    for (int p = kg; p < parts; p += 4) s += ss[p * 16 + t];
+    s += __shfl_xor(s, 16, 64);
+    s += __shfl_xor(s, 32, 64);
+    if (threadIdx.x == 0) scale_s = 1.0f / sqrtf(s / (float)width + eps);
+  }
+  __syncthreads();
+  const float scale = scale_s;
+  for (int i = threadIdx.x; i < width; i += 256)
+    out[(size_t)t * width + i] = f32_to_bf16_bits(bf16_bits_to_f32(u[(size_t)t * width + i]) * scale);
+}
+
+extern "C" int atoma_finish_norm(const void* u, const float* ss, int parts, float eps, void* out, int n_rows,
+                                 int width, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (n_rows > 16 || parts <= 0 || width <= 0) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(finish_norm_kernel, dim3(n_rows), dim3(256), 0, stream, (const uint16_t*)u, ss, parts, eps,
+                     (uint16_t*)out, width);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
@@ -75,26 +202,6 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
 
 // The same for rows of at most 4096 columns, a multiple of 4, with 16-byte aligned rows: every thread keeps its
 // values in registers between the two passes and all loads of a pass are issued together.
-struct f4 { float v[4]; };
-__device__ __forceinline__ f4 load4(const float* p) {
-  const float4 t = *reinterpret_cast<const float4*>(p);
-  return f4{{t.x, t.y, t.z, t.w}};
-}
-__device__ __forceinline__ f4 load4(const bf16_t* p) {
-  const uint2 t = *reinterpret_cast<const uint2*>(p);
-  return f4{{bf16_bits_to_f32((uint16_t)(t.x & 0xffff)), bf16_bits_to_f32((uint16_t)(t.x >> 16)),
-             bf16_bits_to_f32((uint16_t)(t.y & 0xffff)), bf16_bits_to_f32((uint16_t)(t.y >> 16))}};
-}
-__device__ __forceinline__ void store4(float* p, const f4& a) {
-  *reinterpret_cast<float4*>(p) = make_float4(a.v[0], a.v[1], a.v[2], a.v[3]);
-}
-__device__ __forceinline__ void store4(bf16_t* p, const f4& a) {
-  uint2 t;
-  t.x = (uint32_t)f32_to_bf16_bits(a.v[0]) | ((uint32_t)f32_to_bf16_bits(a.v[1]) << 16);
-  t.y = (uint32_t)f32_to_bf16_bits(a.v[2]) | ((uint32_t)f32_to_bf16_bits(a.v[3]) << 16);
-  *reinterpret_cast<uint2*>(p) = t;
-}
-
 template <typename TD, typename TW, typename TO>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(float* __restrict__ resid, const TD* __restrict__ delta, const TW* __restrict__ w,

@@ -31,18 +31,44 @@ struct RopeArgs {
   int page_size, nh, nkv, hd;
 };
 
-template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false, bool ROPE = false>
+// A norm that is finished by its neighbours (at most 16 rows of activations).
+//   In: the rows of A are residual rows times the norm's weight, not yet divided by their root mean square; the
+//   sums of squares of the residual rows arrive as ss_in [parts_in][16] (a part per producing wave), and every sum
+//   of this product is multiplied by 1 / sqrt(sum_p ss_in[p][row] / width_in + eps_in) before its epilogue: the
+//   product is linear in its rows, so this is the product of the normed rows.
+//   Out (resid != null): the product is not stored; it is added to the float32 residual rows resid [M][N] in
+//   place, u_out [M][N] receives residual times gamma as bfloat16 (the A of the next product) and ss_out
+//   [waves][16] each wave's share of the rows' sums of squares (the next product's ss_in).
+struct FuseArgs {
+  const float* ss_in;
+  int parts_in;
+  float eps_in, inv_width_in;
+  float* resid;
+  const void* gamma;       // [N] norm weight of the following norm
+  int gamma_is_bf16;
+  uint16_t* u_out;
+  float* ss_out;
+};
+
+// HALF (one tile of W, at most 16 rows of A, the residual epilogue): a wave owns 8 rows of W, not 16; the lanes of
+// the other 8 rows load nothing.  Twice as many workgroups then share a small N, and what a workgroup may have in
+// flight, not the matrix cores, is what bounds these products.
+template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false, bool ROPE = false, int UO = 0,
+          bool HALF = false>
 __global__ void __launch_bounds__(64 * WN * WK)
 gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
-                   int K, int lda, int ldw, int ldc, size_t plane, RopeArgs ra) {
+                   int K, int lda, int ldw, int ldc, size_t plane, RopeArgs ra, FuseArgs fa) {
   // loads of U steps of K are issued together before their MFMAs, so that a wave keeps U * (RT + MT) 16-byte
   // loads per lane in flight: the product is bound by memory latency and bandwidth, not by arithmetic
   // (eight waves of many tiles have 256 registers each: one step)
-  constexpr int U = (RT + MT <= 2) ? 4 : (RT + MT > 5 && WK > 4) ? 1 : 2;
+  constexpr int U = UO ? UO : (RT + MT <= 2) ? 4 : (RT + MT > 5 && WK > 4) ? 1 : 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wn = wave % WN, wk = wave / WN;
   const int r16 = lane & 15, kg = lane >> 4;
-  const int n_base = (blockIdx.x * WN + wn) * (RT * 16);
+  static_assert(!HALF || (RT == 1 && MT == 1 && !SWIGLU && !ROPE), "half tiles: one tile, residual epilogue");
+  const int n_base = (blockIdx.x * WN + wn) * (HALF ? 8 : RT * 16);
+  const bool w_on = !HALF || r16 < 8;                 // this lane loads a row of W
+  const bool a_on = !HALF || M > 8 || r16 < 8;        // ... and a row of A
   const int k_slices = gridDim.y * WK;
   const int k_len = K / k_slices;
   const int k_begin = (blockIdx.y * WK + wk) * k_len;
@@ -69,15 +95,43 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[r][m] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // what the fused norm needs from memory is asked for first, so that it has arrived when the sums are done
+  // The shares of the rows' sums of squares are added by all waves of the workgroup, up to sixteen per lane and row,
+  // and meet in LDS (behind the barrier that the K-split needs anyway).  They are asked for after the first loads
+  // of the weight (below) and added after the last MFMA, so that nothing waits for them.
+  __shared__ float ss_red[WN * WK][16];
+  const bool scaled = MT == 1 && fa.ss_in != nullptr;
+  constexpr int SS_STRIDE = 4 * WN * WK;
+  float ss_v[16];
+  auto load_shares = [&]() {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int p = wave * 4 + kg + j * SS_STRIDE;
+      ss_v[j] = (scaled && p < fa.parts_in) ? fa.ss_in[p * 16 + r16] : 0.f;
+    }
+  };
+  f32x4 res_in[RT];
+  if (MT == 1 && fa.resid != nullptr && wk == 0) {
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      const int n0 = n_base + r * 16 + kg * 4;
+      res_in[r] = (r16 < M && n0 + 3 < N && (!HALF || kg < 2))
+                      ? *reinterpret_cast<const f32x4*>(fa.resid + (size_t)r16 * N + n0)
+                      : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
   // two buffers of U steps each: while the MFMAs of one run, the loads of the other are in flight
   bf16x8 wf[2][U][RT], af[2][U][MT];
   auto load = [&](int buf, int k0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int r = 0; r < RT; ++r) wf[buf][u][r] = *reinterpret_cast<const bf16x8*>(wp[r] + k0 + u * 32);
+      for (int r = 0; r < RT; ++r)
+        wf[buf][u][r] = w_on ? *reinterpret_cast<const bf16x8*>(wp[r] + k0 + u * 32) : bf16x8{};
 #pragma unroll
-      for (int m = 0; m < MT; ++m) af[buf][u][m] = *reinterpret_cast<const bf16x8*>(ap[m] + k0 + u * 32);
+      for (int m = 0; m < MT; ++m)
+        af[buf][u][m] = a_on ? *reinterpret_cast<const bf16x8*>(ap[m] + k0 + u * 32) : bf16x8{};
     }
   };
   auto multiply = [&](int buf) {
@@ -94,6 +148,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   int k = 0;
   if (n_batches > 0) {
     load(0, 0);
+    if constexpr (MT == 1) load_shares();
     int b = 0;
     for (; b + 2 <= n_batches; b += 2) {
       load(1, (b + 1) * STEP);
@@ -107,14 +162,26 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   for (; k < k_len; k += 32) {
     bf16x8 wt[RT], at[MT];
 #pragma unroll
-    for (int r = 0; r < RT; ++r) wt[r] = *reinterpret_cast<const bf16x8*>(wp[r] + k);
+    for (int r = 0; r < RT; ++r) wt[r] = w_on ? *reinterpret_cast<const bf16x8*>(wp[r] + k) : bf16x8{};
 #pragma unroll
-    for (int m = 0; m < MT; ++m) at[m] = *reinterpret_cast<const bf16x8*>(ap[m] + k);
+    for (int m = 0; m < MT; ++m) at[m] = a_on ? *reinterpret_cast<const bf16x8*>(ap[m] + k) : bf16x8{};
 #pragma unroll
     for (int r = 0; r < RT; ++r)
 #pragma unroll
       for (int m = 0; m < MT; ++m)
         acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt[r], at[m], acc[r][m], 0, 0, 0);
+  }
+
+  if (scaled) {
+    if (n_batches <= 0) load_shares();
+    float ss_mine = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) ss_mine += ss_v[j];
+    for (int p = wave * 4 + kg + 16 * SS_STRIDE; p < fa.parts_in; p += SS_STRIDE) ss_mine += fa.ss_in[p * 16 + r16];
+    ss_mine += __shfl_xor(ss_mine, 16, 64);
+    ss_mine += __shfl_xor(ss_mine, 32, 64);
+    if (kg == 0) ss_red[wave][r16] = ss_mine;
+    if constexpr (WK == 1) __syncthreads();
   }
 
   if constexpr (WK > 1) {
@@ -141,6 +208,54 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
         for (int m = 0; m < MT; ++m)
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[r][m][i] += src[((r * MT + m) * 4 + i) * 64 + lane];
+    }
+  }
+
+  if constexpr (MT == 1) {
+    if (scaled) {
+      float t = 0.f;
+#pragma unroll
+      for (int i = 0; i < WN * WK; ++i) t += ss_red[i][r16];
+      const float row_scale = 1.0f / sqrtf(t * fa.inv_width_in + fa.eps_in);
+#pragma unroll
+      for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[r][0][i] *= row_scale;
+    }
+    if constexpr (!SWIGLU && !ROPE) {
+      if (fa.resid != nullptr) {
+        // lane (row r16, columns n0 .. n0 + 3 of each of its RT tiles): residual, next activations, squares
+        float ssq = 0.f;
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+          const int n0 = n_base + r * 16 + kg * 4;
+          if (r16 >= M || n0 + 3 >= N || (HALF && kg >= 2)) continue;
+          float g[4];
+          if (fa.gamma_is_bf16) {
+            const uint2 t = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(fa.gamma) + n0);
+            g[0] = bf16_bits_to_f32((uint16_t)(t.x & 0xffff)), g[1] = bf16_bits_to_f32((uint16_t)(t.x >> 16));
+            g[2] = bf16_bits_to_f32((uint16_t)(t.y & 0xffff)), g[3] = bf16_bits_to_f32((uint16_t)(t.y >> 16));
+          } else {
+            const f32x4 t = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(fa.gamma) + n0);
+            g[0] = t[0], g[1] = t[1], g[2] = t[2], g[3] = t[3];
+          }
+          f32x4 v;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            v[i] = res_in[r][i] + acc[r][0][i];
+            ssq += v[i] * v[i];
+          }
+          *reinterpret_cast<f32x4*>(fa.resid + (size_t)r16 * N + n0) = v;
+          uint2 o;
+          o.x = (uint32_t)f32_to_bf16_bits(v[0] * g[0]) | ((uint32_t)f32_to_bf16_bits(v[1] * g[1]) << 16);
+          o.y = (uint32_t)f32_to_bf16_bits(v[2] * g[2]) | ((uint32_t)f32_to_bf16_bits(v[3] * g[3]) << 16);
+          *reinterpret_cast<uint2*>(fa.u_out + (size_t)r16 * N + n0) = o;
+        }
+        ssq += __shfl_xor(ssq, 16, 64);
+        ssq += __shfl_xor(ssq, 32, 64);
+        if (kg == 0) fa.ss_out[(size_t)(blockIdx.x * WN + wn) * 16 + r16] = ssq;
+        return;
+      }
     }
   }
 
@@ -255,15 +370,15 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
 
 template <int MT, int RT, int WN, int WK>
 static int launch(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc,
-                  int slices, hipStream_t stream) {
+                  int slices, const FuseArgs& fa, hipStream_t stream) {
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), slices), block(64 * WN * WK);
   const size_t plane = (size_t)M * ldc;
   if (c_dtype == kF32)
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, float>), grid, block, 0, stream, (const uint16_t*)a,
-                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane, RopeArgs{});
+                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane, RopeArgs{}, fa);
   else if (c_dtype == kBF16)
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t>), grid, block, 0, stream, (const uint16_t*)a,
-                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane, RopeArgs{});
+                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane, RopeArgs{}, fa);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();
@@ -272,9 +387,10 @@ static int launch(const void* a, const void* w, void* c, int c_dtype, int M, int
 
 template <int MT>
 static int launch_mt(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, int lda, int ldw,
-                     int ldc, int rt, int wk, int slices, hipStream_t stream) {
+                     int ldc, int rt, int wk, int slices, const FuseArgs& fa, hipStream_t stream) {
 #define ATOMA_CASE(R, WN_, WK_)                                                                                   \
-  if (rt == R && wk == WK_) return launch<MT, R, WN_, WK_>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, slices, stream)
+  if (rt == R && wk == WK_)                                                                                       \
+  return launch<MT, R, WN_, WK_>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, slices, fa, stream)
   ATOMA_CASE(1, 4, 1);
   ATOMA_CASE(2, 4, 1);
   ATOMA_CASE(4, 4, 1);
@@ -290,81 +406,155 @@ static int launch_mt(const void* a, const void* w, void* c, int c_dtype, int M, 
 // a [M <= 64, K] bf16, w [N, K] bf16 -> c [slices][M, N] (bf16 only with slices == 1, or float32).
 // rt: tiles of 16 rows of W per wave (1, 2, 4); wk: 1 (four waves on different rows), 4 or 8 (that many waves
 // split K for the same rows; four tiles only with 4); slices: K split across the grid.
-extern "C" int atoma_gemm_bf16_skinny(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
-                                      int lda, int ldw, int ldc, int rt, int wk, int slices, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || slices <= 0 || K % (32 * wk * slices) || (lda & 7) || (ldw & 7) || lda < K || ldw < K ||
-      ldc < N || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || (slices > 1 && c_dtype != kF32) || slices > 65535)
-    return ATOMA_ERR_SHAPE;
+static bool fuse_in_ok(const float* ss_in, int parts_in, float eps_in, int width_in, int M) {
+  return ss_in == nullptr || (M <= 16 && parts_in > 0 && width_in > 0 && eps_in >= 0.f);
+}
+
+static FuseArgs fuse_in(const float* ss_in, int parts_in, float eps_in, int width_in) {
+  FuseArgs fa{};
+  fa.ss_in = ss_in;
+  fa.parts_in = parts_in;
+  fa.eps_in = eps_in;
+  fa.inv_width_in = width_in > 0 ? 1.0f / (float)width_in : 0.f;
+  return fa;
+}
+
+static int skinny_dispatch(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K, int lda, int ldw,
+                           int ldc, int rt, int wk, int slices, const FuseArgs& fa, hipStream_t stream) {
   const int mt = (M + 15) / 16;
   switch (mt) {
-    case 1: return launch_mt<1>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
-    case 2: return launch_mt<2>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
-    case 3: return launch_mt<3>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
-    default: return launch_mt<4>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, stream);
+    case 1: return launch_mt<1>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, fa, stream);
+    case 2: return launch_mt<2>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, fa, stream);
+    case 3: return launch_mt<3>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, fa, stream);
+    default: return launch_mt<4>(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices, fa, stream);
   }
+}
+
+extern "C" int atoma_gemm_bf16_skinny(const void* a, const void* w, void* c, int c_dtype, int M, int N, int K,
+                                      int lda, int ldw, int ldc, int rt, int wk, int slices, const float* ss_in,
+                                      int parts_in, float eps_in, int width_in, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || slices <= 0 || K % (32 * wk * slices) || (lda & 7) || (ldw & 7) || lda < K || ldw < K ||
+      ldc < N || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || (slices > 1 && c_dtype != kF32) || slices > 65535 ||
+      !fuse_in_ok(ss_in, parts_in, eps_in, width_in, M) || (ss_in && slices > 1))
+    return ATOMA_ERR_SHAPE;
+  return skinny_dispatch(a, w, c, c_dtype, M, N, K, lda, ldw, ldc, rt, wk, slices,
+                         fuse_in(ss_in, parts_in, eps_in, width_in), stream);
+}
+
+// The product of at most 16 rows added to the residual stream, with the following norm begun (see FuseArgs):
+// resid [M][N] float32 += a w^T in place, u_out [M][N] bfloat16 = resid * gamma, ss_out [parts][16] the shares of
+// the rows' sums of squares, parts = atoma_gemm_bf16_resid_parts(N, rt, wk, half).  half: 8 rows of W a wave (see the kernel).  depth: steps of K whose loads a wave
+// issues together (two such batches are in flight).  The rows of a may themselves be an
+// unfinished norm (ss_in).  K is split over the waves of a workgroup only, so every sum has one owner.
+extern "C" int atoma_gemm_bf16_resid_parts(int N, int rt, int wk, int half) {
+  const int wn = wk == 1 ? 4 : 1;
+  const int cols = half ? wn * 8 : wn * rt * 16;
+  return ((N + cols - 1) / cols) * wn;
+}
+
+extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M, int N, int K, int lda, int ldw,
+                                            int rt, int wk, int depth, int half, const float* ss_in, int parts_in, float eps_in,
+                                            int width_in, float* resid, const void* gamma, int gamma_dtype,
+                                            void* u_out, float* ss_out, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K <= 0 || K % (32 * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K || (N & 3) ||
+      ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || !resid || !gamma || !u_out || !ss_out ||
+      ((uintptr_t)resid & 15) || ((uintptr_t)gamma & 15) || ((uintptr_t)u_out & 7) ||
+      (gamma_dtype != kF32 && gamma_dtype != kBF16) || !fuse_in_ok(ss_in, parts_in, eps_in, width_in, M))
+    return ATOMA_ERR_SHAPE;
+  FuseArgs fa = fuse_in(ss_in, parts_in, eps_in, width_in);
+  fa.resid = resid;
+  fa.gamma = gamma;
+  fa.gamma_is_bf16 = gamma_dtype == kBF16;
+  fa.u_out = (uint16_t*)u_out;
+  fa.ss_out = ss_out;
+  // (the float32 instance; nothing is stored through c)
+#define ATOMA_RESID(R, WN_, WK_, U_, H_)                                                                           \
+  if (rt == R && wk == WK_ && depth == U_ && (half != 0) == H_) {                                                  \
+    const int cols = H_ ? WN_ * 8 : WN_ * R * 16;                                                                  \
+    dim3 grid((N + cols - 1) / cols, 1), block(64 * WN_ * WK_);                                                    \
+    hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN_, WK_, float, false, false, U_, H_>), grid, block, 0, stream,  \
+                       (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0, RopeArgs{}, \
+                       fa);                                                                                        \
+    ATOMA_LAUNCH_CHECK();                                                                                          \
+    return 0;                                                                                                      \
+  }
+  ATOMA_RESID(1, 1, 4, 4, false)
+  ATOMA_RESID(1, 1, 8, 4, false)
+  ATOMA_RESID(1, 4, 1, 4, false)
+  ATOMA_RESID(1, 1, 4, 4, true)
+  ATOMA_RESID(1, 1, 4, 8, true)
+  ATOMA_RESID(1, 1, 8, 4, true)
+  ATOMA_RESID(1, 1, 8, 8, true)
+  ATOMA_RESID(1, 4, 1, 4, true)
+#undef ATOMA_RESID
+  return ATOMA_ERR_SHAPE;
 }
 
 template <int MT, int RT, int WN, int WK>
 static int launch_swiglu(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
-                         hipStream_t stream) {
+                         const FuseArgs& fa, hipStream_t stream) {
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, true>), grid, block, 0, stream, (const uint16_t*)a,
-                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, RopeArgs{});
+                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, RopeArgs{}, fa);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
 
 template <int MT>
 static int launch_swiglu_mt(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
-                            int rt, int wk, hipStream_t stream) {
-  if (rt == 2 && wk == 1) return launch_swiglu<MT, 2, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, stream);
-  if (rt == 4 && wk == 1) return launch_swiglu<MT, 4, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, stream);
-  if (rt == 2 && wk == 4) return launch_swiglu<MT, 2, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+                            int rt, int wk, const FuseArgs& fa, hipStream_t stream) {
+  if (rt == 2 && wk == 1) return launch_swiglu<MT, 2, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, fa, stream);
+  if (rt == 4 && wk == 1) return launch_swiglu<MT, 4, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, fa, stream);
+  if (rt == 2 && wk == 4) return launch_swiglu<MT, 2, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, fa, stream);
   if constexpr (MT < 4) {   // with four tiles of rows the epilogue does not fit the registers of eight waves
-    if (rt == 2 && wk == 8) return launch_swiglu<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+    if (rt == 2 && wk == 8) return launch_swiglu<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, fa, stream);
   }
-  if (rt == 4 && wk == 4) return launch_swiglu<MT, 4, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, stream);
+  if (rt == 4 && wk == 4) return launch_swiglu<MT, 4, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, fa, stream);
   return ATOMA_ERR_SHAPE;
 }
 
 // The gate-up product with SiLU(gate) * up in its epilogue.  w [N, K] holds gate and up rows interleaved in blocks
 // of 16 (16 gate rows, then the 16 up rows of the same outputs); c is [M, N / 2] bfloat16.  N % 32 == 0.
 extern "C" int atoma_gemm_bf16_skinny_swiglu(const void* a, const void* w, void* c, int M, int N, int K, int lda,
-                                             int ldw, int ldc, int rt, int wk, hipStream_t stream) {
+                                             int ldw, int ldc, int rt, int wk, const float* ss_in, int parts_in,
+                                             float eps_in, int width_in, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % (32 * wk) || (N & 31) || (lda & 7) || (ldw & 7) || lda < K || ldw < K || ldc < N / 2 ||
-      (ldc & 3) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)c & 7))
+      (ldc & 3) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)c & 7) ||
+      !fuse_in_ok(ss_in, parts_in, eps_in, width_in, M))
     return ATOMA_ERR_SHAPE;
+  const FuseArgs fa = fuse_in(ss_in, parts_in, eps_in, width_in);
   switch ((M + 15) / 16) {
-    case 1: return launch_swiglu_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
-    case 2: return launch_swiglu_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
-    case 3: return launch_swiglu_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
-    default: return launch_swiglu_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, stream);
+    case 1: return launch_swiglu_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, fa, stream);
+    case 2: return launch_swiglu_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, fa, stream);
+    case 3: return launch_swiglu_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, fa, stream);
+    default: return launch_swiglu_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, fa, stream);
   }
 }
 
 template <int MT, int RT, int WN, int WK>
 static int launch_rope(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
-                       const RopeArgs& ra, hipStream_t stream) {
+                       const RopeArgs& ra, const FuseArgs& fa, hipStream_t stream) {
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, false, true>), grid, block, 0, stream,
-                     (const uint16_t*)a, (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, ra);
+                     (const uint16_t*)a, (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, ra, fa);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
 
 template <int MT>
 static int launch_rope_mt(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
-                          int rt, int wk, const RopeArgs& ra, hipStream_t stream) {
-  if (rt == 1 && wk == 4) return launch_rope<MT, 1, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
-  if (rt == 2 && wk == 4) return launch_rope<MT, 2, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
-  if (rt == 1 && wk == 8) return launch_rope<MT, 1, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+                          int rt, int wk, const RopeArgs& ra, const FuseArgs& fa, hipStream_t stream) {
+  if (rt == 1 && wk == 4) return launch_rope<MT, 1, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, ra, fa, stream);
+  if (rt == 2 && wk == 4) return launch_rope<MT, 2, 1, 4>(a, w, c, M, N, K, lda, ldw, ldc, ra, fa, stream);
+  if (rt == 1 && wk == 8) return launch_rope<MT, 1, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, fa, stream);
   if constexpr (MT < 4) {   // with four tiles of rows the epilogue does not fit the registers of eight waves
-    if (rt == 2 && wk == 8) return launch_rope<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+    if (rt == 2 && wk == 8) return launch_rope<MT, 2, 1, 8>(a, w, c, M, N, K, lda, ldw, ldc, ra, fa, stream);
   }
-  if (rt == 1 && wk == 1) return launch_rope<MT, 1, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
-  if (rt == 2 && wk == 1) return launch_rope<MT, 2, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, ra, stream);
+  if (rt == 1 && wk == 1) return launch_rope<MT, 1, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, ra, fa, stream);
+  if (rt == 2 && wk == 1) return launch_rope<MT, 2, 4, 1>(a, w, c, M, N, K, lda, ldw, ldc, ra, fa, stream);
   return ATOMA_ERR_SHAPE;
 }
 
@@ -377,9 +567,12 @@ extern "C" int atoma_gemm_bf16_skinny_rope(const void* a, const void* w, void* c
                                            int ldc, int rt, int wk, const int32_t* positions, const float* cos_t,
                                            const float* sin_t, void* kcache, void* vcache,
                                            const int32_t* slot_mapping, int page_size, int nh, int nkv, int hd,
+                                           const float* ss_in, int parts_in, float eps_in, int width_in,
                                            hipStream_t stream) {
   if (M <= 0) return 0;
   const int N = (nh + 2 * nkv) * hd;
+  if (!fuse_in_ok(ss_in, parts_in, eps_in, width_in, M)) return ATOMA_ERR_SHAPE;
+  const FuseArgs fa = fuse_in(ss_in, parts_in, eps_in, width_in);
   if (M > 64 || K <= 0 || wk <= 0 || K % (32 * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K ||
       ldc < nh * hd || (ldc & 1) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)c & 3) || (hd & 3) ||
       nh <= 0 || nkv <= 0 || page_size <= 0 || !positions || !cos_t || !sin_t || !kcache || !vcache ||
@@ -387,9 +580,9 @@ extern "C" int atoma_gemm_bf16_skinny_rope(const void* a, const void* w, void* c
     return ATOMA_ERR_SHAPE;
   const RopeArgs ra{positions, cos_t, sin_t, (uint16_t*)kcache, (uint16_t*)vcache, slot_mapping, page_size, nh, nkv, hd};
   switch ((M + 15) / 16) {
-    case 1: return launch_rope_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
-    case 2: return launch_rope_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
-    case 3: return launch_rope_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
-    default: return launch_rope_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, stream);
+    case 1: return launch_rope_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, fa, stream);
+    case 2: return launch_rope_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, fa, stream);
+    case 3: return launch_rope_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, fa, stream);
+    default: return launch_rope_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, fa, stream);
   }
 }

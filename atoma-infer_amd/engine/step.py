@@ -78,6 +78,8 @@ class StepContext:
     scratch: Dict[object, object] = dataclasses.field(default_factory=dict)
     #: not None inside a decode graph: the number of 256-token buckets the graph serves
     decode_bucket: Optional[int] = None
+    #: the logits of every token are wanted, in the order of the tokens (``want_rows`` counts 0, 1, 2, ...)
+    wants_all_rows: bool = False
 
     def layer_cache(self, pos: int) -> LayerCache:
         return self.pool.layer_cache(pos, self.slot_mappings, self.block_tables)
@@ -302,7 +304,9 @@ class ModelRunner:
             slot_mappings=[dev[o_sm + g * t: o_sm + (g + 1) * t] for g in range(n_groups)],
             block_tables=[dev[o_bt + g * s * max_blocks: o_bt + (g + 1) * s * max_blocks].view(s, max_blocks)
                           for g in range(n_groups)],
-            pool=self.pool, decode_bucket=bucket)
+            pool=self.pool, decode_bucket=bucket,
+            wants_all_rows=n_want == t and all(len(e.want) == len(e.tokens) and
+                                               all(w == j for j, w in enumerate(e.want)) for e in entries))
         for off, (key, arr, meta) in zip(ex_off, extras):
             ctx.plans[key] = (dev[off: off + arr.size].view(arr.shape), meta)
         return ctx

@@ -10,6 +10,8 @@
 """
 from __future__ import annotations
 
+import ctypes
+import dataclasses
 from typing import Optional
 
 import torch
@@ -18,6 +20,40 @@ from .library import load_hip_module
 from .ops import BF16, F32, _check, _p, _stream
 
 SKINNY_MAX_M = 64
+BEGUN_MAX_M = 16              # rows of a step whose norms are begun and finished by the products around them
+
+
+@dataclasses.dataclass
+class Begun:
+    """Activations whose norm is begun: ``data`` [T <= 16, W] bfloat16 is residual times norm weight, ``shares``
+    [parts, 16] float32 the rows' sums of squares in parts; the finished row is
+    ``data[t] / sqrt(shares[:, t].sum() / width + eps)``.  Products of this module finish it in their epilogue
+    (they are linear in their rows); ``tensor()`` finishes it into a tensor for any other reader."""
+    data: torch.Tensor
+    shares: torch.Tensor
+    eps: float
+    width: int
+    norm: object = None      # the part whose norm this is, so that no other takes it for its own
+
+    @property
+    def shape(self):
+        return self.data.shape
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    def tensor(self) -> torch.Tensor:
+        from . import ops
+        return ops.finish_norm(self.data, self.shares, self.eps, self.width)
+
+
+def _begun_args(x):
+    """The four trailing arguments of a product whose rows may be a begun norm."""
+    if isinstance(x, Begun):
+        return _p(x.shares), x.shares.shape[0], ctypes.c_float(x.eps), x.width
+    return _p(None), 0, ctypes.c_float(0.0), 0
+
 LIBRARY_MIN_M_WIDE = 32       # beyond this many rows the library takes products whose weight has 2^24 elements or more
 SWIGLU_WIDE = 1 << 25         # weights up to this size keep the fused SiLU-multiply up to 64 rows
 _lib = None
@@ -89,8 +125,11 @@ def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
             and x.shape[1] == w.shape[1] and x.shape[1] % 32 == 0 and _aligned(x) and _aligned(w))
 
 
-def skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, slices: int = 1, rt: int = 0, wk: int = 0) -> None:
-    """out [M, N] (or [slices, M, N] float32 planes) = x [M <= 64, K] @ w [N, K]^T."""
+def skinny(x, w: torch.Tensor, out: torch.Tensor, slices: int = 1, rt: int = 0, wk: int = 0) -> None:
+    """out [M, N] (or [slices, M, N] float32 planes) = x [M <= 64, K] @ w [N, K]^T; x may be a ``Begun`` norm."""
+    begun = _begun_args(x)
+    if isinstance(x, Begun):
+        x = x.data
     m, k = x.shape
     n = w.shape[0]
     if not rt:
@@ -100,7 +139,7 @@ def skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, slices: int = 1,
     ldc = out.stride(-2) if m > 1 else n
     code = {torch.float32: F32, torch.bfloat16: BF16}[out.dtype]
     _check(lib().atoma_gemm_bf16_skinny(_p(x), _p(w), _p(out), code, m, n, k, x.stride(0) if m > 1 else k,
-                                        w.stride(0) if n > 1 else k, ldc, rt, wk, slices, _stream()),
+                                        w.stride(0) if n > 1 else k, ldc, rt, wk, slices, *begun, _stream()),
            "gemm_bf16_skinny")
 
 
@@ -130,6 +169,13 @@ def try_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Op
                library_only: bool = False) -> Optional[torch.Tensor]:
     """x [M, K] @ w [N, K]^T if a fast kernel takes the shape, else None (the caller falls back to float32 FMAs).
     ``library_only``: None also where the library would not be the choice."""
+    if isinstance(x, Begun):
+        if not skinny_ok(x.data, w):
+            return None
+        if out is None:
+            out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=w.device)
+        skinny(x, w, out)
+        return out
     m, n = x.shape[0], w.shape[0]
     k = x.shape[1]
     ok = skinny_ok(x, w)
@@ -173,6 +219,9 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
 
     None when the shape is not taken (the caller then runs the product and the activation separately).
     """
+    begun = _begun_args(x)
+    if isinstance(x, Begun):
+        x = x.data
     m, k = x.shape
     n = w.shape[0]
     if m > SKINNY_MAX_M or (m > LIBRARY_MIN_M_WIDE and n * k > SWIGLU_WIDE) or n % 32 or not skinny_ok(x, w):
@@ -184,7 +233,8 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
         return None
     out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     _check(lib().atoma_gemm_bf16_skinny_swiglu(_p(x), _p(w), _p(out), m, n, k, x.stride(0) if m > 1 else k,
-                                               w.stride(0), n // 2, rt, wk, _stream()), "gemm_bf16_skinny_swiglu")
+                                               w.stride(0), n // 2, rt, wk, *begun, _stream()),
+           "gemm_bf16_skinny_swiglu")
     return out
 
 
@@ -200,6 +250,9 @@ def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, c
     [M, nh * hd]; k (rotated) and v are in the cache.  None when the shape is not taken, or when the library's
     product followed by the rotary kernel is the quicker way (unless ``always``).
     """
+    begun = _begun_args(x)
+    if isinstance(x, Begun):
+        x = x.data
     m, k = x.shape
     n = w.shape[0]
     if (m > ROPE_MAX_M or (not always and _library_wins(m, n, k, torch.bfloat16)) or n != (nh + 2 * nkv) * hd or hd % 4 or not skinny_ok(x, w)
@@ -213,6 +266,41 @@ def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, c
     out = torch.empty((m, nh * hd), dtype=torch.bfloat16, device=x.device)
     _check(lib().atoma_gemm_bf16_skinny_rope(_p(x), _p(w), _p(out), m, k, x.stride(0) if m > 1 else k, w.stride(0),
                                              nh * hd, rt, wk, _p(positions), _p(cos), _p(sin), _p(kcache), _p(vcache),
-                                             _p(slot_mapping), int(page_size), nh, nkv, hd, _stream()),
+                                             _p(slot_mapping), int(page_size), nh, nkv, hd, *begun, _stream()),
            "gemm_bf16_skinny_rope")
     return out
+
+
+def resid_plan(m: int, n: int, k: int):
+    """(rows-of-16 per wave, waves splitting K, steps of K per batch of loads) of the product that adds into the residual stream: K is split over
+    the waves of a workgroup only (every sum has one owner, which also begins the norm), as many ways as K allows,
+    and a wave owns 8 rows of the weight, so that N = 2048 still makes 256 workgroups (measured at Llama 1B's o and
+    down products: 5.3 and 12.7 us against 5.9 and 15.0 with 16 rows a wave)."""
+    wk = 8
+    while wk > 1 and k % (32 * wk):
+        wk //= 2
+    if wk == 2:
+        wk = 1
+    return 1, wk, 4, 1
+
+
+def try_linear_resid(x, w: torch.Tensor, resid: torch.Tensor, gamma: torch.Tensor, eps: float) -> Optional[Begun]:
+    """resid [M <= 16, N] float32 += x @ w^T in place, with the norm (gamma, eps) of the new rows begun: returns
+    it as ``Begun``, or None (and nothing done) when the shape is not taken.  x may itself be ``Begun``."""
+    begun = _begun_args(x)
+    xd = x.data if isinstance(x, Begun) else x
+    m, k = xd.shape
+    n = w.shape[0]
+    if (m > BEGUN_MAX_M or not skinny_ok(xd, w) or n % 4 or resid.dtype is not torch.float32
+            or tuple(resid.shape) != (m, n) or not resid.is_contiguous() or not gamma.is_contiguous()
+            or gamma.numel() != n or gamma.dtype not in (torch.float32, torch.bfloat16)):
+        return None
+    rt, wk, depth, half = resid_plan(m, n, k)
+    parts = lib().atoma_gemm_bf16_resid_parts(n, rt, wk, half)
+    u = torch.empty((m, n), dtype=torch.bfloat16, device=w.device)
+    shares = torch.empty((parts, 16), dtype=torch.float32, device=w.device)
+    code = F32 if gamma.dtype is torch.float32 else BF16
+    _check(lib().atoma_gemm_bf16_skinny_resid(_p(xd), _p(w), m, n, k, xd.stride(0) if m > 1 else k, w.stride(0), rt, wk,
+                                              depth, half, *begun, _p(resid), _p(gamma), code, _p(u), _p(shares), _stream()),
+           "gemm_bf16_skinny_resid")
+    return Begun(u, shares, float(eps), n)

@@ -98,6 +98,36 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor]
     return out
 
 
+def embed_begin_norm(tokens: torch.Tensor, table: torch.Tensor, gamma: torch.Tensor):
+    """The embedding gather with a norm begun, for at most 16 tokens: (resid float32 [T, W], u bfloat16 [T, W] =
+    resid * gamma, ss float32 [1, 16] the rows' sums of squares).  A product finishes the norm (gemm_bf16)."""
+    _dev(tokens, table, gamma)
+    _i32(tokens, "tokens")
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, width]")
+    n, width = tokens.numel(), table.shape[1]
+    _need(0 < n <= 16, "embed_begin_norm takes at most 16 tokens")
+    _need(gamma.is_contiguous() and gamma.numel() == width, "norm weight must have one entry per column")
+    resid = torch.empty((n, width), dtype=torch.float32, device=table.device)
+    u = torch.empty((n, width), dtype=torch.bfloat16, device=table.device)
+    ss = torch.empty((1, 16), dtype=torch.float32, device=table.device)
+    _check(core().atoma_embed_begin_norm(_p(tokens), _p(table), _code(table, "embedding table"), _p(resid), _p(gamma),
+                                         _code(gamma, "norm weight"), _p(u), _p(ss), n, width, table.shape[0],
+                                         _stream()), "embed_begin_norm")
+    return resid, u, ss
+
+
+def finish_norm(u: torch.Tensor, ss: torch.Tensor, eps: float, width: int) -> torch.Tensor:
+    """u [T <= 16, W] bfloat16 divided by sqrt(sum_p ss[p, row] / width + eps), row by row, as bfloat16."""
+    _dev(u, ss)
+    _need(u.dtype is torch.bfloat16 and u.dim() == 2 and u.is_contiguous() and u.shape[0] <= 16, "finish_norm: bad u")
+    _need(ss.dtype is torch.float32 and ss.dim() == 2 and ss.shape[1] == 16 and ss.is_contiguous(),
+          "finish_norm: shares must be float32 [parts, 16]")
+    out = torch.empty_like(u)
+    _check(core().atoma_finish_norm(_p(u), _p(ss), ss.shape[0], ctypes.c_float(eps), _p(out), u.shape[0], u.shape[1],
+                                    _stream()), "finish_norm")
+    return out
+
+
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:

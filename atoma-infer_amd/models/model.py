@@ -13,6 +13,7 @@ import torch
 
 from ..config.base import ModelConfig
 from ..config.registry import Architecture, load_model_config
+from ..kernels.gemm_bf16 import Begun
 from ..weights.loader import load_into, load_random_into
 from .spec import ModelSpec
 
@@ -38,13 +39,23 @@ class Model:
     def forward(self, ctx) -> Optional[torch.Tensor]:
         """Logits [wanted rows, vocab] in float32, or None when the step wants none."""
         spec = self.spec
-        resid = spec.embedding[1].forward(ctx.tokens)
-        delta = None
-        for pos, call in enumerate(spec.run_order):
-            delta = spec.layers[call.layer][1].forward(resid, delta, ctx, ctx.layer_cache(pos))
+        blocks = [spec.layers[call.layer][1] for call in spec.run_order]
+        # the norm that reads each block's output: a block that can lets its last product begin that norm
+        readers = [b.entry_norm() for b in blocks[1:]]
+        readers.append(spec.final_norm[1] if getattr(ctx, "wants_all_rows", False) else None)
+        first = blocks[0].entry_norm() if blocks else None
+        resid, pending = spec.embedding[1].forward(ctx.tokens, first) if first is not None else \
+            (spec.embedding[1].forward(ctx.tokens), None)
+        for pos, block in enumerate(blocks):
+            if block.fuses_next_norm:
+                pending = block.forward(resid, pending, ctx, ctx.layer_cache(pos), next_norm=readers[pos])
+            else:
+                pending = block.forward(resid, pending, ctx, ctx.layer_cache(pos))
         if ctx.n_want == 0:
             return None
-        x = spec.final_norm[1].add_norm(resid, delta, rows=ctx.want_rows)
+        if isinstance(pending, Begun):      # the final norm, begun by the last product, on every row
+            return spec.head[1].forward(pending)
+        x = spec.final_norm[1].add_norm(resid, pending, rows=ctx.want_rows)
         return spec.head[1].forward(x)
 
 

@@ -23,7 +23,7 @@ import torch
 
 from ..kernels import ops
 from .base import CacheSpec, Mixer, PositionEncoding, WeightSpec, register_mixer
-from .linear import linear, linear_delta
+from .linear import as_tensor, linear, linear_delta
 
 
 class PagedAttention(Mixer):
@@ -91,7 +91,10 @@ class PagedAttention(Mixer):
                     max_waves=attention_bf16.max_waves_for(self.hd)))
 
     # -- execution ------------------------------------------------------------------------------------
-    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+    accepts_begun = True
+    takes_sink = True
+
+    def forward(self, x, ctx, cache, sink=None):
         nh, nkv, hd = self.nh, self.nkv, self.hd
         t = x.shape[0]
         writes = cache.writable
@@ -104,6 +107,8 @@ class PagedAttention(Mixer):
             from ..kernels import gemm_bf16
             qkv = gemm_bf16.try_linear_rope(x, w, ctx.positions, tables[0], tables[1], k_cache, v_cache,
                                             cache.slot_mapping, cache.page_size, nh, nkv, hd)
+        if qkv is None:
+            x = as_tensor(x)
         if qkv is not None:
             pass        # rotated and stored by the product's epilogue
         elif tables is not None or self.position is None:
@@ -129,7 +134,7 @@ class PagedAttention(Mixer):
                 self.position.apply(q, q[:, :0], ctx.positions)
         out = torch.empty((t, nh * hd), dtype=qkv.dtype, device=qkv.device)
         self.attend(qkv, k_cache, v_cache, out, ctx, cache)
-        return linear_delta(out, self.w_o)
+        return linear_delta(out, self.w_o, sink)
 
     def attend(self, q, k_cache, v_cache, out, ctx, cache) -> None:
         if q.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16:

@@ -91,6 +91,17 @@ class Norm(Part):
         """
         raise NotImplementedError
 
+    # Optional: a norm may be *begun* by the kernel that makes its input rows and finished by the product that reads
+    # them (``kernels.gemm_bf16.Begun``), which saves the norm's own launch where launches are what a step costs.
+    # A norm that cannot says None, and the caller runs ``add_norm``.
+    def add_product(self, resid: torch.Tensor, x, w: torch.Tensor):
+        """``resid += x @ w^T`` in place with this norm of the new rows begun, as ``Begun``; or None, nothing done."""
+        return None
+
+    def embed(self, table: torch.Tensor, tokens: torch.Tensor):
+        """(resid, Begun) for the rows ``table[tokens]`` with this norm begun; or None."""
+        return None
+
 
 class PositionEncoding(Part):
     """Encodes positions into queries and keys."""
@@ -109,7 +120,14 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    """Mixes information between the tokens of a request (attention here)."""
+    """Mixes information between the tokens of a request (attention here).
+
+    Two class attributes widen the contract for parts that know how (both default to False, and a part that leaves
+    them so sees tensors only): ``accepts_begun``: ``x`` may be a ``Begun`` norm, to be handed to ``linear`` and its
+    fused relatives; ``takes_sink``: ``forward`` has a keyword ``sink`` (a ``ResidualSink`` or None) and may hand its
+    last product to ``linear_delta(x, w, sink)``, whose result it returns as it is."""
+    accepts_begun = False
+    takes_sink = False
 
     def cache_spec(self) -> Optional[CacheSpec]:
         return None
@@ -123,6 +141,9 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_begun = False      # as for mixers
+    takes_sink = False
+
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         raise NotImplementedError
 
@@ -131,10 +152,17 @@ class Block(Part):
     """An arrangement of norms, a mixer and a feed-forward around the residual stream."""
 
     mixer: Mixer
+    #: True if ``forward`` has a keyword ``next_norm``: the norm that will read this block's output (the next
+    #: block's ``entry_norm()``, or the final norm), so that the block's last product may begin it
+    fuses_next_norm = False
 
     def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], ctx, cache) -> torch.Tensor:
         """Consume the pending ``delta`` into ``resid`` (float32 [T, width], in place) and return the new pending delta."""
         raise NotImplementedError
+
+    def entry_norm(self) -> Optional[Norm]:
+        """The norm that consumes the pending delta, if the block before may begin it; None otherwise."""
+        return None
 
 
 _KINDS: Dict[str, Dict[str, Callable]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}}

@@ -8,7 +8,9 @@ from __future__ import annotations
 
 from typing import Dict
 
+from ..kernels.gemm_bf16 import Begun
 from .base import Block, FeedForward, Mixer, Norm, WeightSpec, register_block
+from .linear import ResidualSink
 
 
 class PreNormBlock(Block):
@@ -33,10 +35,30 @@ class PreNormBlock(Block):
     def device_bytes(self) -> int:
         return sum(part.device_bytes() for _, part in self._children())
 
-    def forward(self, resid, delta, ctx, cache):
-        x = self.norm1.add_norm(resid, delta)
-        a = self.mixer.forward(x, ctx, cache)
-        x = self.norm2.add_norm(resid, a)
+    fuses_next_norm = True
+
+    def entry_norm(self):
+        return self.norm1
+
+    @staticmethod
+    def _normed(norm, resid, pending, reader):
+        """The input of ``reader``: ``pending`` is either a delta still to be added and normed, or ``norm`` already
+        begun by the product that made it (which has also added it to ``resid``)."""
+        if isinstance(pending, Begun):
+            if pending.norm is not norm:
+                raise RuntimeError("a begun norm reached another norm than the one it was begun for")
+            return pending if reader.accepts_begun else pending.tensor()
+        return norm.add_norm(resid, pending)
+
+    def forward(self, resid, delta, ctx, cache, next_norm=None):
+        x = self._normed(self.norm1, resid, delta, self.mixer)
+        if self.mixer.takes_sink:
+            a = self.mixer.forward(x, ctx, cache, sink=ResidualSink(resid, self.norm2))
+        else:
+            a = self.mixer.forward(x, ctx, cache)
+        x = self._normed(self.norm2, resid, a, self.feed_forward)
+        if self.feed_forward.takes_sink and next_norm is not None:
+            return self.feed_forward.forward(x, ctx, sink=ResidualSink(resid, next_norm))
         return self.feed_forward.forward(x, ctx)
 
 

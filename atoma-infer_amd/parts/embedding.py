@@ -32,8 +32,13 @@ class TokenEmbedding(Part):
     def device_bytes(self) -> int:
         return 0  # a step reads only the rows of its tokens
 
-    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
-        return ops.embed(tokens, self.weight)
+    def forward(self, tokens: torch.Tensor, norm=None):
+        """The float32 residual rows of ``tokens``; with ``norm`` (the norm that reads them first) a pair (rows,
+        that norm begun or None)."""
+        if norm is None:
+            return ops.embed(tokens, self.weight)
+        got = norm.embed(self.weight, tokens)
+        return got if got is not None else (ops.embed(tokens, self.weight), None)
 
 
 class OutputHead(Part):
@@ -53,5 +58,5 @@ class OutputHead(Part):
     def device_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x) -> torch.Tensor:
         return linear(x, self.weight, torch.float32)

@@ -46,14 +46,17 @@ class SwiGLU(FeedForward):
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+    accepts_begun = True
+    takes_sink = True
+
+    def forward(self, x, ctx, sink=None):
         h = None
         if self.block and x.dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16:
             from ..kernels import gemm_bf16
             h = gemm_bf16.try_linear_swiglu(x, self.w_gate_up)
         if h is None:
             h = ops.swiglu(linear(x, self.w_gate_up), block=self.block)
-        return linear_delta(h, self.w_down)
+        return linear_delta(h, self.w_down, sink)
 
 
 register_feed_forward("swiglu", SwiGLU)

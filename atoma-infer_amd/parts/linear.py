@@ -10,31 +10,53 @@ Which kernel runs is decided by the operands, never by the model:
 """
 from __future__ import annotations
 
+import dataclasses
 from typing import Optional
 
 import torch
 
 from ..kernels import ops
+from ..kernels.gemm_bf16 import Begun
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+@dataclasses.dataclass
+class ResidualSink:
+    """Where a part's last product may add itself: the float32 residual rows and the norm that reads them next."""
+    resid: torch.Tensor
+    norm: object
+
+
+def as_tensor(x) -> torch.Tensor:
+    """``x`` as a tensor: a begun norm is finished."""
+    return x.tensor() if isinstance(x, Begun) else x
+
+
+def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
            out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x [M, K] (row stride free) times w [N, K] transposed -> [M, N] in ``out_dtype`` (default: x's dtype)."""
+    """x [M, K] (row stride free) times w [N, K] transposed -> [M, N] in ``out_dtype`` (default: x's dtype).
+    x may be a ``Begun`` norm."""
     out_dtype = out_dtype or x.dtype
     if x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16:
         from ..kernels import gemm_bf16
         y = gemm_bf16.try_linear(x, w, out_dtype, out)
         if y is not None:
             return y
-    return ops.gemm_generic(x, w, out_dtype, out)
+    return ops.gemm_generic(as_tensor(x), w, out_dtype, out)
 
 
-def linear_delta(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """A product whose result is only ever added to the residual stream by ``Norm.add_norm``.
+def linear_delta(x, w: torch.Tensor, sink: Optional[ResidualSink] = None):
+    """A product whose result is only ever added to the residual stream.
 
-    For few rows it comes back as float32 planes [slices, M, N] of a K-split product, which ``add_norm`` sums:
-    the split keeps the whole GPU busy on a small product and costs no extra kernel.
+    With a ``sink`` whose norm can, the product adds itself to the residual rows and begins that norm: the result
+    is then a ``Begun`` norm, not a delta, and the caller hands it on as it is.  Otherwise the delta comes back for
+    ``Norm.add_norm``: for few rows as float32 planes [slices, M, N] of a K-split product, which ``add_norm`` sums
+    (the split keeps the whole GPU busy on a small product and costs no extra kernel).
     """
+    if sink is not None:
+        y = sink.norm.add_product(sink.resid, x, w)
+        if y is not None:
+            return y
+    x = as_tensor(x)
     if x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16:
         from ..kernels import gemm_bf16
         y = gemm_bf16.linear_planes(x, w)

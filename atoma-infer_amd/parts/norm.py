@@ -35,5 +35,22 @@ class RMSNorm(Norm):
     def add_norm(self, resid, delta, rows=None):
         return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.act_dtype, rows)
 
+    # the norm begun by its neighbours (bfloat16 steps of at most 16 rows): see kernels/gemm_bf16.py
+    def add_product(self, resid, x, w):
+        if self.act_dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16:
+            return None
+        from ..kernels import gemm_bf16
+        y = gemm_bf16.try_linear_resid(x, w, resid, self.weight, self.eps)
+        if y is not None:
+            y.norm = self
+        return y
+
+    def embed(self, table, tokens):
+        if self.act_dtype is not torch.bfloat16 or tokens.numel() > 16 or table.shape[1] != self.width:
+            return None
+        from ..kernels.gemm_bf16 import Begun
+        resid, u, ss = ops.embed_begin_norm(tokens, table, self.weight)
+        return resid, Begun(u, ss, self.eps, self.width, self)
+
 
 register_norm("rmsnorm", RMSNorm)

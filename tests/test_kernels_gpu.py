@@ -546,6 +546,102 @@ def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
                                      hd) is None   # too many rows
 
 
+def _rms(x, g, eps):
+    x = x.double()
+    return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * g.double()
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 16])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (96, 64), (200, 96), (3072, 512)])
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+def test_product_into_the_residual_begins_the_norm(m, n, k, gdt):
+    """``resid += x w^T`` with the following RMSNorm begun in the product's epilogue (residual times norm weight and
+    the rows' sums of squares in shares), against the product, the sum and the norm done apart in float64; then the
+    begun norm finished as a tensor, and finished inside plain, SiLU-multiply and rotary products."""
+    from atoma_infer_amd.kernels import gemm_bf16
+    eps = 1e-5
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    resid0 = rnd(m, n, dtype=torch.float32, seed=3)
+    gamma = (1 + 0.1 * rnd(n, dtype=torch.float32, seed=4)).to(gdt)
+    resid = resid0.clone()
+    b = gemm_bf16.try_linear_resid(x, w, resid, gamma, eps)
+    assert b is not None and b.shares.shape[1] == 16
+    want_resid = resid0.double().cpu() + x.double().cpu() @ w.double().cpu().T
+    assert (resid.double().cpu() - want_resid).abs().max() <= 1e-5 * want_resid.abs().max()
+    want_u = want_resid * gamma.double().cpu()
+    assert (b.data.double().cpu() - want_u).abs().max() <= 1e-2 * want_u.abs().max()
+    ss = b.shares.double().cpu().sum(0)
+    assert torch.allclose(ss[:m], want_resid.pow(2).sum(-1), rtol=1e-5)
+    assert float(ss[m:].abs().sum()) == 0.0
+    want_normed = _rms(want_resid, gamma.cpu(), eps)
+    got = b.tensor()
+    assert got.dtype is torch.bfloat16
+    assert (got.double().cpu() - want_normed).abs().max() <= 1.2e-2 * want_normed.abs().max()
+    # finished inside the products that read it: float32 sums of the normed rows
+    w2 = rnd(72, n, dtype=torch.bfloat16, seed=5)
+    if n % 32 == 0:
+        y = gemm_bf16.try_linear(b, w2, torch.float32)
+        exact = b.data.double().cpu() / torch.sqrt(want_resid.pow(2).mean(-1, keepdim=True) + eps)   # same bf16 rows
+        want_y = exact @ w2.double().cpu().T
+        assert (y.double().cpu() - want_y).abs().max() <= 1e-5 * want_y.abs().max()
+        # a second product into the residual whose rows are the begun norm
+        resid2 = resid.clone()
+        b2 = gemm_bf16.try_linear_resid(b, rnd(n, n, dtype=torch.bfloat16, seed=6, scale=0.05), resid2, gamma, eps)
+        want2 = resid.double().cpu() + exact @ rnd(n, n, dtype=torch.bfloat16, seed=6, scale=0.05).double().cpu().T
+        assert (resid2.double().cpu() - want2).abs().max() <= 1e-5 * want2.abs().max()
+        assert torch.allclose(b2.shares.double().cpu().sum(0)[:m], want2.pow(2).sum(-1), rtol=1e-5)
+
+
+@pytest.mark.parametrize("m", [1, 8, 13])
+def test_begun_norms_are_finished_by_the_fused_products(m):
+    from atoma_infer_amd.kernels import gemm_bf16, ops
+    from atoma_infer_amd.cache.layout import pack_keys, pack_values
+    eps, width = 1e-6, 256
+    table = rnd(50, width, dtype=torch.bfloat16, seed=1)
+    gamma = (1 + 0.1 * rnd(width, dtype=torch.float32, seed=2)).bfloat16()
+    tokens = torch.randint(0, 50, (m,), generator=torch.Generator().manual_seed(3)).int().to(DEV)
+    resid, u, ss = ops.embed_begin_norm(tokens, table, gamma)
+    rows = table[tokens.long()].double().cpu()
+    assert torch.equal(resid.cpu(), rows.float())
+    assert torch.allclose(ss.double().cpu()[0, :m], rows.pow(2).sum(-1), rtol=1e-6)
+    b = gemm_bf16.Begun(u, ss, eps, width)
+    normed = b.tensor()                      # bfloat16 rows of the finished norm
+    want = _rms(rows, gamma.cpu(), eps)
+    assert (normed.double().cpu() - want).abs().max() <= 1.2e-2 * want.abs().max()
+    exact = u.double().cpu() / torch.sqrt(rows.pow(2).mean(-1, keepdim=True) + eps)
+    # SiLU-multiply epilogue
+    inter = 160
+    wg, wu = rnd(inter, width, dtype=torch.bfloat16, seed=4, scale=0.1), rnd(inter, width, dtype=torch.bfloat16, seed=5, scale=0.1)
+    out = gemm_bf16.try_linear_swiglu(b, interleave16(wg, wu))
+    g, up = exact @ wg.double().cpu().T, exact @ wu.double().cpu().T
+    want = torch.nn.functional.silu(g) * up
+    assert (out.double().cpu() - want).abs().max() <= 1e-2 * want.abs().max()
+    # rotary epilogue with the cache write
+    nh, nkv, hd, page, pages = 4, 2, 32, 16, 4
+    w = rnd((nh + 2 * nkv) * hd, width, dtype=torch.bfloat16, seed=6, scale=0.2)
+    gen = torch.Generator().manual_seed(7)
+    pos = torch.randint(0, 60, (m,), generator=gen).int().to(DEV)
+    slots = torch.randperm(pages * page, generator=gen)[:m].int().to(DEV)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))
+    ang = torch.arange(64).float()[:, None] * inv[None]
+    cos, sin = torch.cos(ang).to(DEV), torch.sin(ang).to(DEV)
+
+    def caches():
+        gg = torch.Generator().manual_seed(9)
+        return (pack_keys(torch.randn(pages, nkv, page, hd, generator=gg).bfloat16()).to(DEV),
+                pack_values(torch.randn(pages, nkv, hd, page, generator=gg).bfloat16()).to(DEV))
+    kc1, vc1 = caches()
+    q1 = gemm_bf16.try_linear_rope(b, w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv, hd, always=True)
+    kc2, vc2 = caches()
+    qkv = (exact @ w.double().cpu().T).float().to(DEV)
+    kc2f, vc2f = kc2.float(), vc2.float()
+    q2 = torch.empty(m, nh * hd, dtype=torch.float32, device=DEV)
+    ops.rope_cache_write(qkv, pos, cos, sin, hd, kc2f, vc2f, slots, page, nh, nkv, hd, q2)
+    assert (q1.float() - q2).abs().max() <= 1e-2 * q2.abs().max()
+    assert (kc1.float() - kc2f).abs().max() <= 1e-2 * kc2f.abs().max()
+    assert (vc1.float() - vc2f).abs().max() <= 1e-2 * vc2f.abs().max()
+
+
 @pytest.mark.parametrize("m,n,k,cdt", [(40, 2048, 8192, torch.bfloat16), (64, 16384, 2048, torch.bfloat16),
                                        (48, 40000, 2048, torch.float32), (64, 3072, 2048, torch.bfloat16)])
 def test_products_replay_in_graphs(m, n, k, cdt):
