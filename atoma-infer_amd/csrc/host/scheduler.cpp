@@ -52,6 +52,7 @@ struct Sched {
   void* cm = nullptr;
   int max_tokens = 0, max_seqs = 0, max_model_len = 0, chunked = 1, max_chunk = 0;
   bool windowed = false;  // some cache group keeps a window of keys only
+  int chunk_align = 1;    // where a prompt may be cut
   double delay_factor = 0.0;
   std::deque<int64_t> waiting;
   std::vector<int64_t> running;
@@ -69,11 +70,19 @@ struct Sched {
     return s;
   }
 
+  // A portion that does not end what the request holds ends at a multiple of chunk_align (a mixer that scans its
+  // tokens in blocks asks for that); 0 if no such portion of at most n tokens exists.
+  int aligned(const Req& r, int n) const {
+    if (chunk_align <= 1 || n >= r.uncomputed()) return n;
+    const int end = (r.computed + n) / chunk_align * chunk_align;
+    return end > r.computed ? end - r.computed : 0;
+  }
+
   int chunk(const Req& r, int budget) const {
     int n = std::min(r.uncomputed(), budget);
     if (max_chunk > 0 && r.uncomputed() > 1) n = std::min(n, max_chunk);
     if (!chunked && n < r.uncomputed()) return 0;  // prompts are not cut: wait for a step with room for all of it
-    return n;
+    return aligned(r, n);
   }
 
   void release(int64_t uid) {
@@ -156,8 +165,9 @@ struct Sched {
         // A shorter portion may still find its pages: when nothing else could give any back, and, with a window
         // of keys, always (pages come back as the request moves on, so a portion too long for what is free now
         // is no reason to throw away what another request has computed).
-        if (n > 1 && chunked && (alone || windowed)) {
-          n /= 2;
+        const int shorter = n > 1 ? aligned(r, n / 2) : 0;
+        if (shorter > 0 && chunked && (alone || windowed)) {
+          n = shorter;
           continue;
         }
         if (alone) {
@@ -192,8 +202,8 @@ struct Sched {
         // If nothing holds pages, waiting frees none: only a shorter first portion helps (a prompt longer than
         // the pool gets in through a window of keys); when one token finds no page the request can never run.
         const bool pool_is_idle = cm_num_requests(cm) == 0;
-        while (n > 1 && chunked && pool_is_idle && !cm_can_admit(cm, r.length, n)) n /= 2;
-        if (!cm_can_admit(cm, r.length, n)) {
+        while (n > 1 && chunked && pool_is_idle && !cm_can_admit(cm, r.length, n)) n = aligned(r, n / 2);
+        if (n <= 0 || !cm_can_admit(cm, r.length, n)) {
           if (!pool_is_idle) break;  // later
           waiting.pop_front();
           ignored.push_back(r.uid);
@@ -226,8 +236,12 @@ int copy_out(const std::vector<int64_t>& v, int64_t* out, int cap) {
 extern "C" {
 
 void* sc_create(void* cache_manager, int max_tokens, int max_seqs, int max_model_len, int chunked, int max_chunk,
-                double delay_factor) {
-  if (!cache_manager || max_tokens <= 0 || max_seqs <= 0 || max_model_len <= 0 || max_chunk < 0) return nullptr;
+                double delay_factor, int chunk_align) {
+  if (!cache_manager || max_tokens <= 0 || max_seqs <= 0 || max_model_len <= 0 || max_chunk < 0 || chunk_align <= 0)
+    return nullptr;
+  // a cut prompt needs room for one aligned portion
+  if (chunked && chunk_align > 1 && (max_tokens < chunk_align || (max_chunk > 0 && max_chunk < chunk_align)))
+    return nullptr;
   Sched* s = new Sched();
   s->cm = cache_manager;
   s->max_tokens = max_tokens;
@@ -237,6 +251,7 @@ void* sc_create(void* cache_manager, int max_tokens, int max_seqs, int max_model
   s->max_chunk = max_chunk;
   s->delay_factor = delay_factor;
   s->windowed = cm_has_window(cache_manager) != 0;
+  s->chunk_align = chunk_align;
   return s;
 }
 

@@ -35,7 +35,6 @@ constexpr int DTILES = (HD + 31) / 32; // 32-row tiles of O^T
 constexpr int PAGE = 16;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kSlack = 8.0f;   // see the softmax in the kernel
-constexpr int kCUs = 256;        // MI355X
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -455,6 +454,19 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
 constexpr bool kSplit2Fits = (DTILES * 16 + 2) * 64 * 4 * sizeof(float) <= 65536;
 constexpr bool kSplit8Fits = (DTILES * 16 + 2) * 64 * 7 * sizeof(float) <= 65536;
 
+// compute units of the current device, asked for once per device
+static int compute_units() {
+  static int cus[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return cus[dev];
+}
+
 extern "C" int atoma_attention_mfma_head_size() { return HD; }
 extern "C" int atoma_attention_mfma_max_ksplit() { return kSplit8Fits ? 8 : kSplit2Fits ? 2 : 1; }
 
@@ -482,7 +494,7 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
   else if (ksplit == 8 && kSplit8Fits) {
     // more workgroups than CUs: two of them to a CU finish sooner than two rounds of one (measured; with fewer,
     // the loads in flight during the softmax count for more)
-    if ((long long)n_tasks * nkv > kCUs) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), true);
+    if ((long long)n_tasks * nkv > compute_units()) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), true);
     else ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1));
   }
   else return ATOMA_ERR_SHAPE;

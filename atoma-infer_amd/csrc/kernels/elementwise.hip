@@ -137,22 +137,16 @@ extern "C" int atoma_embed_begin_norm(const int32_t* tokens, const void* table, 
 }
 
 // out [T][width] = u [T][width] / sqrt(sum_p ss[p][row] / width + eps), both bfloat16: the finished norm as a tensor,
-// for a reader that cannot finish it itself.  The shares are added in the order the products add them.
+// for a reader that cannot finish it itself.
 __global__ void __launch_bounds__(256)
 finish_norm_kernel(const uint16_t* __restrict__ u, const float* __restrict__ ss, int parts, float eps,
                    uint16_t* __restrict__ out, int width) {
-  __shared__ float scale_s;
+  __shared__ float scratch[4];
   const int t = blockIdx.x;
-  if (threadIdx.x < 64) {
-    const int kg = threadIdx.x >> 4;
-    float s = 0.f;
-    for (int p = kg; p < parts; p += 4) s += ss[p * 16 + t];
-    s += __shfl_xor(s, 16, 64);
-    s += __shfl_xor(s, 32, 64);
-    if (threadIdx.x == 0) scale_s = 1.0f / sqrtf(s / (float)width + eps);
-  }
-  __syncthreads();
-  const float scale = scale_s;
+  float s = 0.f;
+  for (int p = threadIdx.x; p < parts; p += 256) s += ss[(size_t)p * 16 + t];
+  s = block_sum<4>(s, scratch);
+  const float scale = 1.0f / sqrtf(s / (float)width + eps);
   for (int i = threadIdx.x; i < width; i += 256)
     out[(size_t)t * width + i] = f32_to_bf16_bits(bf16_bits_to_f32(u[(size_t)t * width + i]) * scale);
 }

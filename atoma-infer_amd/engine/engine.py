@@ -73,7 +73,8 @@ class LlmEngine:
             pages = [min(p, cap) for p in pages]
         pool = CachePool(plan, page, pages, self.scheduler_config.max_num_sequences, cache_dtype, self.model.device)
         self.runner = ModelRunner(self.model, pool)
-        self.scheduler = Scheduler(self.scheduler_config, RunnerCache(self.runner))
+        self.scheduler = Scheduler(self.scheduler_config, RunnerCache(self.runner),
+                                   chunk_alignment=spec.chunk_alignment)
         self.sampler = Sampler(self.model.device)
         self.eos_ids = set(spec.eos_token_ids)
         self._next_uid = 0

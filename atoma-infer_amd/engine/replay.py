@@ -19,11 +19,12 @@ from typing import Dict, IO
 
 import torch
 
+from ..cache.manager import OutOfPages
 from ..cache.pool import CachePool, pages_for_tokens, plan_cache
 from ..models.model import load_model
 from .step import ModelRunner, StepEntry
 
-REPLAY_PAGE_SIZE = 16
+REPLAY_PAGE_SIZE = 16       # the engine's default block size ([cache] block_size)
 REPLAY_MAX_LIVE = 16
 
 
@@ -50,9 +51,13 @@ def replay(runner: ModelRunner, lines: IO[str], out_dir: str, report: IO[str] = 
         for e in obj.get("entries", []):
             name = str(e["id"])
             if name not in ids:
+                try:
+                    runner.add_request(next_id)
+                except OutOfPages:
+                    raise SystemExit(f"trace_run: step {step} brings request '{name}' while {len(ids)} others are "
+                                     f"live, which is all that --max-live allows") from None
                 ids[name] = next_id
                 next_id += 1
-                runner.add_request(ids[name])
             rid = ids[name]
             entries.append(StepEntry(rid, [int(t) for t in e["tokens"]], runner.computed_len(rid),
                                      [int(w) for w in e.get("want", [])]))
@@ -80,8 +85,15 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time (each request rounded up to 64)")
+                    help="most tokens that live requests hold at any time, each request's count rounded up to a "
+                         "multiple of 64 by the caller; the cache pool is made for this many")
+    ap.add_argument("--page-size", type=int, default=REPLAY_PAGE_SIZE,
+                    help=f"tokens a page of the cache (default {REPLAY_PAGE_SIZE}, the engine's [cache] block_size)")
+    ap.add_argument("--max-live", type=int, default=REPLAY_MAX_LIVE,
+                    help=f"most requests live at a time (default {REPLAY_MAX_LIVE})")
     args = ap.parse_args(argv)
+    if args.page_size <= 0 or args.max_live <= 0 or args.max_tokens <= 0:
+        ap.error("--max-tokens, --page-size and --max-live must be positive")
     print(f"[trace_run] loading {args.model} ({args.dtype})", file=sys.stderr, flush=True)
-    runner = make_runner(args.model, args.dtype, args.max_tokens)
+    runner = make_runner(args.model, args.dtype, args.max_tokens, args.page_size, args.max_live)
     return replay(runner, sys.stdin, args.out)

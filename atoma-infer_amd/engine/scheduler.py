@@ -79,7 +79,7 @@ def _native():
         lib = load_host_library()
         p, i, i64, f64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_double
         lib.sc_create.restype = p
-        lib.sc_create.argtypes = [p, i, i, i, i, i, f64]
+        lib.sc_create.argtypes = [p, i, i, i, i, i, f64, i]
         lib.sc_destroy.restype = None
         lib.sc_destroy.argtypes = [p]
         lib.sc_add.argtypes = [p, i64, f64, ctypes.c_int32]
@@ -101,15 +101,17 @@ class Scheduler:
     draws pages from).  If it has ``adopted(request)`` and ``forgot(request)``, they are called for every request
     that a plan registered with the manager or released from it, so that books kept beside the manager follow."""
 
-    def __init__(self, config: SchedulerConfig, cache: CacheManager, clock=time.monotonic):
+    def __init__(self, config: SchedulerConfig, cache: CacheManager, clock=time.monotonic, chunk_alignment: int = 1):
+        """``chunk_alignment``: a portion that does not end a request's tokens ends at a multiple of it (what the
+        model asks for, ``ModelSpec.chunk_alignment``)."""
         config.validate()
         self.config, self.cache, self.clock = config, cache, clock
         self._lib = _native()
         self._h = self._lib.sc_create(cache.handle, config.max_num_batched_tokens, config.max_num_sequences,
                                       config.max_model_len, int(config.enable_chunked_prefill),
-                                      config.max_prefill_chunk, float(config.delay_factor))
+                                      config.max_prefill_chunk, float(config.delay_factor), int(chunk_alignment))
         if not self._h:
-            raise SchedulerError(f"the native scheduler refused {config}")
+            raise SchedulerError(f"the native scheduler refused {config} with portions aligned to {chunk_alignment}")
         self._requests: Dict[int, Request] = {}
         self._running: Dict[int, Request] = {}
         self._adopted = getattr(cache, "adopted", None)

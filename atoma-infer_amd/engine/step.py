@@ -246,7 +246,9 @@ class ModelRunner:
         plan_bucket = bucket
         if plan_bucket is None and int(counts.max()) == 1:
             plan_bucket = -(-max_seq // DECODE_BUCKET)
-        extras = [(key, *fn(starts, counts, plan_bucket)) for key, fn in self._planners.items()]
+        # (planners are told the context length that the bucket serves, in tokens)
+        bucket_tokens = None if plan_bucket is None else plan_bucket * DECODE_BUCKET
+        extras = [(key, *fn(starts, counts, bucket_tokens)) for key, fn in self._planners.items()]
         # layout of the one staging buffer
         o_tok, o_pos, o_seq = 0, t, 2 * t
         o_qs, o_len, o_slot = 3 * t, 3 * t + s + 1, 3 * t + 2 * s + 1

@@ -59,7 +59,7 @@ WHOLE_MIN_PAIRS = 128
 LONG_KEYS = 16384
 
 
-def chunk_for(n_split: int, max_keys: int, kv_heads: int = 8, whole_ok: bool = False) -> Tuple[int, int]:
+def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False) -> Tuple[int, int]:
     """(keys per partial task, waves that share a task) for the entries of a step that are split along their keys;
     keys per task 0 means all of them: with ``whole_ok`` (a decode step, head size that allows eight waves) and
     enough (request, KV head) pairs to occupy the GPU, eight waves walk all keys of a pair and merge in LDS, which
@@ -104,10 +104,10 @@ def _live_pieces(rows: int, qt: int, live_tokens: int):
     return out
 
 
-def _chunk_slots(bucket: int, chunk: int, window: int) -> int:
+def _chunk_slots(bucket_keys: int, chunk: int, window: int) -> int:
     """Partial results that a decoded token of a graph's bucket owns: one per chunk of the bucket's keys, or, with
     a window, per chunk that a window can touch wherever it lies (its first chunk is then slot 0)."""
-    slots = -(-(bucket * CHUNK) // chunk)
+    slots = -(-bucket_keys // chunk)
     if window > 0:
         slots = min(slots, -(-window // chunk) + 1)
     return slots
@@ -155,16 +155,18 @@ def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, windo
     return lengths, t.reshape(tiles * fours, 4, 12)
 
 
-def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket: Optional[int] = None,
-                vectorized: bool = True, kv_heads: int = 8, max_waves: int = 2,
+def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket_keys: Optional[int] = None,
+                vectorized: bool = True, *, kv_heads: int, max_waves: int = 2,
                 ) -> Tuple[np.ndarray, Tuple[int, int, int, int]]:
     """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials, waves that
     share a task: two when a prompt tile walks many keys, else what ``chunk_for`` says for the split entries).
 
     Main tasks are padded to a multiple of 4 (one workgroup runs 4) and ordered so that tasks sharing keys are
-    neighbours and long tasks come first.  With ``bucket`` (decode graphs: one token per entry) every entry is
-    split and owns ``bucket`` chunk slots, used or not, so all counts depend on (entries, bucket) alone.
+    neighbours and long tasks come first.  With ``bucket_keys`` (decode steps: one token per entry; the context
+    length that the step's graph serves, in tokens) every entry is split and owns the chunk slots of that many keys,
+    used or not, so all counts depend on (entries, bucket_keys) alone.
     """
+    bucket = bucket_keys
     if vectorized and bucket is not None and len(counts) and int(counts.max()) == 1:
         return _build_decode_tasks(starts, group, window, bucket, kv_heads, max_waves)
     qt_max = max(1, 128 // group)
@@ -182,7 +184,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     split_entries = [e for e in range(len(starts)) if splits(e)]
     chunk, waves = CHUNK, 1
     if split_entries:
-        most = bucket * CHUNK if bucket is not None else max(int(starts[e]) + int(counts[e]) for e in split_entries)
+        most = bucket if bucket is not None else max(int(starts[e]) + int(counts[e]) for e in split_entries)
         if bucket is not None and window > 0:
             most = min(most, window + CHUNK)
         chunk, waves = chunk_for(len(split_entries), most, kv_heads)
@@ -239,7 +241,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     return arr, (len(head) + len(split), len(combine), n_part, waves)
 
 
-def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int, kv_heads: int = 8,
+def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int, kv_heads: int,
                         max_waves: int = 2):
     """``build_tasks`` for a step in which every entry brings one token, without a Python loop over entries."""
     s = len(starts)
@@ -248,7 +250,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     lo = np.maximum(0, starts - window + 1) if window > 0 else np.zeros(s, dtype=np.int64)
     row_chunks = -(-group // 32)
     # the bucket, not the step's longest request, decides between whole ranges and chunks: a graph holds one of them
-    keys = bucket * CHUNK if window <= 0 else min(bucket * CHUNK, window + CHUNK)      # what a token can see
+    keys = bucket if window <= 0 else min(bucket, window + CHUNK)      # what a token can see
     chunk, waves = chunk_for(s, keys, kv_heads, whole_ok=max_waves >= 8)
     waves = min(waves, max_waves)
     if chunk == 0:

@@ -31,8 +31,13 @@ class ModelSpec:
     eos_token_ids: Tuple[int, ...] = ()
     #: regular expressions of checkpoint tensors that are neither bound nor an error
     ignorable: Tuple[str, ...] = ()
+    #: where the scheduler may cut a prompt: a portion that does not end the request's tokens ends at a multiple of
+    #: this (1: anywhere; a mixer that scans its tokens in blocks asks for the block length)
+    chunk_alignment: int = 1
 
     def __post_init__(self):
+        if self.chunk_alignment < 1:
+            raise ValueError("chunk_alignment must be at least 1")
         if not self.run_order:
             self.run_order = [LayerCall(i) for i in range(len(self.layers))]
         for pos, call in enumerate(self.run_order):

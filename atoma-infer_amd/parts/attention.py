@@ -79,9 +79,15 @@ class PagedAttention(Mixer):
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
 
     def step_planner(self, page_size: int, cache_dtype: torch.dtype):
-        """(key, fn(starts, counts, bucket) -> (int32 array, meta)): the task list of the MFMA attention kernels,
-        built once per step on the host and shipped with the step's metadata."""
+        """(key, fn(starts, counts, bucket_tokens) -> (int32 array, meta)): the task list of the MFMA attention
+        kernels, built once per step on the host and shipped with the step's metadata.  ``bucket_tokens`` is None, or
+        for a step that only decodes the context length its plan must serve (a multiple of the runner's bucket)."""
         from ..kernels import attention_bf16
+        if cache_dtype is torch.bfloat16 and page_size != attention_bf16.PAGE:
+            import warnings
+            warnings.warn(f"bfloat16 attention with pages of {page_size} tokens runs the general kernel (one wave per "
+                          f"token and head), many times slower than the matrix-core kernel, which needs pages of "
+                          f"{attention_bf16.PAGE} tokens ([cache] block_size = {attention_bf16.PAGE})", stacklevel=2)
         if cache_dtype is not torch.bfloat16 or page_size != attention_bf16.PAGE:
             return None
         group, window, nkv = self.nh // self.nkv, self.window or 0, self.nkv

@@ -147,13 +147,21 @@ class PlainScheduler:
         if self.pages.has(r.uid):
             self.pages.free(r.uid)
 
+    def _aligned(self, r, n):
+        """A portion that does not end the request's tokens ends at a multiple of ``limits.align``; 0 if none fits."""
+        a = getattr(self.limits, "align", 1)
+        if a <= 1 or n >= r.num_uncomputed:
+            return n
+        end = (r.num_computed + n) // a * a
+        return max(end - r.num_computed, 0)
+
     def _portion(self, r, budget):
         n = min(r.num_uncomputed, budget)
         if self.limits.max_portion > 0 and r.num_uncomputed > 1:
             n = min(n, self.limits.max_portion)
         if not self.limits.cut and n < r.num_uncomputed:
             return 0
-        return n
+        return self._aligned(r, n)
 
     def _preempt(self, victim, out):
         self.running.remove(victim)
@@ -194,8 +202,9 @@ class PlainScheduler:
             while not self.pages.can_reserve(r.uid, r.num_computed + n):
                 victim = next((v for v in reversed(self.running) if not v.frozen), r)
                 alone = victim is r and len(self.running) == 1
-                if n > 1 and lim.cut and (alone or self.pages.window):
-                    n //= 2           # a shorter portion may still find its pages
+                shorter = self._aligned(r, n // 2) if n > 1 else 0
+                if shorter > 0 and lim.cut and (alone or self.pages.window):
+                    n = shorter       # a shorter portion may still find its pages
                     continue
                 if alone:
                     self.running.remove(r)
@@ -227,8 +236,8 @@ class PlainScheduler:
                     break
                 idle = self.pages.idle()
                 while n > 1 and lim.cut and idle and not self.pages.can_admit(r.length, n):
-                    n //= 2           # nothing holds pages: only a shorter first portion helps
-                if not self.pages.can_admit(r.length, n):
+                    n = self._aligned(r, n // 2)       # nothing holds pages: only a shorter first portion helps
+                if n <= 0 or not self.pages.can_admit(r.length, n):
                     if not idle:
                         break
                     self.waiting.popleft()

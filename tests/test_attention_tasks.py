@@ -56,7 +56,7 @@ def test_tasks_cover_every_visible_key_once(seed):
     window = int(rng.choice([0, 0, 50, 700]))
     counts = rng.choice([1, 1, 2, 7, 33, 150], size=s).astype(np.int32)
     starts = rng.integers(0, 2500, size=s).astype(np.int32)
-    arr, meta = A.build_tasks(starts, counts, group, window)
+    arr, meta = A.build_tasks(starts, counts, group, window, kv_heads=8)
     coverage(arr, meta, starts, counts, group, window)
 
 
@@ -68,9 +68,9 @@ def test_decode_builder_equals_the_general_one(seed):
     window = int(rng.choice([0, 0, 100, 700]))
     starts = rng.integers(0, 3000, size=s).astype(np.int32)
     counts = np.ones(s, dtype=np.int32)
-    bucket = -(-int(starts.max() + 1) // 256)
-    fast, mf = A.build_tasks(starts, counts, group, window, bucket)
-    slow, ms = A.build_tasks(starts, counts, group, window, bucket, vectorized=False)
+    bucket = -(-int(starts.max() + 1) // 256) * 256
+    fast, mf = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8)
+    slow, ms = A.build_tasks(starts, counts, group, window, bucket, vectorized=False, kv_heads=8)
     assert mf == ms
     # null tasks may differ in their unused fields; compare what the kernels read
     live = fast[:, 0] >= 0
@@ -78,8 +78,8 @@ def test_decode_builder_equals_the_general_one(seed):
     assert np.array_equal(fast[live], slow[live])
     coverage(fast, mf, starts, counts, group, window)
     # sizes depend on (entries, bucket) alone
-    other = rng.integers(0, bucket * 256, size=s).astype(np.int32)
-    assert A.build_tasks(other, counts, group, window, bucket)[1] == mf
+    other = rng.integers(0, bucket, size=s).astype(np.int32)
+    assert A.build_tasks(other, counts, group, window, bucket, kv_heads=8)[1] == mf
 
 
 @pytest.mark.parametrize("seed", range(8))
@@ -90,21 +90,21 @@ def test_long_contexts(seed):
     group, window = int(rng.choice([1, 4, 8])), int(rng.choice([0, 0, 9000]))
     starts = rng.integers(15000, 40000, size=s).astype(np.int32)
     counts = np.ones(s, dtype=np.int32)
-    bucket = -(-int(starts.max() + 1) // 256)
+    bucket = -(-int(starts.max() + 1) // 256) * 256
     fast, mf = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
     slow, ms = A.build_tasks(starts, counts, group, window, bucket, vectorized=False, kv_heads=8, max_waves=8)
     assert mf == ms
     live = fast[:, 0] >= 0
     assert np.array_equal(live, slow[:, 0] >= 0) and np.array_equal(fast[live], slow[live])
     coverage(fast, mf, starts, counts, group, window)
-    seen = min(bucket * 256, window + 256) if window else bucket * 256       # keys a token can see
+    seen = min(bucket, window + 256) if window else bucket       # keys a token can see
     if seen >= A.LONG_KEYS and s * -(-seen // 256) * 8 > 800:
         spans = fast[live][:, 5] - fast[live][:, 4]
         assert int(spans.max()) == 512 and mf[3] == 2
     # a portion of a prompt beside them
     counts2 = counts.copy()
     counts2[0] = 40
-    arr, meta = A.build_tasks(starts, counts2, group, window)
+    arr, meta = A.build_tasks(starts, counts2, group, window, kv_heads=8)
     coverage(arr, meta, starts, counts2, group, window)
 
 
@@ -117,7 +117,7 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     group, window = int(rng.choice([1, 4, 8])), int(rng.choice([0, 0, 300]))
     starts = rng.integers(0, 3000, size=s).astype(np.int32)
     counts = np.ones(s, dtype=np.int32)
-    bucket = -(-int(starts.max() + 1) // 256)
+    bucket = -(-int(starts.max() + 1) // 256) * 256
     arr, meta = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
     assert meta == (s * -(-group // 32), 0, 0, 8)
     coverage(arr, meta, starts, counts, group, window)
@@ -137,8 +137,8 @@ def test_tile_builder_equals_the_general_one(seed):
     window = int(rng.choice([0, 0, 50, 700]))
     counts = rng.choice([1, 1, 2, 7, 33, 150, 600], size=s).astype(np.int32)
     starts = rng.integers(0, 2500, size=s).astype(np.int32)
-    fast, mf = A.build_tasks(starts, counts, group, window)
-    slow, ms = A.build_tasks(starts, counts, group, window, vectorized=False)
+    fast, mf = A.build_tasks(starts, counts, group, window, kv_heads=8)
+    slow, ms = A.build_tasks(starts, counts, group, window, vectorized=False, kv_heads=8)
     assert mf[1:] == ms[1:]
     live = lambda arr, meta: sorted(map(tuple, arr[:meta[0]][arr[:meta[0], 0] >= 0].tolist()))
     assert live(fast, mf) == live(slow, ms)
@@ -151,7 +151,7 @@ def test_a_window_far_into_a_context_owns_few_slots():
     not for every chunk of its context."""
     starts = np.asarray([100_000, 70_001, 5], dtype=np.int32)
     counts = np.ones(3, dtype=np.int32)
-    bucket = -(-100_001 // 256)
+    bucket = -(-100_001 // 256) * 256
     for builder in (True, False):
         arr, meta = A.build_tasks(starts, counts, 4, 1000, bucket, vectorized=builder, kv_heads=8, max_waves=2)
         coverage(arr, meta, starts, counts, 4, 1000)

@@ -189,6 +189,13 @@ def test_mixed_batches_with_few_pages(model_dirs, name, dtype):
     assert runner.manager.num_free_pages(0) == need and runner.manager.num_requests() == 0
 
 
+def test_pages_the_matrix_core_attention_refuses_are_announced(model_dirs):
+    """bfloat16 with pages of 4 tokens is right (the tests above run it) but takes the general attention kernel:
+    building the runner says so once."""
+    with pytest.warns(UserWarning, match="general kernel"):
+        make_runner(model_dirs["A"], "bfloat16", 4, 8)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_first_tokens_and_long_decoding(model_dirs, dtype):
     """A one-token prompt, then everything decoded token by token up to the model's last position."""

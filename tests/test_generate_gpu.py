@@ -93,18 +93,22 @@ def test_cache_option_sliding_window(model_dirs, dtype):
         if dtype == "float32":
             assert got == plain_llama.greedy_generate(p, 30, w, cfg)
         else:
-            # bfloat16 may turn a near tie: every token must be among the plain model's best few given the same past
-            seq = list(p)
-            for tok in got:
-                logits = plain_llama.forward(seq, w, cfg)[-1]
-                assert logits[tok] >= logits.max() - 0.05 * (logits.max() - logits.min())
-                seq.append(tok)
-    # all keys again without the option: other tokens (the window does change what is computed)
-    full = LlmEngine(d, "float32", cache=CacheConfig(block_size=16, num_gpu_blocks_override=40),
+            # bfloat16 may turn a near tie: every token and its logit against the plain windowed model on the same past
+            check_greedy_tokens(p, got, o.inference_outputs[0].logprobs, w, cfg, TOL_BF16)
+    # all keys again without the option: the plain model without a window, and other tokens and logits than with it
+    # (the window does change what is computed, in either dtype)
+    full = LlmEngine(d, dtype, cache=CacheConfig(block_size=16, num_gpu_blocks_override=40),
                      scheduler=SchedulerConfig(max_num_batched_tokens=32, max_num_sequences=2, max_model_len=400))
     outs_full = full.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=30, ignore_eos_token=True))
-    assert [o.inference_outputs[0].token_ids for o in outs_full] == \
-        [plain_llama.greedy_generate(p, 30, w, plain_config(d)) for p in prompts]
+    for p, o, ow in zip(prompts, outs_full, outs):
+        check_greedy_tokens(p, o.inference_outputs[0].token_ids, o.inference_outputs[0].logprobs, w, plain_config(d),
+                            TOL_F32 * 10 if dtype == "float32" else TOL_BF16)
+        first_full, first_win = o.inference_outputs[0].logprobs[0], ow.inference_outputs[0].logprobs[0]
+        assert o.inference_outputs[0].token_ids != ow.inference_outputs[0].token_ids or \
+            abs(first_full - first_win) > 1e-3 * abs(first_full), "the window changed nothing"
+    if dtype == "float32":
+        assert [o.inference_outputs[0].token_ids for o in outs_full] == \
+            [plain_llama.greedy_generate(p, 30, w, plain_config(d)) for p in prompts]
 
 
 def test_tiny_b_workload_portions_beside_decodes_with_temperature(model_dirs):
@@ -285,15 +289,48 @@ def test_repeat_penalty_kernel_and_temperature_limit():
 # bin/trace_run as a program
 
 
-def run_trace(model_dir, dtype, steps, out_dir, max_tokens):
+def run_trace(model_dir, dtype, steps, out_dir, max_tokens, extra=(), ok=True):
     env = dict(os.environ)
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype",
-                           dtype, "--out", out_dir, "--max-tokens", str(max_tokens)],
+                           dtype, "--out", out_dir, "--max-tokens", str(max_tokens), *extra],
                           input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
                           env=env, timeout=300)
+    if not ok:
+        return proc
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
     return proc
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_with_pages_of_four_tokens(model_dirs, tmp_path, dtype):
+    """Tiny A with its own block size of 4 through the program's --page-size, three requests with two live at a time
+    in a pool of 128 tokens; then a third live request beyond --max-live ends the program with a clear message."""
+    d = model_dirs["A"]
+    vocab = TINY["A"]["vocab_size"]
+    a, b, c = random_tokens(50, vocab, 1), random_tokens(9, vocab, 2), random_tokens(30, vocab, 3)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:21], "want": [20]}, {"id": "b", "tokens": b[:5], "want": [4]}],
+         "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[5:], "want": [3]}, {"id": "a", "tokens": a[21:], "want": [0, 28]}],
+         "end": ["b"]},
+        {"step": 2, "entries": [{"id": "c", "tokens": c[:2], "want": [1]}], "end": ["a"]},
+        {"step": 3, "entries": [{"id": "c", "tokens": c[2:], "want": [27]}], "end": ["c"]},
+    ]
+    out = str(tmp_path / "out")
+    run_trace(d, dtype, steps, out, 128, extra=("--page-size", "4", "--max-live", "2"))
+    w, cfg = plain_weights(d), plain_config(d)
+    pa, pb, pc = (plain_llama.forward(t, w, cfg) for t in (a, b, c))
+    want = {0: torch.stack([pa[20], pb[4]]), 1: torch.stack([pb[8], pa[21], pa[49]]), 2: pc[1][None], 3: pc[29][None]}
+    for step, ref in want.items():
+        got = torch.from_numpy(np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, vocab))
+        assert got.shape == ref.shape
+        assert (rel_err(got, ref) < TOL_F32) if dtype == "float32" else (frob_err(got, ref) < TOL_BF16)
+    if dtype == "float32":
+        crowd = [{"step": 0, "entries": [{"id": n, "tokens": a[:3], "want": []} for n in ("x", "y", "z")], "end": []}]
+        proc = run_trace(d, dtype, crowd, str(tmp_path / "out2"), 128, extra=("--page-size", "4", "--max-live", "2"),
+                         ok=False)
+        assert proc.returncode != 0 and "--max-live" in proc.stderr and "Traceback" not in proc.stderr
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -683,7 +683,7 @@ def test_attention_whole_ranges_with_eight_waves(window, more):
     q = (torch.randn(len(starts), (nh + 2 * nkv) * hd, generator=g) * 1.5).bfloat16().to(DEV)
     out = torch.empty(len(starts), nh * hd, dtype=torch.bfloat16, device=DEV)
     ctx, cache = FakeCtx(starts, counts), FakeCache(bt, page)
-    bucket = -(-max(lens) // 256)
+    bucket = -(-max(lens) // 256) * 256
     arr, meta = A.build_tasks(ctx.h_starts, ctx.h_counts, nh // nkv, window, bucket, kv_heads=nkv, max_waves=8)
     assert meta[1:] == (0, 0, 8)
     ctx.plans = {A.plan_key(nh // nkv, window, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
@@ -741,7 +741,7 @@ def test_decode_plans_with_large_groups(nh, nkv, hd, whole, monkeypatch):
     out = torch.full((t, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
     ctx = FakeCtx(starts, counts)
     arr, meta = attention_bf16.build_tasks(np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32),
-                                           group, 0, 3, kv_heads=nkv, max_waves=attention_bf16.max_waves_for(hd))
+                                           group, 0, 3 * 256, kv_heads=nkv, max_waves=attention_bf16.max_waves_for(hd))
     assert (meta[1] == 0) == whole                       # no merge records with whole ranges
     ctx.plans = {attention_bf16.plan_key(group, 0, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
     scale = 1.0 / math.sqrt(hd)
@@ -771,7 +771,7 @@ def test_decode_plans_behind_a_window(window):
     qkv = (torch.randn(t, (nh + 2 * nkv) * hd, generator=g) * 1.5).bfloat16().to(DEV)
     out = torch.full((t, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
     ctx = FakeCtx(starts, counts)
-    bucket = -(-(max(starts) + 1) // 256)
+    bucket = -(-(max(starts) + 1) // 256) * 256
     arr, meta = attention_bf16.build_tasks(np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32),
                                            nh // nkv, window, bucket, kv_heads=nkv,
                                            max_waves=attention_bf16.max_waves_for(hd))

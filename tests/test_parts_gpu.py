@@ -213,8 +213,11 @@ def _toy_parts():
     class DecayMixer(Mixer):
         """state <- decay * state + x W_in (per token, in order); y = state W_out.  State: [inner] per request."""
 
-        def __init__(self, width: int, inner: int, decay: float):
-            self.width, self.inner, self.decay = width, inner, decay
+        #: (start, tokens) of every entry a mixer with ``align`` > 1 has seen
+        seen = []
+
+        def __init__(self, width: int, inner: int, decay: float, align: int = 1):
+            self.width, self.inner, self.decay, self.align = width, inner, decay, align
 
         def weight_specs(self):
             return {"in_proj.weight": WeightSpec((self.inner, self.width)),
@@ -235,6 +238,10 @@ def _toy_parts():
             row = 0
             for e in range(ctx.n_entries):
                 slot, n = int(ctx.h_state_slots[e]), int(ctx.h_counts[e])
+                if self.align > 1:
+                    # a mixer that scans its tokens in blocks: portions of several tokens must start on a block
+                    assert n == 1 or int(ctx.h_starts[e]) % self.align == 0, (int(ctx.h_starts[e]), n)
+                    DecayMixer.seen.append((int(ctx.h_starts[e]), n))
                 st = cache.state[slot]
                 for i in range(n):
                     st.mul_(self.decay).add_(u[row + i])
@@ -321,6 +328,7 @@ def _toy_architecture():
         max_positions: int = key(convert=as_positive_int)
         layers: tuple = key(convert=lambda v: tuple(dict(x) for x in v))
         order: tuple = key(convert=lambda v: tuple(dict(x) for x in v))
+        align: int = key(convert=as_positive_int, default=1)
 
         def to_dict(self):
             d = {f.name: getattr(self, f.name) for f in dataclasses.fields(self)}
@@ -341,7 +349,8 @@ def _toy_architecture():
                 mixer = make_part("mixer", "attention", width=cfg.width, num_heads=cfg.heads,
                                   num_kv_heads=cfg.kv_heads, head_size=hd, position=pos, window=ld.get("window"))
             else:
-                mixer = make_part("mixer", "toy_decay", width=cfg.width, inner=ld["inner"], decay=ld["decay"])
+                mixer = make_part("mixer", "toy_decay", width=cfg.width, inner=ld["inner"], decay=ld["decay"],
+                                  align=cfg.align)
             if "experts" in ld:
                 ffn = make_part("feed_forward", "toy_routed", width=cfg.width, inter=ld["expert_inter"],
                                 experts=ld["experts"], top=ld["top"])
@@ -357,7 +366,8 @@ def _toy_architecture():
                          embedding=("toy.embed", emb), layers=layers,
                          final_norm=("toy.final_norm", make_part("norm", "rmsnorm", width=cfg.width, eps=cfg.eps)),
                          head=("toy.head", OutputHead(cfg.width, cfg.vocab)),
-                         run_order=[LayerCall(o["layer"], o.get("kv_from")) for o in cfg.order])
+                         run_order=[LayerCall(o["layer"], o.get("kv_from")) for o in cfg.order],
+                         chunk_alignment=cfg.align)
 
     register_architecture("ToyMixedForCausalLM", ToyConfig, build, replace=True)
 
@@ -584,6 +594,39 @@ def test_toy_architecture_generates_through_the_engine(toy_dir):
                     scheduler=SchedulerConfig(max_num_batched_tokens=8, max_num_sequences=2, max_model_len=64))
     outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=5, ignore_eos_token=True))
     assert [o.inference_outputs[0].token_ids for o in outs] == want
+
+
+def test_prompts_are_cut_where_the_model_allows(tmp_path):
+    """The toy model with ``chunk_alignment`` 8 (its state mixer asserts that portions of several tokens start on a
+    multiple of 8): prompts of 45 and 30 tokens under a budget of 21 tokens a step, a pool so small that one request
+    is preempted and computed again, against the plain model."""
+    from atoma_infer_amd.config import CacheConfig, SchedulerConfig
+    from atoma_infer_amd.engine.engine import LlmEngine
+    from atoma_infer_amd.sampling import GenerateParameters
+    from atoma_infer_amd.weights import write_random_model
+    _toy_parts()
+    _toy_architecture()
+    cfg = dict(TOY, align=8)
+    d = write_random_model(str(tmp_path / "toy8"), cfg, seed=5, dtype="bfloat16", norm_jitter=0.1)
+    w = plain_weights(d)
+    prompts = [random_tokens(45, TOY["vocab"], 7), random_tokens(30, TOY["vocab"], 8)]
+    want = []
+    for p in prompts:
+        seq = list(p)
+        for _ in range(12):
+            seq.append(int(torch.argmax(toy_plain_forward(seq, w, cfg)[-1])))
+        want.append(seq[len(p):])
+    eng = LlmEngine(d, "float32", cache=CacheConfig(block_size=16, num_gpu_blocks_override=6),
+                    scheduler=SchedulerConfig(max_num_batched_tokens=21, max_num_sequences=2, max_model_len=64))
+    assert eng.model.spec.chunk_alignment == 8
+    mixer_cls = type(eng.model.spec.layers[1][1].mixer)
+    del mixer_cls.seen[:]
+    outs = eng.generate(prompts, GenerateParameters(do_sample=False, max_new_tokens=12, ignore_eos_token=True))
+    assert [o.inference_outputs[0].token_ids for o in outs] == want
+    portions = [(s0, n) for s0, n in mixer_cls.seen if n > 1]
+    assert portions and all(s0 % 8 == 0 for s0, _ in portions)
+    assert any(n == 16 for _, n in portions) and any(n % 8 for _, n in portions)    # 21 -> 16; the last is ragged
+    assert eng.stats["preemptions"] > 0
 
 
 # ----------------------------------------------------------------------------------------------------------

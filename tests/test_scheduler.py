@@ -292,6 +292,34 @@ def test_abort_frees_and_unchunked_prompts_wait_for_room():
     assert s.abort("nobody") is None
 
 
+def test_portions_end_where_the_model_allows():
+    """``ModelSpec.chunk_alignment``: a portion that does not end the request's tokens ends at a multiple of it,
+    under a token budget shared with decoding requests, and the last portion is free."""
+    cache = CacheManager([GroupGeometry(4, 64)], 8)
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=21, max_num_sequences=8, max_model_len=256), cache,
+                  chunk_alignment=8)
+    a, b = make_request(0, 45, max_new=3), make_request(1, 30, max_new=3)
+    s.add(a)
+    s.add(b)
+    seen = []
+    while s.has_unfinished():
+        out = s.schedule()
+        assert out.num_tokens <= 21
+        for e in out.entries:
+            end = e.start + e.num_tokens
+            assert e.num_tokens == 1 or e.start % 8 == 0
+            assert end % 8 == 0 or end == e.request.length, (e.request.uid, e.start, e.num_tokens)
+        seen.append([(e.request.uid, e.num_tokens) for e in out.entries])
+        run_step(s, out)
+    assert seen[0] == [(0, 16)] and seen[1] == [(0, 16)]          # 21 tokens of budget: 16 is what ends aligned
+    assert seen[2] == [(0, 13), (1, 8)]                             # the rest of a (unaligned, its last), 8 of b
+    import pytest
+    from atoma_infer_amd.engine.scheduler import SchedulerError
+    with pytest.raises(SchedulerError):                              # no aligned portion fits such a budget
+        Scheduler(SchedulerConfig(max_num_batched_tokens=6, max_num_sequences=4, max_model_len=256), cache,
+                  chunk_alignment=8)
+
+
 def test_max_prefill_chunk_caps_portions():
     s, cache = make_scheduler(max_num_batched_tokens=32, max_prefill_chunk=16)
     a = make_request(0, 37)
@@ -350,16 +378,19 @@ def _random_world(seed):
     lim = _Limits(max_tokens=rng.randint(4, 48), max_requests=rng.randint(1, 6), max_model_len=rng.randint(30, 120),
                   cut=rng.random() < 0.8, max_portion=rng.choice([0, 0, 5, 16]),
                   delay_factor=rng.choice([0.0, 0.0, 0.5, 3.0]))
+    lim.align = rng.choice([1, 1, 1, 4, 8])
     if not lim.cut:
         lim.max_tokens = max(lim.max_tokens, lim.max_model_len)      # the configuration demands it
-    lim.max_tokens = max(lim.max_tokens, lim.max_requests)
+    lim.max_tokens = max(lim.max_tokens, lim.max_requests, lim.align)
+    if lim.max_portion:
+        lim.max_portion = max(lim.max_portion, lim.align)
     now = [0.0]
     window = rng.choice([0, 0, 5, 12, 33])
     cache = CacheManager([GroupGeometry(page, pages, window=window or None)], slots)
     native = Scheduler(SchedulerConfig(max_num_batched_tokens=lim.max_tokens, max_num_sequences=lim.max_requests,
                                        max_model_len=lim.max_model_len, enable_chunked_prefill=lim.cut,
                                        max_prefill_chunk=lim.max_portion, delay_factor=lim.delay_factor),
-                       cache, clock=lambda: now[0])
+                       cache, clock=lambda: now[0], chunk_alignment=lim.align)
     plain_pages = PlainPages(page, pages, slots, window)
     plain = PlainScheduler(lim, plain_pages)
     mine, theirs, uid = {}, {}, 0
