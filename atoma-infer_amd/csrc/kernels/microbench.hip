@@ -1,0 +1,80 @@
+// What this GPU delivers, measured: a read stream and a copy over device memory, and a loop of bfloat16 MFMAs.
+// bench.py prints these beside the published peaks (8 TB/s, 2.5 PFLOP/s), which stay the yardstick of its fractions.
+#include "common.h"
+
+using namespace atoma;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+// every thread reads 16-byte words with a stride of the whole grid, four in flight; what is read is folded into one
+// word that is stored only if it has a value it practically never has
+__global__ void __launch_bounds__(256)
+probe_read_kernel(const uint4* __restrict__ src, size_t n16, uint32_t* __restrict__ sink) {
+  uint32_t acc = 0;
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    acc ^= a.x ^ b.y ^ c.z ^ d.w;
+  }
+  for (; i < n16; i += stride) acc ^= src[i].x;
+  if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
+__global__ void __launch_bounds__(256)
+probe_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    dst[i] = a, dst[i + stride] = b, dst[i + 2 * stride] = c, dst[i + 3 * stride] = d;
+  }
+  for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+// four independent accumulators a wave, so that the matrix core's pipeline stays full
+__global__ void __launch_bounds__(256)
+probe_mfma_kernel(int iters, float* __restrict__ sink) {
+  bf16x8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (__bf16)(float)((threadIdx.x + i) & 3);
+    b[i] = (__bf16)(float)((threadIdx.x * 3 + i) & 1);
+  }
+  f32x16 c0 = {}, c1 = {}, c2 = {}, c3 = {};
+  for (int it = 0; it < iters; ++it) {
+    c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
+    c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
+    c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
+    c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += c0[i] + c1[i] + c2[i] + c3[i];
+  if (s == -1.0f) sink[0] = s;      // sums of non-negative products: never
+}
+
+// grid: workgroups of 256 threads.  src (and dst) hold `bytes` bytes, a multiple of 16.
+extern "C" int atoma_probe_read(const void* src, size_t bytes, int grid, void* sink, hipStream_t stream) {
+  if (grid <= 0 || bytes % 16 || ((uintptr_t)src & 15)) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, (const uint4*)src, bytes / 16,
+                     (uint32_t*)sink);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int atoma_probe_copy(const void* src, void* dst, size_t bytes, int grid, hipStream_t stream) {
+  if (grid <= 0 || bytes % 16 || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(probe_copy_kernel, dim3(grid), dim3(256), 0, stream, (const uint4*)src, (uint4*)dst, bytes / 16);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// floating-point operations of one launch: grid * 4 waves * iters * 4 MFMAs * (2 * 32 * 32 * 16)
+extern "C" int atoma_probe_mfma(int iters, int grid, void* sink, hipStream_t stream) {
+  if (grid <= 0 || iters <= 0) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(probe_mfma_kernel, dim3(grid), dim3(256), 0, stream, iters, (float*)sink);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}

@@ -44,6 +44,7 @@ class KernelBuildError(RuntimeError):
 HIP_MODULES: Dict[str, Tuple[Sequence[str], Sequence[str]]] = {
     "core": (("elementwise.hip", "attention_generic.hip", "gemm_generic.hip", "sampling.hip"), ()),
     "gemm_bf16": (("gemm_bf16.hip",), ()),
+    "microbench": (("microbench.hip",), ()),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

@@ -311,3 +311,40 @@ def feed_tokens(dst: torch.Tensor, src: torch.Tensor, pairs: torch.Tensor) -> No
     _need(pairs.dtype is torch.int32 and pairs.is_contiguous() and pairs.dim() == 2 and pairs.shape[1] == 2,
           "pairs must be contiguous int32 [n, 2]")
     _check(core().atoma_feed_tokens(_p(dst), _p(src), _p(pairs), pairs.shape[0], _stream()), "feed_tokens")
+
+
+def measure_device_peaks(device: Optional[torch.device] = None, size_bytes: int = 1 << 30) -> dict:
+    """What the GPU delivers, measured with the probes of ``microbench.hip``: GB/s of a read stream and of a copy
+    (bytes read plus bytes written) over ``size_bytes`` of device memory, and TFLOP/s of a loop of bfloat16 MFMAs."""
+    lib = load_hip_module("microbench")
+    dev = device or torch.device("cuda:0")
+    src = torch.empty(size_bytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    sink = torch.zeros(4, dtype=torch.float32, device=dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+
+    def best(launch, reps=5):
+        launch()
+        torch.cuda.synchronize(dev)
+        times = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            launch()
+            b.record()
+            torch.cuda.synchronize(dev)
+            times.append(a.elapsed_time(b) * 1e-3)
+        return min(times)
+
+    out = {}
+    with torch.cuda.device(dev):
+        read = min(best(lambda g=g: _check(lib.atoma_probe_read(_p(src), ctypes.c_size_t(size_bytes), g, _p(sink),
+                                                                 _stream()), "probe_read")) for g in (cus * 8, cus * 16))
+        copy = min(best(lambda g=g: _check(lib.atoma_probe_copy(_p(src), _p(dst), ctypes.c_size_t(size_bytes), g,
+                                                                 _stream()), "probe_copy")) for g in (cus * 8, cus * 16))
+        iters, grid = 20000, cus * 8
+        mfma = best(lambda: _check(lib.atoma_probe_mfma(iters, grid, _p(sink), _stream()), "probe_mfma"), reps=3)
+    out["hbm_read_gbs"] = round(size_bytes / read / 1e9, 1)
+    out["hbm_copy_gbs"] = round(2 * size_bytes / copy / 1e9, 1)
+    out["mfma_bf16_tflops"] = round(grid * 4 * iters * 4 * 2 * 32 * 32 * 16 / mfma / 1e12, 1)
+    return out

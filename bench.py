@@ -2,13 +2,21 @@
 """Decode and prefill throughput of the engine at Llama-3.2-1B sizes with random weights, on one GPU.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--sizes 1b|3b|8b] [--layers N]
+    python bench.py --workload serve3b|long8b [--layers N] [--requests R]
 
 A "step" is one decode step of the whole engine (scheduler, step function, sampler).  The default run has the
 layer sizes of Llama-3.2-1B (16 layers, width 2048, 32 heads over 8 KV heads of 64, feed-forward 8192, vocabulary
 128256, llama3 rope scaling, tied head), bfloat16, random weights N(0, 0.02), 2048-token prompts of uniform random
 token ids, a batch of 8, and a maximum context of 8192.  It prints ONE JSON line: decoded tokens a second as
 ``value``, plus the 2048-token prefill, the decode step's roofline fraction (bytes it has to read / time / 8 TB/s)
-and decode throughput at batch 1 and 64.
+and decode throughput at batch 1 and 64; the read and copy bandwidth and the MFMA rate that this GPU delivers,
+measured by small probes, stand beside the published peaks (which stay the yardstick of every fraction).
+
+``--workload`` runs one of the other two workloads instead and prints ONE line of its own:
+``serve3b``: Llama-3.2-3B sizes, 64 requests with prompt lengths uniform in [128, 4096] (seeded), 256 generated tokens
+each, continuous batching with chunked prefill under 2,048 tokens a step; ``long8b``: Llama-3.1-8B sizes, 16 requests
+of 32,768 tokens of context (32,512 of prompt, 256 generated), prompts in 2,048-token portions beside decoding
+requests.  ``value`` is generated tokens a second over the whole run, prompts included.
 """
 from __future__ import annotations
 
@@ -115,6 +123,88 @@ def prefill_run(model, n_tokens, reps, context):
     return min(times[1:])
 
 
+WORKLOADS = {
+    # name: (sizes, requests, shortest prompt, longest prompt, generated tokens, tokens a step)
+    "serve3b": ("3b", 64, 128, 4096, 256, 2048),
+    "long8b": ("8b", 16, 32768 - 256, 32768 - 256, 256, 2048),
+}
+
+
+def serve_run(model, n_req, lo, hi, out_tokens, budget, seed=3):
+    """All requests arrive at once; the engine runs them to their end.  Returns what was measured."""
+    import random
+
+    import torch
+    from atoma_infer_amd.config import CacheConfig, SchedulerConfig, ValidationConfig
+    from atoma_infer_amd.engine.engine import LlmEngine
+    from atoma_infer_amd.sampling import GenerateParameters
+    rnd = random.Random(seed)
+    lens = [rnd.randint(lo, hi) for _ in range(n_req)]
+    ctx = hi + out_tokens + 16
+    pages = sum(-(-(n + out_tokens) // 16) + 1 for n in lens) + 64
+    eng = LlmEngine(model, cache=CacheConfig(block_size=16, num_gpu_blocks_override=pages),
+                    scheduler=SchedulerConfig(max_num_batched_tokens=budget, max_num_sequences=n_req,
+                                              max_model_len=ctx, enable_chunked_prefill=True),
+                    validation=ValidationConfig(max_input_length=ctx - 1, max_total_tokens=ctx))
+    g = torch.Generator().manual_seed(1)
+    params = GenerateParameters(do_sample=False, max_new_tokens=out_tokens, ignore_eos_token=True)
+    for n in lens:
+        eng.add_request(torch.randint(0, model.vocab_size, (n,), generator=g).tolist(), params)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps, done, times, last = 0, 0, [], t0
+    while eng.has_unfinished():
+        done += len(eng.step())
+        now = time.perf_counter()
+        times.append(now - last)
+        last = now
+        steps += 1
+        if steps % 200 == 0:
+            log(f"  step {steps}: {done} of {n_req} requests done, {now - t0:.1f} s")
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    times.sort()
+    assert done == n_req
+    return {"seconds": dt, "prompt_tokens": sum(lens), "generated": n_req * out_tokens, "steps": steps,
+            "preemptions": eng.stats["preemptions"], "step_median_ms": times[len(times) // 2] * 1e3,
+            "step_p99_ms": times[int(len(times) * 0.99)] * 1e3}
+
+
+def workload_main(args) -> int:
+    import atoma_infer_amd  # noqa: F401
+    from atoma_infer_amd.models import random_model
+    sizes, n_req, lo, hi, out_tokens, budget = WORKLOADS[args.workload]
+    n_req = args.requests or n_req
+    base = dict(LLAMA_1B, **OTHER_SIZES[sizes])
+    full_layers = base["num_hidden_layers"]
+    layers = args.layers or full_layers
+    name = {"3b": "Llama-3.2-3B", "8b": "Llama-3.1-8B"}[sizes]
+    log(f"{args.workload}: building {name} sizes ({layers} of {full_layers} layers, random weights) ...")
+    model = random_model(dict(base, num_hidden_layers=layers), seed=0, dtype="bfloat16", stored="bfloat16")
+    log(f"{n_req} requests, prompts of {lo} to {hi} tokens, {out_tokens} generated each, {budget} tokens a step ...")
+    r = serve_run(model, n_req, lo, hi, out_tokens, budget)
+    c = model.config
+    line = {
+        "metric": f"generated tok/s, workload {args.workload} ({name} sizes, {n_req} requests, continuous batching "
+                  f"with chunked prefill)",
+        "value": round(r["generated"] / r["seconds"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": r["steps"],
+        "warmup": 0, "ms_per_step": round(r["seconds"] / r["steps"] * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (uniform random token ids, random weights N(0, 0.02))",
+        "config": {"model": name + " sizes", "layers": layers, "layers_full": full_layers, "hidden": c.hidden_size,
+                   "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads, "head_dim": c.head_size,
+                   "intermediate": c.intermediate_size, "vocab": c.vocab_size, "requests": n_req,
+                   "prompt_min": lo, "prompt_max": hi, "generated_each": out_tokens, "tokens_a_step": budget,
+                   "kv_block": 16, "sampling": "argmax", "parallelism": "single GPU"},
+        "total_tokens_per_s": round((r["prompt_tokens"] + r["generated"]) / r["seconds"], 1),
+        "prompt_tokens": r["prompt_tokens"], "generated_tokens": r["generated"], "seconds": round(r["seconds"], 3),
+        "preemptions": r["preemptions"], "step_median_ms": round(r["step_median_ms"], 3),
+        "step_p99_ms": round(r["step_p99_ms"], 3),
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -132,6 +222,10 @@ def main() -> int:
                     help="sample with this temperature (and --top-k, --top-p) instead of the default argmax")
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--top-p", type=float, default=1.0)
+    ap.add_argument("--workload", choices=["decode", *WORKLOADS], default="decode",
+                    help="decode: the default run; serve3b, long8b: the other two workloads, one line of their own")
+    ap.add_argument("--requests", type=int, default=0, help="requests of a --workload run (default: the workload's)")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the probes of what the GPU delivers")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
@@ -139,6 +233,8 @@ def main() -> int:
     if int(os.environ.get("WORLD_SIZE", "1")) > 1:
         print("bench.py: started with WORLD_SIZE > 1; this engine runs on one GPU", flush=True)
         return 2
+    if args.workload != "decode":
+        return workload_main(args)
     if args.prompt_len + args.steps + args.warmup + 2 * args.batch * (-(-args.prompt_len // 2048)) + 8 > args.context:
         print("bench.py: prompt + steps exceed the context", file=sys.stderr)
         return 1
@@ -158,6 +254,13 @@ def main() -> int:
     model = random_model(cfg, seed=0, dtype="bfloat16", stored="bfloat16")
     log(f"model ready in {time.time() - t0:.1f} s; weights read per step: {model.weight_bytes() / 1e6:.1f} MB")
     kv_bytes_per_token = plan_cache(model.spec).bytes_per_token(2)
+
+    peaks = {}
+    if not args.no_peaks:
+        from atoma_infer_amd.kernels.ops import measure_device_peaks
+        log("probing what the GPU delivers (read stream, copy, MFMA loop) ...")
+        peaks = measure_device_peaks(model.device)
+        log(f"  {peaks}")
 
     log(f"prefill of {args.prefill_tokens} tokens ...")
     pre_s = prefill_run(model, args.prefill_tokens, 3, args.context)
@@ -182,6 +285,13 @@ def main() -> int:
     achieved = step_bytes / (dt / args.steps) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4)}
+    if peaks:
+        # what the probes reached on this GPU, beside the published peaks that the fractions above are of
+        roofline["measured_peak"] = peaks["hbm_read_gbs"]
+        roofline["measured_copy"] = peaks["hbm_copy_gbs"]
+        roofline["frac_of_measured"] = round(achieved / peaks["hbm_read_gbs"], 4)
+        prefill["measured_peak_tflops"] = peaks["mfma_bf16_tflops"]
+        prefill["frac_of_measured"] = round(pre_flops / pre_s / (peaks["mfma_bf16_tflops"] * 1e12), 4)
 
     points = {}
     if not args.no_points:
