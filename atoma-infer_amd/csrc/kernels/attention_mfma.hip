@@ -294,8 +294,10 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   if constexpr (KSPLIT > 1) {
     // Merge the shares of a task: the waves with part > 0 lay down (m, l, o), lane by lane; the wave with part 0
     // rescales all to the common maximum and adds them in order.  Same lanes hold the same (row, column) in all.
+    // (the launch asks for (KSPLIT - 1) * TASKS * PER_LANE * 64 floats of LDS: more than the 64 KB that a kernel may
+    // declare for itself when heads are wide, hence not declared here)
     constexpr int PER_LANE = DTILES * 16 + 2;
-    __shared__ float merge[(KSPLIT - 1) * TASKS * PER_LANE * 64];
+    extern __shared__ float merge[];
     if (part > 0) {
       float* dst = merge + (size_t)((part - 1) * TASKS + slot) * PER_LANE * 64 + lane;
       dst[0] = m;
@@ -450,9 +452,20 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
   }
 }
 
-// the merge needs (DTILES * 16 + 2) floats per lane of (KSPLIT - 1) * TASKS waves in LDS: 4 waves for 4 x 2, 7 for 1 x 8
-constexpr bool kSplit2Fits = (DTILES * 16 + 2) * 64 * 4 * sizeof(float) <= 65536;
-constexpr bool kSplit8Fits = (DTILES * 16 + 2) * 64 * 7 * sizeof(float) <= 65536;
+// the merge needs (DTILES * 16 + 2) floats per lane of (KSPLIT - 1) * TASKS waves in LDS: 4 waves for 4 x 2, 7 for 1 x 8;
+// a workgroup may have the 160 KB of a CU
+constexpr size_t kLdsBytes = 160 * 1024;
+constexpr size_t kMerge2Bytes = (DTILES * 16 + 2) * 64 * 4 * sizeof(float);
+constexpr size_t kMerge8Bytes = (DTILES * 16 + 2) * 64 * 7 * sizeof(float);
+constexpr bool kSplit2Fits = kMerge2Bytes <= kLdsBytes;
+constexpr bool kSplit8Fits = kMerge8Bytes <= kLdsBytes;
+
+// A kernel that wants more than 64 KB of LDS at launch must be told so once (per device).
+template <typename K> static int allow_lds(K kernel, size_t bytes) {
+  if (bytes <= 65536) return 0;
+  return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)bytes);
+}
 
 // compute units of the current device, asked for once per device
 static int compute_units() {
@@ -482,20 +495,24 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
   const Task* t = reinterpret_cast<const Task*>(tasks);
   // ksplit: waves that share a task's keys: 1, 2 (four tasks a workgroup) or 8 (one task a workgroup), the latter
   // two for head sizes whose merge fits in LDS
-#define ATOMA_ATTN(T, KS, ...)                                                                                     \
-  hipLaunchKernelGGL((attention_mfma_kernel<T, KS, ##__VA_ARGS__>), dim3(((n_tasks + T - 1) / T) * nkv),          \
-                     dim3(64 * T * KS), 0,                                                                        \
-                     stream, (const uint16_t*)q, q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,      \
-                     (uint16_t*)out, out_stride, part_o, part_lse, t, n_tasks, block_tables, max_blocks, scale,   \
-                     window, nh, nkv)
-  if (ksplit == 1) ATOMA_ATTN(4, 1);
+#define ATOMA_ATTN(T, KS, BYTES, ...)                                                                              \
+  do {                                                                                                             \
+    const int rc_lds = allow_lds(attention_mfma_kernel<T, KS, ##__VA_ARGS__>, BYTES);                              \
+    if (rc_lds != 0) return rc_lds;                                                                                \
+    hipLaunchKernelGGL((attention_mfma_kernel<T, KS, ##__VA_ARGS__>), dim3(((n_tasks + T - 1) / T) * nkv),        \
+                       dim3(64 * T * KS), BYTES,                                                                   \
+                       stream, (const uint16_t*)q, q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,     \
+                       (uint16_t*)out, out_stride, part_o, part_lse, t, n_tasks, block_tables, max_blocks, scale,  \
+                       window, nh, nkv);                                                                           \
+  } while (0)
+  if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
   // (two waves a task: always the late loads, two workgroups to a CU; long prompts gain 9 %, short ones nothing)
-  else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1), true);
+  else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1), kMerge2Bytes, true);
   else if (ksplit == 8 && kSplit8Fits) {
     // more workgroups than CUs: two of them to a CU finish sooner than two rounds of one (measured; with fewer,
     // the loads in flight during the softmax count for more)
-    if ((long long)n_tasks * nkv > compute_units()) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), true);
-    else ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1));
+    if ((long long)n_tasks * nkv > compute_units()) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), kMerge8Bytes, true);
+    else ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), kMerge8Bytes);
   }
   else return ATOMA_ERR_SHAPE;
 #undef ATOMA_ATTN

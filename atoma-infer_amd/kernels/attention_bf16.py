@@ -43,12 +43,12 @@ def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
 
 
 def max_waves_for(hd: int) -> int:
-    """Waves that may share a task for this head size: their merge must fit into LDS (the kernel module says the
-    same: ``atoma_attention_mfma_max_ksplit``)."""
+    """Waves that may share a task for this head size: their merge must fit into the 160 KB of LDS of a CU (the
+    kernel module says the same: ``atoma_attention_mfma_max_ksplit``)."""
     per_lane = -(-hd // 32) * 16 + 2
-    if per_lane * 64 * 7 * 4 <= 65536:
+    if per_lane * 64 * 7 * 4 <= 160 * 1024:
         return 8
-    return 2 if per_lane * 64 * 4 * 4 <= 65536 else 1
+    return 2 if per_lane * 64 * 4 * 4 <= 160 * 1024 else 1
 
 
 # (request, KV head) pairs from which on a decoded token's keys are not cut into chunks: measured on MI355X (256 CUs),

@@ -124,7 +124,9 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     # a head size that does not allow eight waves, or few pairs: chunks as before
     assert A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=2)[1][1] > 0
     assert A.build_tasks(starts[:8], counts[:8], group, window, bucket, kv_heads=8, max_waves=8)[1][1] > 0
-    assert A.max_waves_for(64) == 8 and A.max_waves_for(96) == 2 and A.max_waves_for(128) == 1
+    # the merge of the waves' shares must fit the 160 KB of LDS of a CU: eight waves up to heads of 160, two beyond
+    assert A.max_waves_for(64) == 8 and A.max_waves_for(128) == 8 and A.max_waves_for(160) == 8
+    assert A.max_waves_for(176) == 2 and A.max_waves_for(256) == 2
 
 
 @pytest.mark.parametrize("seed", range(20))
