@@ -52,7 +52,7 @@ struct Task {
   int32_t tok_base; // row of the entry's first token in the step's batch
   int32_t count;    // tokens of the entry in this step
   int32_t pos0;     // absolute position of the entry's first token
-  int32_t pad;
+  int32_t tiles;    // pieces of 32 rows that the task covers from row0 on: 2 in launches of two-tile waves, else 0 or 1
 };
 
 // x of the lane 32 away, by one cross-half register swap (no trip through LDS as a shuffle would take)
@@ -77,7 +77,13 @@ __device__ __forceinline__ bf16x8 pack8(const float* v) {
 //   4 x 2  prompts and mixed steps;
 //   1 x 8  decode steps of many requests: a task is all keys of a request's token, so nothing is left to the
 //          second kernel (there are enough requests and KV heads to fill the GPU without cutting keys into tasks).
-template <int TASKS, int KSPLIT, bool LATE = false>
+// RT: pieces of 32 rows a wave works on, against the same keys: with two, every fragment of keys and values that a
+// wave fetches, and the page and loop arithmetic of a block, serve 64 rows.  A wave's pace is set by its vector
+// instructions (about a hundred a block and piece, of which some 35 are that arithmetic), so portions behind long
+// prefixes gain (2,048 tokens behind 30,720: 882 -> 755 us at head size 64); short prompts lose, because twice as
+// few waves, each with a chain twice as long, fill the GPU worse (2,048 tokens alone: 43 -> 54 us).  The host asks
+// for two pieces from 16,384 keys on.
+template <int TASKS, int KSPLIT, bool LATE = false, int RT = 1>
 __global__ void __launch_bounds__(64 * TASKS * KSPLIT)
 attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
                       const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
@@ -104,14 +110,23 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const int k_end = has_task ? __builtin_amdgcn_readfirstlane(task.k_end) : k_begin;
   const int entry = has_task ? __builtin_amdgcn_readfirstlane(task.entry) : 0;
 
-  // this lane's row
-  const int r = task.row0 + c;
-  const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
-  const bool row_ok = has_task && hq < g && tok < task.count;
-  const int trow = row_ok ? task.tok_base + tok : 0;
-  const int p_row = row_ok ? task.pos0 + tok : -1;
-  const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
-  const int head = kvh * g + (row_ok ? hq : 0);
+  // this lane's row in each piece
+  bool row_ok[RT];
+  int trow[RT], p_row[RT], lo_row[RT], head[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    const int r = task.row0 + 32 * t + c;
+    const int hq = r / task.qt, tok = task.tok0 + r % task.qt;
+    row_ok[t] = has_task && hq < g && tok < task.count && (t == 0 || task.tiles > t);
+    trow[t] = row_ok[t] ? task.tok_base + tok : 0;
+    p_row[t] = row_ok[t] ? task.pos0 + tok : -1;
+    lo_row[t] = (window > 0 && p_row[t] - window + 1 > 0) ? p_row[t] - window + 1 : 0;
+    head[t] = kvh * g + (row_ok[t] ? hq : 0);
+  }
+  // a piece without a live row is skipped altogether (the same for all lanes)
+  bool piece_on[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) piece_on[t] = RT == 1 || __ballot(row_ok[t]) != 0;
 
   // page numbers of the task's keys: lane i holds the page of block first_block + i, fetched by one load for 64
   // blocks (1024 keys) at a time, so that no load of keys waits for a load of its page number
@@ -125,16 +140,25 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   int my_page = fetch_pages(first_block);
 
   // Q fragments: B operand, lane (row c, k half hg) holds 8 consecutive d per step
-  bf16x8 qf[KSTEPS];
-  {
-    const uint16_t* qp = q + (size_t)trow * q_stride + (size_t)head * HD + hg * 8;
+  bf16x8 qf[RT][KSTEPS];
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
+  for (int t = 0; t < RT; ++t) {
+    const uint16_t* qp = q + (size_t)trow[t] * q_stride + (size_t)head[t] * HD + hg * 8;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) qf[t][s] = *reinterpret_cast<const bf16x8*>(qp + s * 16);
   }
 
   // the lowest own position and the highest window start among this wave's live rows: blocks wholly between
   // them need no mask
-  int p_lo = row_ok ? p_row : 0x7fffffff, lo_hi = row_ok ? lo_row : 0;
+  int p_lo = 0x7fffffff, lo_hi = 0;
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    if (row_ok[t]) {
+      p_lo = min(p_lo, p_row[t]);
+      lo_hi = max(lo_hi, lo_row[t]);
+    }
+  }
+  if (p_lo == 0x7fffffff) p_lo = 0;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     p_lo = min(p_lo, __shfl_xor(p_lo, off, 64));
@@ -142,12 +166,16 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   }
 
   const float sc2 = scale * kLog2e;
-  float m = -INFINITY, l = 0.f;
-  f32x16 o[DTILES];
+  float m[RT], l[RT];
+  f32x16 o[RT][DTILES];
 #pragma unroll
-  for (int dt = 0; dt < DTILES; ++dt)
+  for (int t = 0; t < RT; ++t) {
+    m[t] = -INFINITY, l[t] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[t][dt][i] = 0.f;
+  }
 
   const size_t kv_head_stride = (size_t)PAGE * HD;            // one (page, head) tile
   const size_t page_stride = (size_t)nkv * kv_head_stride;
@@ -194,12 +222,91 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     }
   };
 
-  // One block is in flight: the next block's loads are issued right after S^T (the values move aside first) when
-  // registers allow, else at the end of the block.  LATE asks for the end of the block as well: 25 registers fewer,
-  // which lets two workgroups of eight waves share a CU.
-  constexpr bool EARLY = HD <= 128 && !LATE;
+  // The work on one block of 32 keys whose fragments have arrived; `after_scores` runs between S^T and the softmax
+  // (where the next loads go when they are issued early).
+  auto block = [&](int kb, const bf16x8* kf, const bf16x8 (*vf)[DTILES], auto after_scores) {
+    // S^T = K Q^T, for each piece of rows against the same fragments of the keys
+    f32x16 s[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[t][i] = 0.f;
+      if (piece_on[t]) {
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st)
+          s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[t][st], s[t], 0, 0, 0);
+      }
+    }
+    after_scores();
+
+    // Online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4.  The running maximum is kept in
+    // units of the scaled score (score * scale * log2 e), so one fused multiply-add feeds exp2.  Only blocks
+    // that touch a row's own position, the window's edge or the end of the key range need the mask.
+    const bool edge = kb + 31 > p_lo || kb < lo_hi || kb + 32 > k_end;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      if (!piece_on[t]) continue;
+      float sv[16];
+      float bmax = -INFINITY;
+      if (edge) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
+          const bool ok = key <= p_row[t] && key >= lo_row[t] && key < k_end;
+          sv[i] = ok ? s[t][i] : -INFINITY;
+          bmax = fmaxf(bmax, sv[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          sv[i] = s[t][i];
+          bmax = fmaxf(bmax, sv[i]);
+        }
+      }
+      bmax = fmaxf(bmax, from_other_half(bmax, hg != 0)) * sc2;
+      // The reference point m of a row's exponentials follows its maximum only in jumps: as long as no row of the
+      // wave has grown by more than kSlack (in powers of two) beyond its m, m stays, the weights may exceed one (by
+      // at most 2^kSlack, nothing to float32 sums or to bfloat16 weights, whose precision is relative) and the
+      // accumulators need no rescaling, which is most of a block's vector work.  out = o / l does not depend on m.
+      const float m_new = fmaxf(m[t], bmax);
+      const bool grew = __ballot(m_new > m[t] + kSlack) != 0;    // (-inf + kSlack = -inf: a row's first key always counts)
+      if (grew) {
+        const float corr = __builtin_amdgcn_exp2f(m[t] - ((m_new == -INFINITY) ? 0.f : m_new));
+        l[t] *= corr;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[t][dt][i] *= corr;
+        m[t] = m_new;
+      }
+      const float m_use = (m[t] == -INFINITY) ? 0.f : m[t];
+      float psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
+        psum += sv[i];
+      }
+      psum += from_other_half(psum, hg != 0);
+      l[t] += psum;
+
+      // O^T += V^T P^T
+      const bf16x8 pf0 = pack8(sv), pf1 = pack8(sv + 8);
+#pragma unroll
+      for (int dt = 0; dt < DTILES; ++dt) {
+        o[t][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[0][dt], pf0, o[t][dt], 0, 0, 0);
+        o[t][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[1][dt], pf1, o[t][dt], 0, 0, 0);
+      }
+    }
+  };
+
   constexpr int STRIDE = 32 * KSPLIT;
   const int k_first = k_begin + 32 * part;
+  // One block is in flight: the next block's loads are issued right after S^T (the values move aside first) when
+  // registers allow, else at the end of the block.  LATE asks for the end of the block as well: 25 registers fewer,
+  // which lets two workgroups of eight waves share a CU.  (More blocks in flight, each in registers of its own,
+  // gain nothing, for prompts as for decoding: a wave's pace is set by its vector instructions, about a hundred a
+  // block, not by the trip to the L2.)
+  constexpr bool EARLY = HD <= 128 && !LATE;
   bf16x8 kf[KSTEPS];
   bf16x8 vf[2][DTILES];
   if (k_first < k_end) {
@@ -208,81 +315,21 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     load_keys(p0, p1, kf);
     load_vals(p0, p1, vf);
   }
-
   for (int kb = k_first; kb < k_end; kb += STRIDE) {
-    // S^T = K Q^T
-    f32x16 s;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
-#pragma unroll
-    for (int st = 0; st < KSTEPS; ++st) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[st], s, 0, 0, 0);
     const bool has_next = kb + STRIDE < k_end;
     bf16x8 vc[2][DTILES];
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
       for (int dt = 0; dt < DTILES; ++dt) vc[jj][dt] = vf[jj][dt];
-    if (EARLY && has_next) {
-      int p0, p1;
-      pages_of(kb + STRIDE, p0, p1);
-      load_keys(p0, p1, kf);
-      load_vals(p0, p1, vf);
-    }
-
-    // Online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4.  The running maximum is kept in
-    // units of the scaled score (score * scale * log2 e), so one fused multiply-add feeds exp2.  Only blocks
-    // that touch a row's own position, the window's edge or the end of the key range need the mask.
-    const bool edge = kb + 31 > p_lo || kb < lo_hi || kb + 32 > k_end;
-    float sv[16];
-    float bmax = -INFINITY;
-    if (edge) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = kb + (i >> 2) * 8 + hg * 4 + (i & 3);
-        const bool ok = key <= p_row && key >= lo_row && key < k_end;
-        sv[i] = ok ? s[i] : -INFINITY;
-        bmax = fmaxf(bmax, sv[i]);
+    block(kb, kf, vc, [&]() {
+      if (EARLY && has_next) {
+        int p0, p1;
+        pages_of(kb + STRIDE, p0, p1);
+        load_keys(p0, p1, kf);
+        load_vals(p0, p1, vf);
       }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        sv[i] = s[i];
-        bmax = fmaxf(bmax, sv[i]);
-      }
-    }
-    bmax = fmaxf(bmax, from_other_half(bmax, hg != 0)) * sc2;
-    // The reference point m of a row's exponentials follows its maximum only in jumps: as long as no row of the
-    // wave has grown by more than kSlack (in powers of two) beyond its m, m stays, the weights may exceed one (by
-    // at most 2^kSlack, nothing to float32 sums or to bfloat16 weights, whose precision is relative) and the
-    // accumulators need no rescaling, which is most of a block's vector work.  out = o / l does not depend on m.
-    const float m_new = fmaxf(m, bmax);
-    const bool grew = __ballot(m_new > m + kSlack) != 0;    // (-inf + kSlack = -inf: a row's first key always counts)
-    if (grew) {
-      const float corr = __builtin_amdgcn_exp2f(m - ((m_new == -INFINITY) ? 0.f : m_new));
-      l *= corr;
-#pragma unroll
-      for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[dt][i] *= corr;
-      m = m_new;
-    }
-    const float m_use = (m == -INFINITY) ? 0.f : m;
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
-      psum += sv[i];
-    }
-    psum += from_other_half(psum, hg != 0);
-    l += psum;
-
-    // O^T += V^T P^T
-    const bf16x8 pf0 = pack8(sv), pf1 = pack8(sv + 8);
-#pragma unroll
-    for (int dt = 0; dt < DTILES; ++dt) {
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[0][dt], pf0, o[dt], 0, 0, 0);
-      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vc[1][dt], pf1, o[dt], 0, 0, 0);
-    }
+    });
     if (!EARLY && has_next) {
       int p0, p1;
       pages_of(kb + STRIDE, p0, p1);
@@ -296,69 +343,83 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     // rescales all to the common maximum and adds them in order.  Same lanes hold the same (row, column) in all.
     // (the launch asks for (KSPLIT - 1) * TASKS * PER_LANE * 64 floats of LDS: more than the 64 KB that a kernel may
     // declare for itself when heads are wide, hence not declared here)
-    constexpr int PER_LANE = DTILES * 16 + 2;
+    constexpr int PER_LANE = RT * (DTILES * 16 + 2);
     extern __shared__ float merge[];
     if (part > 0) {
       float* dst = merge + (size_t)((part - 1) * TASKS + slot) * PER_LANE * 64 + lane;
-      dst[0] = m;
-      dst[64] = l;
 #pragma unroll
-      for (int dt = 0; dt < DTILES; ++dt)
+      for (int t = 0; t < RT; ++t) {
+        float* d2 = dst + (size_t)t * (DTILES * 16 + 2) * 64;
+        d2[0] = m[t];
+        d2[64] = l[t];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[(2 + dt * 16 + i) * 64] = o[dt][i];
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) d2[(2 + dt * 16 + i) * 64] = o[t][dt][i];
+      }
     }
     __syncthreads();
     if (part > 0 || !has_task) return;
 #pragma unroll
     for (int h = 1; h < KSPLIT; ++h) {
       const float* src = merge + (size_t)((h - 1) * TASKS + slot) * PER_LANE * 64 + lane;
-      const float m2 = src[0], l2 = src[64];
-      const float m_all = fmaxf(m, m2);
-      const float m_use = (m_all == -INFINITY) ? 0.f : m_all;
-      const float a = __builtin_amdgcn_exp2f(m - m_use), b2 = __builtin_amdgcn_exp2f(m2 - m_use);
-      l = l * a + l2 * b2;
 #pragma unroll
-      for (int dt = 0; dt < DTILES; ++dt)
+      for (int t = 0; t < RT; ++t) {
+        const float* s2 = src + (size_t)t * (DTILES * 16 + 2) * 64;
+        const float m2 = s2[0], l2 = s2[64];
+        const float m_all = fmaxf(m[t], m2);
+        const float m_use = (m_all == -INFINITY) ? 0.f : m_all;
+        const float a = __builtin_amdgcn_exp2f(m[t] - m_use), b2 = __builtin_amdgcn_exp2f(m2 - m_use);
+        l[t] = l[t] * a + l2 * b2;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o[dt][i] = o[dt][i] * a + src[(2 + dt * 16 + i) * 64] * b2;
-      m = m_all;
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[t][dt][i] = o[t][dt][i] * a + s2[(2 + dt * 16 + i) * 64] * b2;
+        m[t] = m_all;
+      }
     }
   }
 
   // accumulator element i of tile dt is d = dt*32 + (i/4)*8 + hg*4 + i%4 of row c
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
   if (task.dest < 0) {
-    if (!row_ok) return;
-    uint16_t* op = out + (size_t)trow * out_stride + (size_t)head * HD;
 #pragma unroll
-    for (int dt = 0; dt < DTILES; ++dt)
+    for (int t = 0; t < RT; ++t) {
+      if (!row_ok[t]) continue;
+      const float inv = l[t] > 0.f ? 1.0f / l[t] : 0.f;
+      uint16_t* op = out + (size_t)trow[t] * out_stride + (size_t)head[t] * HD;
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int d = dt * 32 + q4 * 8 + hg * 4;
-        if (HD % 32 == 0 || d < HD) {
-          uint2 v;
-          v.x = (uint32_t)f32_to_bf16_bits(o[dt][q4 * 4 + 0] * inv) |
-                ((uint32_t)f32_to_bf16_bits(o[dt][q4 * 4 + 1] * inv) << 16);
-          v.y = (uint32_t)f32_to_bf16_bits(o[dt][q4 * 4 + 2] * inv) |
-                ((uint32_t)f32_to_bf16_bits(o[dt][q4 * 4 + 3] * inv) << 16);
-          *reinterpret_cast<uint2*>(op + d) = v;
+      for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int d = dt * 32 + q4 * 8 + hg * 4;
+          if (HD % 32 == 0 || d < HD) {
+            uint2 v;
+            v.x = (uint32_t)f32_to_bf16_bits(o[t][dt][q4 * 4 + 0] * inv) |
+                  ((uint32_t)f32_to_bf16_bits(o[t][dt][q4 * 4 + 1] * inv) << 16);
+            v.y = (uint32_t)f32_to_bf16_bits(o[t][dt][q4 * 4 + 2] * inv) |
+                  ((uint32_t)f32_to_bf16_bits(o[t][dt][q4 * 4 + 3] * inv) << 16);
+            *reinterpret_cast<uint2*>(op + d) = v;
+          }
         }
-      }
+    }
   } else {
+    // a partial result is one piece of 32 rows (the host gives such tasks one piece, whatever RT is);
     // rows that are not live are never read by the combine kernel (their log-sum-exp is, and says -inf)
+    const float inv = l[0] > 0.f ? 1.0f / l[0] : 0.f;
     float* po = part_o + (((size_t)task.dest * nkv + kvh) * 32 + c) * HD;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         const int d = dt * 32 + q4 * 8 + hg * 4;
-        if (row_ok && (HD % 32 == 0 || d < HD)) {
-          float4 v = make_float4(o[dt][q4 * 4 + 0] * inv, o[dt][q4 * 4 + 1] * inv, o[dt][q4 * 4 + 2] * inv,
-                                 o[dt][q4 * 4 + 3] * inv);
+        if (row_ok[0] && (HD % 32 == 0 || d < HD)) {
+          float4 v = make_float4(o[0][dt][q4 * 4 + 0] * inv, o[0][dt][q4 * 4 + 1] * inv, o[0][dt][q4 * 4 + 2] * inv,
+                                 o[0][dt][q4 * 4 + 3] * inv);
           *reinterpret_cast<float4*>(po + d) = v;
         }
       }
-    if (hg == 0) part_lse[((size_t)task.dest * nkv + kvh) * 32 + c] = l > 0.f ? m + __builtin_amdgcn_logf(l) : -INFINITY;
+    if (hg == 0)
+      part_lse[((size_t)task.dest * nkv + kvh) * 32 + c] = l[0] > 0.f ? m[0] + __builtin_amdgcn_logf(l[0]) : -INFINITY;
   }
 }
 
@@ -459,6 +520,9 @@ constexpr size_t kMerge2Bytes = (DTILES * 16 + 2) * 64 * 4 * sizeof(float);
 constexpr size_t kMerge8Bytes = (DTILES * 16 + 2) * 64 * 7 * sizeof(float);
 constexpr bool kSplit2Fits = kMerge2Bytes <= kLdsBytes;
 constexpr bool kSplit8Fits = kMerge8Bytes <= kLdsBytes;
+// two pieces of rows a wave: where the accumulators of both fit the registers of eight waves a workgroup, and the
+// merge of two waves a task (twice as large) lets two workgroups share a CU
+constexpr bool kTwoPieces = HD <= 64;
 
 // A kernel that wants more than 64 KB of LDS at launch must be told so once (per device).
 template <typename K> static int allow_lds(K kernel, size_t bytes) {
@@ -482,13 +546,16 @@ static int compute_units() {
 
 extern "C" int atoma_attention_mfma_head_size() { return HD; }
 extern "C" int atoma_attention_mfma_max_ksplit() { return kSplit8Fits ? 8 : kSplit2Fits ? 2 : 1; }
+extern "C" int atoma_attention_mfma_max_row_tiles() { return kTwoPieces ? 2 : 1; }
 
 // tasks: device array of n_tasks Task records (main kernel), followed by n_combine records for the combine kernel.
 extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kcache, const void* vcache, void* out,
                                     int out_stride, float* part_o, float* part_lse, const int32_t* tasks, int n_tasks,
                                     int n_combine, const int32_t* block_tables, int max_blocks, float scale,
-                                    int window, int nh, int nkv, int ksplit, hipStream_t stream) {
+                                    int window, int nh, int nkv, int ksplit, int row_tiles, hipStream_t stream) {
   if (n_tasks <= 0) return 0;
+  // row_tiles: 1, or 2: the tasks that write the output cover 64 rows (Task::tiles says so), two waves a task
+  if (row_tiles != 1 && !(row_tiles == 2 && kTwoPieces && ksplit == 2)) return ATOMA_ERR_SHAPE;
   if (nkv <= 0 || nh % nkv || nkv > 65535 || max_blocks <= 0 || (q_stride & 7) || (out_stride & 3) ||
       ((uintptr_t)q & 15) || ((uintptr_t)out & 7))
     return ATOMA_ERR_SHAPE;
@@ -507,6 +574,7 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
   } while (0)
   if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
   // (two waves a task: always the late loads, two workgroups to a CU; long prompts gain 9 %, short ones nothing)
+  else if (ksplit == 2 && row_tiles == 2) ATOMA_ATTN(4, 2, 2 * kMerge2Bytes, true, (kTwoPieces ? 2 : 1));
   else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1), kMerge2Bytes, true);
   else if (ksplit == 8 && kSplit8Fits) {
     // more workgroups than CUs: two of them to a CU finish sooner than two rounds of one (measured; with fewer,

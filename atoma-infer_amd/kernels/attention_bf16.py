@@ -39,6 +39,7 @@ def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
                                     force_build=force_build)
         assert _libs[hd].atoma_attention_mfma_head_size() == hd
         assert _libs[hd].atoma_attention_mfma_max_ksplit() == max_waves_for(hd)
+        assert _libs[hd].atoma_attention_mfma_max_row_tiles() == max_row_tiles_for(hd)
     return _libs[hd]
 
 
@@ -49,6 +50,15 @@ def max_waves_for(hd: int) -> int:
     if per_lane * 64 * 7 * 4 <= 160 * 1024:
         return 8
     return 2 if per_lane * 64 * 4 * 4 <= 160 * 1024 else 1
+
+
+TWO_PIECES_MIN_KEYS = 16384     # keys from which on a wave of a prompt step works on two pieces of rows
+
+
+def max_row_tiles_for(hd: int) -> int:
+    """Pieces of 32 rows that a wave of a prompt step may work on against the same keys (the kernel module says the
+    same: ``atoma_attention_mfma_max_row_tiles``): two where the accumulators of both fit a wave's registers."""
+    return 2 if hd <= 64 else 1
 
 
 # (request, KV head) pairs from which on a decoded token's keys are not cut into chunks: measured on MI355X (256 CUs),
@@ -88,14 +98,14 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False
     return CHUNK, 1
 
 
-def _live_pieces(rows: int, qt: int, live_tokens: int):
-    """First rows of the 32-row pieces of a tile that hold a live row.  Row r is token r % qt of head r // qt, and
-    the tile's first ``live_tokens`` tokens exist (fewer than qt only in the last tile of an entry)."""
+def _live_pieces(rows: int, qt: int, live_tokens: int, piece: int = 32):
+    """First rows of the ``piece``-row pieces of a tile that hold a live row.  Row r is token r % qt of head r // qt,
+    and the tile's first ``live_tokens`` tokens exist (fewer than qt only in the last tile of an entry)."""
     if live_tokens >= qt:
-        return list(range(0, rows, 32))
+        return list(range(0, rows, piece))
     out = []
-    for row0 in range(0, rows, 32):
-        n = min(32, rows - row0)
+    for row0 in range(0, rows, piece):
+        n = min(piece, rows - row0)
         first = row0 % qt
         # rows row0 .. row0 + n - 1 hold tokens first, first + 1, ... modulo qt: live if the run starts below
         # live_tokens or wraps around to token 0
@@ -116,12 +126,13 @@ def _chunk_slots(bucket_keys: int, chunk: int, window: int) -> int:
 _NULL_TASK = np.asarray((-1, 0, 1, 0, 0, 0, -1, 0, 0, 0, 0, 0), dtype=np.int32)
 
 
-def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, window: int, qt: int):
+def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, window: int, qt: int, row_tiles: int = 1):
     """The tasks of an entry that is not split along its keys, without a loop over its tiles: (keys per group of
-    four tasks, tasks [groups, 4, 12]).  A tile is ``qt`` tokens times ``group`` heads, cut into pieces of 32 rows;
-    pieces are padded to fours with empty tasks."""
+    four tasks, tasks [groups, 4, 12]).  A tile is ``qt`` tokens times ``group`` heads, cut into pieces of
+    32 * ``row_tiles`` rows, a task each; pieces are padded to fours with empty tasks."""
+    piece = 32 * row_tiles
     rows = qt * group
-    pieces = -(-rows // 32)
+    pieces = -(-rows // piece)
     fours = -(-pieces // 4)
     tok0 = np.arange(0, count, qt, dtype=np.int64)                           # [tiles]
     last = np.minimum(tok0 + qt, count)
@@ -131,11 +142,11 @@ def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, windo
     tiles = len(tok0)
     t = np.empty((tiles, fours * 4, 12), dtype=np.int32)
     t[:] = _NULL_TASK
-    row0 = 32 * np.arange(pieces, dtype=np.int64)
+    row0 = piece * np.arange(pieces, dtype=np.int64)
     live = np.ones((tiles, pieces), dtype=bool)
     if int(last[-1] - tok0[-1]) < qt:                                        # the short last tile
         live[-1] = False
-        live[-1, [r // 32 for r in _live_pieces(rows, qt, int(last[-1] - tok0[-1]))]] = True
+        live[-1, [r // piece for r in _live_pieces(rows, qt, int(last[-1] - tok0[-1]), piece)]] = True
     body = t[:, :pieces]
     vals = np.empty((tiles, pieces, 12), dtype=np.int32)
     vals[..., 0] = e
@@ -149,17 +160,19 @@ def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, windo
     vals[..., 8] = tok_base
     vals[..., 9] = count
     vals[..., 10] = start
-    vals[..., 11] = 0
+    vals[..., 11] = row_tiles
     body[live] = vals[live]
     lengths = np.repeat(k_end - kb, fours)
     return lengths, t.reshape(tiles * fours, 4, 12)
 
 
 def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket_keys: Optional[int] = None,
-                vectorized: bool = True, *, kv_heads: int, max_waves: int = 2,
-                ) -> Tuple[np.ndarray, Tuple[int, int, int, int]]:
+                vectorized: bool = True, *, kv_heads: int, max_waves: int = 2, row_tiles: int = 1,
+                ) -> Tuple[np.ndarray, tuple]:
     """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials, waves that
-    share a task: two when a prompt tile walks many keys, else what ``chunk_for`` says for the split entries).
+    share a task: two when a prompt tile walks many keys, else what ``chunk_for`` says for the split entries; pieces
+    of 32 rows that a task which writes the output covers: ``row_tiles`` if the step has such tasks, walks at least
+    ``TWO_PIECES_MIN_KEYS`` keys and two waves may share a task, else 1).
 
     Main tasks are padded to a multiple of 4 (one workgroup runs 4) and ordered so that tasks sharing keys are
     neighbours and long tasks come first.  With ``bucket_keys`` (decode steps: one token per entry; the context
@@ -169,7 +182,13 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     bucket = bucket_keys
     if vectorized and bucket is not None and len(counts) and int(counts.max()) == 1:
         return _build_decode_tasks(starts, group, window, bucket, kv_heads, max_waves)
-    qt_max = max(1, 128 // group)
+    # two pieces of rows a task where the prompt tiles of the step walk long key ranges (see the kernel), and the
+    # head size allows it
+    longest = int((starts + counts).max()) if len(starts) else 0
+    if max_waves < 2 or longest < TWO_PIECES_MIN_KEYS:
+        row_tiles = 1
+    qt_max = max(1, (128 * row_tiles) // group)
+    piece = 32 * row_tiles
     null = (-1, 0, 1, 0, 0, 0, -1, 0, 0, 0, 0, 0)
     tok_bases = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
     direct, split, combine = [], [], []
@@ -196,15 +215,16 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
         do_split = splits(e)
         tail = (int(tok_bases[e]), count, start, 0)
         if vectorized and not do_split:
-            lengths, groups = _tile_tasks(e, start, count, int(tok_bases[e]), group, window, qt)
+            lengths, groups = _tile_tasks(e, start, count, int(tok_bases[e]), group, window, qt, row_tiles)
             direct_arrays.append((lengths, groups))
             continue
         for tok0 in range(0, count, qt):
             last = min(tok0 + qt, count)
             k_end = start + last
             lo = max(0, start + tok0 - window + 1) if window > 0 else 0
-            # 32-row pieces of the tile that hold at least one live row (the last tile of an entry may be short)
-            live = _live_pieces(rows, qt, min(qt, count - tok0))
+            # pieces of the tile that hold at least one live row (the last tile of an entry may be short): 32 rows
+            # each for tasks that leave partial results, 32 * row_tiles for those that write the output
+            live = _live_pieces(rows, qt, min(qt, count - tok0), 32 if do_split else piece)
             if do_split:
                 c_first, c_last = lo // chunk, (k_end - 1) // chunk
                 # slot j holds chunk c_first + j
@@ -220,7 +240,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
                     n_part += slots
             else:
                 kb = (lo // 32) * 32
-                wave_tasks = [(e, tok0, qt, row0, kb, k_end, -1, 0) + tail for row0 in live]
+                wave_tasks = [(e, tok0, qt, row0, kb, k_end, -1, 0) + tail[:3] + (row_tiles,) for row0 in live]
                 while len(wave_tasks) % 4:
                     wave_tasks.append(null)
                 direct.append((k_end - kb, wave_tasks))
@@ -238,7 +258,9 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     arr = np.concatenate([head, rest])
     if len(head) and int((head[:, 5] - head[:, 4]).max()) >= SPLIT_WAVES_MIN_KEYS:
         waves = 2
-    return arr, (len(head) + len(split), len(combine), n_part, waves)
+    if row_tiles > 1 and len(head):
+        waves = 2                     # tasks of two pieces run in the launch of two waves a task only
+    return arr, (len(head) + len(split), len(combine), n_part, waves, row_tiles if len(head) else 1)
 
 
 def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int, kv_heads: int,
@@ -264,7 +286,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
         whole[..., 8] = np.arange(s)[:, None]
         whole[..., 9] = 1
         whole[..., 10] = starts[:, None]
-        return whole.reshape(-1, 12), (s * row_chunks, 0, 0, waves)
+        return whole.reshape(-1, 12), (s * row_chunks, 0, 0, waves, 1)
     slots = _chunk_slots(bucket, chunk, window)
     j = np.arange(slots, dtype=np.int64)
     c_first, c_last = lo // chunk, (k_end - 1) // chunk
@@ -300,7 +322,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     comb[..., 9] = 1
     comb[..., 10] = starts[:, None]
     arr = np.concatenate([main, comb.reshape(-1, 12)])
-    return arr, (len(main), s * row_chunks, s * row_chunks * slots, waves)
+    return arr, (len(main), s * row_chunks, s * row_chunks * slots, waves, 1)
 
 
 def plan_key(group: int, window: int, kv_heads: int, hd: int):
@@ -323,10 +345,10 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
         plan = ctx.scratch.get(key)
         if plan is None:
             arr, meta = build_tasks(ctx.h_starts, ctx.h_counts, group, window, kv_heads=nkv,
-                                    max_waves=max_waves_for(hd))
+                                    max_waves=max_waves_for(hd), row_tiles=max_row_tiles_for(hd))
             plan = (torch.from_numpy(arr).to(q.device), meta)
             ctx.scratch[key] = plan
-    tasks, (n_main, n_comb, n_part, waves) = plan
+    tasks, (n_main, n_comb, n_part, waves, row_tiles) = plan
     ksplit = min(waves, lib(hd).atoma_attention_mfma_max_ksplit())
     part_o = part_lse = None
     if n_part:
@@ -340,6 +362,6 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
     bt = cache.block_tables
     _check(lib(hd).atoma_attention_mfma(_p(q), q.stride(0), _p(k_cache), _p(v_cache), _p(out), out.stride(0),
                                         _p(part_o), _p(part_lse), _p(tasks), n_main, n_comb, _p(bt), bt.shape[1],
-                                        ctypes.c_float(scale), int(window), nh, nkv, ksplit, _stream()),
+                                        ctypes.c_float(scale), int(window), nh, nkv, ksplit, row_tiles, _stream()),
            "attention_mfma")
     return True

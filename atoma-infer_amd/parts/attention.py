@@ -94,7 +94,8 @@ class PagedAttention(Mixer):
         return (attention_bf16.plan_key(group, window, nkv, self.hd),
                 lambda starts, counts, bucket: attention_bf16.build_tasks(
                     starts, counts, group, window, bucket, kv_heads=nkv,
-                    max_waves=attention_bf16.max_waves_for(self.hd)))
+                    max_waves=attention_bf16.max_waves_for(self.hd),
+                    row_tiles=attention_bf16.max_row_tiles_for(self.hd)))
 
     # -- execution ------------------------------------------------------------------------------------
     accepts_begun = True

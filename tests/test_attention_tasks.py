@@ -7,19 +7,22 @@ from atoma_infer_amd.kernels import attention_bf16 as A
 
 
 def coverage(arr, meta, starts, counts, group, window):
-    n_main, n_comb, n_part, waves = meta
-    assert waves in (1, 2, 8)
+    n_main, n_comb, n_part, waves, tiles = meta
+    assert waves in (1, 2, 8) and tiles in (1, 2) and (tiles == 1 or waves == 2)
     main, comb = arr[:n_main], arr[n_main:]
     assert len(comb) == n_comb and (n_main % 4 == 0 or waves == 8)    # (eight waves: one task a workgroup)
     seen = {}          # (entry, token, head) -> list of key ranges, direct
     parts = {}         # partial index -> (entry, token/head rows, key range)
     for t in main:
-        e, tok0, qt, row0, kb, ke, dest, _, tok_base, count, pos0, _ = (int(x) for x in t)
+        e, tok0, qt, row0, kb, ke, dest, _, tok_base, count, pos0, pieces = (int(x) for x in t)
         if e < 0:
             continue
         assert tok_base == int(np.sum(counts[:e])) and count == counts[e] and pos0 == starts[e]
         assert kb % 32 == 0 and kb < ke
-        rows = [(tok0 + r % qt, r // qt) for r in range(row0, row0 + 32) if r // qt < group and tok0 + r % qt < count]
+        # a task that writes the output covers `tiles` pieces of 32 rows, one that leaves a partial result one
+        assert (max(pieces, 1) == tiles) if dest < 0 else pieces <= 1
+        n_rows = 32 * max(pieces, 1)
+        rows = [(tok0 + r % qt, r // qt) for r in range(row0, row0 + n_rows) if r // qt < group and tok0 + r % qt < count]
         assert rows
         if dest < 0:
             for row in rows:
@@ -49,7 +52,7 @@ def coverage(arr, meta, starts, counts, group, window):
 
 
 @pytest.mark.parametrize("seed", range(30))
-def test_tasks_cover_every_visible_key_once(seed):
+def test_tasks_cover_every_visible_key_once(seed, monkeypatch):
     rng = np.random.default_rng(seed)
     s = int(rng.integers(1, 9))
     group = int(rng.choice([1, 3, 4, 8, 40]))
@@ -58,6 +61,13 @@ def test_tasks_cover_every_visible_key_once(seed):
     starts = rng.integers(0, 2500, size=s).astype(np.int32)
     arr, meta = A.build_tasks(starts, counts, group, window, kv_heads=8)
     coverage(arr, meta, starts, counts, group, window)
+    # with two pieces of rows a task (head sizes up to 64, long key ranges), by both builders
+    monkeypatch.setattr(A, "TWO_PIECES_MIN_KEYS", int(rng.choice([0, 0, 1500])))
+    fast, mf = A.build_tasks(starts, counts, group, window, kv_heads=8, max_waves=8, row_tiles=2)
+    coverage(fast, mf, starts, counts, group, window)
+    slow, ms = A.build_tasks(starts, counts, group, window, vectorized=False, kv_heads=8, max_waves=8, row_tiles=2)
+    coverage(slow, ms, starts, counts, group, window)
+    assert mf == ms and sorted(map(tuple, fast.tolist())) == sorted(map(tuple, slow.tolist()))
 
 
 @pytest.mark.parametrize("seed", range(30))
@@ -119,7 +129,7 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     counts = np.ones(s, dtype=np.int32)
     bucket = -(-int(starts.max() + 1) // 256) * 256
     arr, meta = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
-    assert meta == (s * -(-group // 32), 0, 0, 8)
+    assert meta == (s * -(-group // 32), 0, 0, 8, 1)
     coverage(arr, meta, starts, counts, group, window)
     # a head size that does not allow eight waves, or few pairs: chunks as before
     assert A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=2)[1][1] > 0

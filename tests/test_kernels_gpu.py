@@ -291,6 +291,43 @@ def test_paged_attention(nh, nkv, hd, page, window, entries, kind):
         row += c
 
 
+TWO_PIECE_CASES = [c for c in ATTN_CASES if c[2] <= 64] + [
+    # groups of 1, 3, 8, 33 and 40 heads (tiles of 256, 255, 256, 264, 240 rows; the last pieces are short or half
+    # empty), one token, a window, portions beside decoded tokens
+    (5, 5, 64, 16, 0, [(0, 300), (700, 1)]),
+    (3, 1, 16, 16, 0, [(0, 100), (50, 86), (3, 1)]),
+    (16, 2, 64, 16, 0, [(100, 75), (2100, 33), (0, 7)]),
+    (33, 1, 32, 16, 0, [(0, 20), (40, 9)]),
+    (40, 1, 64, 16, 70, [(0, 130), (300, 2)]),
+]
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,window,entries", TWO_PIECE_CASES)
+def test_attention_with_two_pieces_of_rows_a_wave(nh, nkv, hd, page, window, entries, monkeypatch):
+    """Prompt tiles that walk many keys give every wave two pieces of 32 rows against the same keys.  Here the
+    threshold is taken away, so that every step with a prompt tile runs that way."""
+    from atoma_infer_amd.kernels import attention_bf16
+    monkeypatch.setattr(attention_bf16, "TWO_PIECES_MIN_KEYS", 0)
+    starts, counts = [s for s, _ in entries], [c for _, c in entries]
+    ks, vs, kc, vc, bt = paged_setup([s + c for s, c in entries], nkv, hd, page, torch.bfloat16, seed=hd + nh)
+    t = sum(counts)
+    g = torch.Generator().manual_seed(1)
+    qkv = (torch.randn(t, (nh + 2 * nkv) * hd, generator=g) * 1.5).bfloat16().to(DEV)
+    out = torch.full((t, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ctx, cache = FakeCtx(starts, counts), FakeCache(bt, page)
+    scale = 1.0 / math.sqrt(hd)
+    assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, cache, scale, window, nh, nkv, hd)
+    plan = [v for k, v in ctx.scratch.items() if k[0] == "attention_tasks_adhoc"][0]
+    assert plan[1][4] == 2, "the step was meant to run with two pieces a wave"
+    row = 0
+    for e, (s0, c) in enumerate(entries):
+        q = qkv[row:row + c, : nh * hd].cpu().view(c, nh, hd)
+        want = plain_attention(q, ks[e], vs[e], s0, scale, window, nh // nkv).reshape(c, nh * hd)
+        err = (out[row:row + c].double().cpu() - want).abs().max() / want.abs().max()
+        assert err < 2e-2, f"entry {e} ({s0}, {c}): {err:.3e}"
+        row += c
+
+
 HEADS_AND_SIZES = [(6, 2, hd) for hd in range(16, 257, 16)] + [
     # groups of 1, 7, 32, 33 and 40 heads to a KV head (more than 32 take several pieces of rows), many KV heads
     (5, 5, 64), (7, 1, 32), (64, 2, 64), (33, 1, 32), (40, 1, 64), (80, 2, 16), (24, 24, 48), (9, 3, 128)]
@@ -685,7 +722,7 @@ def test_attention_whole_ranges_with_eight_waves(window, more):
     ctx, cache = FakeCtx(starts, counts), FakeCache(bt, page)
     bucket = -(-max(lens) // 256) * 256
     arr, meta = A.build_tasks(ctx.h_starts, ctx.h_counts, nh // nkv, window, bucket, kv_heads=nkv, max_waves=8)
-    assert meta[1:] == (0, 0, 8)
+    assert meta[1:] == (0, 0, 8, 1)
     ctx.plans = {A.plan_key(nh // nkv, window, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
     scale = 1.0 / math.sqrt(hd)
     assert A.try_attention(q, kc, vc, out, ctx, cache, scale, window, nh, nkv, hd)
