@@ -83,7 +83,7 @@ __device__ __forceinline__ bf16x8 pack8(const float* v) {
 // prefixes gain (2,048 tokens behind 30,720: 882 -> 755 us at head size 64); short prompts lose, because twice as
 // few waves, each with a chain twice as long, fill the GPU worse (2,048 tokens alone: 43 -> 54 us).  The host asks
 // for two pieces from 16,384 keys on.
-template <int TASKS, int KSPLIT, bool LATE = false, int RT = 1>
+template <int TASKS, int KSPLIT, int RT = 1>
 __global__ void __launch_bounds__(64 * TASKS * KSPLIT)
 attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
                       const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
@@ -128,16 +128,15 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
 #pragma unroll
   for (int t = 0; t < RT; ++t) piece_on[t] = RT == 1 || __ballot(row_ok[t]) != 0;
 
-  // page numbers of the task's keys: lane i holds the page of block first_block + i, fetched by one load for 64
-  // blocks (1024 keys) at a time, so that no load of keys waits for a load of its page number
+  // page numbers: lane i asks for the page of block (kb / 16 + i) of the task's request; lanes 0 and 1 hold the two
+  // pages of the block of 32 keys at kb.  Asked for at the top of every turn for the next one, before anything else,
+  // so that waiting for the answer leaves the loads of fragments behind it in flight.
   const int32_t* table = block_tables + (size_t)entry * max_blocks;
-  int first_block = k_begin / PAGE;
-  auto fetch_pages = [&](int base) {
-    int b = base + lane;
+  auto page_window = [&](int kb) {
+    int b = kb / PAGE + lane;
     if (b > max_blocks - 1) b = max_blocks - 1;
     return table[b];
   };
-  int my_page = fetch_pages(first_block);
 
   // Q fragments: B operand, lane (row c, k half hg) holds 8 consecutive d per step
   bf16x8 qf[RT][KSTEPS];
@@ -149,7 +148,8 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   }
 
   // the lowest own position and the highest window start among this wave's live rows: blocks wholly between
-  // them need no mask
+  // them need no mask.  (A lane without a live row must stay out of the minimum: with a zero of its own, every block
+  // of a decode step, where 4 of a wave's 32 rows are live, would take the masked path.)
   int p_lo = 0x7fffffff, lo_hi = 0;
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
@@ -158,7 +158,6 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       lo_hi = max(lo_hi, lo_row[t]);
     }
   }
-  if (p_lo == 0x7fffffff) p_lo = 0;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     p_lo = min(p_lo, __shfl_xor(p_lo, off, 64));
@@ -180,17 +179,6 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const size_t kv_head_stride = (size_t)PAGE * HD;            // one (page, head) tile
   const size_t page_stride = (size_t)nkv * kv_head_stride;
 
-  // the two pages of the block of 32 keys at kb (a multiple of 32, asked for in rising order)
-  auto pages_of = [&](int kb, int& p0, int& p1) {
-    int b0 = kb / PAGE - first_block;
-    if (b0 >= 64) {
-      first_block += 64;
-      my_page = fetch_pages(first_block);
-      b0 -= 64;
-    }
-    p0 = __builtin_amdgcn_readlane(my_page, b0);
-    p1 = __builtin_amdgcn_readlane(my_page, b0 + 1);
-  };
   auto load_keys = [&](int p0, int p1, bf16x8* kf) {
     const int pg = (c < 16) ? p0 : p1;
     // tile order (cache_layout.h): for each 16 columns, the 8-column pieces of all 16 tokens side by side
@@ -222,9 +210,30 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     }
   };
 
-  // The work on one block of 32 keys whose fragments have arrived; `after_scores` runs between S^T and the softmax
-  // (where the next loads go when they are issued early).
-  auto block = [&](int kb, const bf16x8* kf, const bf16x8 (*vf)[DTILES], auto after_scores) {
+  // Keys run one block ahead of the values.  A block's values are asked for when its turn begins and arrive while
+  // S^T and the softmax run; the next block's keys are asked for as soon as S^T has used the registers of this
+  // block's, and arrive while the softmax and the P.V products run.  So no fragment needs registers of its own to wait
+  // in.  Every turn but the last issues the same loads, none of them under a condition (the last turn is a copy of
+  // the code without them), which lets the compiler wait for exactly the loads a product needs and leave the younger
+  // ones in flight.
+  constexpr int STRIDE = 32 * KSPLIT;
+  const int k_first = k_begin + 32 * part;
+  bf16x8 kf[KSTEPS];
+  bf16x8 vf[2][DTILES];
+  int p0 = 0, p1 = 0;
+  if (k_first < k_end) {
+    const int pw = page_window(k_first);
+    p0 = __builtin_amdgcn_readlane(pw, 0);
+    p1 = __builtin_amdgcn_readlane(pw, 1);
+    load_keys(p0, p1, kf);
+  }
+  auto turn = [&](int kb, auto more) {
+    constexpr bool MORE = decltype(more)::value;
+    int pw = 0;
+    if constexpr (MORE) pw = page_window(kb + STRIDE);
+    load_vals(p0, p1, vf);
+    // (no instruction: it keeps the compiler from moving these loads down to where their values are used)
+    asm volatile("" ::: "memory");
     // S^T = K Q^T, for each piece of rows against the same fragments of the keys
     f32x16 s[RT];
 #pragma unroll
@@ -237,7 +246,12 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
           s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[t][st], s[t], 0, 0, 0);
       }
     }
-    after_scores();
+    if constexpr (MORE) {
+      p0 = __builtin_amdgcn_readlane(pw, 0);
+      p1 = __builtin_amdgcn_readlane(pw, 1);
+      load_keys(p0, p1, kf);
+      asm volatile("" ::: "memory");
+    }
 
     // Online softmax; accumulator element i is key kb + (i/4)*8 + hg*4 + i%4.  The running maximum is kept in
     // units of the scaled score (score * scale * log2 e), so one fused multiply-add feeds exp2.  Only blocks
@@ -298,45 +312,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       }
     }
   };
-
-  constexpr int STRIDE = 32 * KSPLIT;
-  const int k_first = k_begin + 32 * part;
-  // One block is in flight: the next block's loads are issued right after S^T (the values move aside first) when
-  // registers allow, else at the end of the block.  LATE asks for the end of the block as well: 25 registers fewer,
-  // which lets two workgroups of eight waves share a CU.  (More blocks in flight, each in registers of its own,
-  // gain nothing, for prompts as for decoding: a wave's pace is set by its vector instructions, about a hundred a
-  // block, not by the trip to the L2.)
-  constexpr bool EARLY = HD <= 128 && !LATE;
-  bf16x8 kf[KSTEPS];
-  bf16x8 vf[2][DTILES];
-  if (k_first < k_end) {
-    int p0, p1;
-    pages_of(k_first, p0, p1);
-    load_keys(p0, p1, kf);
-    load_vals(p0, p1, vf);
-  }
-  for (int kb = k_first; kb < k_end; kb += STRIDE) {
-    const bool has_next = kb + STRIDE < k_end;
-    bf16x8 vc[2][DTILES];
-#pragma unroll
-    for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-      for (int dt = 0; dt < DTILES; ++dt) vc[jj][dt] = vf[jj][dt];
-    block(kb, kf, vc, [&]() {
-      if (EARLY && has_next) {
-        int p0, p1;
-        pages_of(kb + STRIDE, p0, p1);
-        load_keys(p0, p1, kf);
-        load_vals(p0, p1, vf);
-      }
-    });
-    if (!EARLY && has_next) {
-      int p0, p1;
-      pages_of(kb + STRIDE, p0, p1);
-      load_keys(p0, p1, kf);
-      load_vals(p0, p1, vf);
-    }
-  }
+  int kb = k_first;
+  for (; kb + STRIDE < k_end; kb += STRIDE) turn(kb, std::true_type{});
+  if (kb < k_end) turn(kb, std::false_type{});
 
   if constexpr (KSPLIT > 1) {
     // Merge the shares of a task: the waves with part > 0 lay down (m, l, o), lane by lane; the wave with part 0
@@ -531,19 +509,6 @@ template <typename K> static int allow_lds(K kernel, size_t bytes) {
                                   (int)bytes);
 }
 
-// compute units of the current device, asked for once per device
-static int compute_units() {
-  static int cus[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cus[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cus[dev] = n;
-  }
-  return cus[dev];
-}
-
 extern "C" int atoma_attention_mfma_head_size() { return HD; }
 extern "C" int atoma_attention_mfma_max_ksplit() { return kSplit8Fits ? 8 : kSplit2Fits ? 2 : 1; }
 extern "C" int atoma_attention_mfma_max_row_tiles() { return kTwoPieces ? 2 : 1; }
@@ -573,15 +538,9 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
                        window, nh, nkv);                                                                           \
   } while (0)
   if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
-  // (two waves a task: always the late loads, two workgroups to a CU; long prompts gain 9 %, short ones nothing)
-  else if (ksplit == 2 && row_tiles == 2) ATOMA_ATTN(4, 2, 2 * kMerge2Bytes, true, (kTwoPieces ? 2 : 1));
-  else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1), kMerge2Bytes, true);
-  else if (ksplit == 8 && kSplit8Fits) {
-    // more workgroups than CUs: two of them to a CU finish sooner than two rounds of one (measured; with fewer,
-    // the loads in flight during the softmax count for more)
-    if ((long long)n_tasks * nkv > compute_units()) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), kMerge8Bytes, true);
-    else ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), kMerge8Bytes);
-  }
+  else if (ksplit == 2 && row_tiles == 2) ATOMA_ATTN(4, 2, 2 * kMerge2Bytes, (kTwoPieces ? 2 : 1));
+  else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1), kMerge2Bytes);
+  else if (ksplit == 8 && kSplit8Fits) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), kMerge8Bytes);
   else return ATOMA_ERR_SHAPE;
 #undef ATOMA_ATTN
   ATOMA_LAUNCH_CHECK();
