@@ -62,18 +62,25 @@ def max_row_tiles_for(hd: int) -> int:
 
 
 # (request, KV head) pairs from which on a decoded token's keys are not cut into chunks: measured on MI355X (256 CUs),
-# half as many pairs as CUs win at contexts from 2,000 to 32,000 tokens; with 64 pairs chunks win at all of them
+# half as many pairs as CUs win at contexts from 2,000 to 32,000 tokens; with 64 pairs chunks win from 2,000 keys on
 WHOLE_MIN_PAIRS = 128
+# Fewer pairs take whole ranges too where a wave's walk is short; the walk is counted in key elements (keys times head
+# size; measured at head sizes 64 and 128, 1 to 16 requests of 8 KV heads, 512 to 32,768 keys).  (pairs from, walk up to):
+# 96 pairs up to 8,192 keys of head size 64 (4 to 13 % quicker than chunks), 32 up to 1,536, any number up to 1,024
+# (there the second kernel costs more than the walk: 7.4 to 7.9 us against 8.9 to 10.8 at 512 keys).
+WHOLE_SHORT_WALKS = ((96, 8192 * 64), (32, 1536 * 64), (1, 1024 * 64))
 # keys from which on the chunks of a decoded token are 512 keys long, walked by two waves (2 to 6 % quicker steps at
 # 16k to 32k tokens with 1 to 12 requests; no gain at 8k)
 LONG_KEYS = 16384
 
 
-def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False) -> Tuple[int, int]:
+def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False, head_size: int = 64,
+              ) -> Tuple[int, int]:
     """(keys per partial task, waves that share a task) for the entries of a step that are split along their keys;
-    keys per task 0 means all of them: with ``whole_ok`` (a decode step, head size that allows eight waves) and
-    enough (request, KV head) pairs to occupy the GPU, eight waves walk all keys of a pair and merge in LDS, which
-    leaves nothing to the merging kernel.
+    keys per task 0 means all of them: with ``whole_ok`` (a decode step, head size that allows eight waves) eight
+    waves walk all keys of a (request, KV head) pair and merge in LDS, which leaves nothing to the merging kernel.
+    That pays where the pairs occupy the GPU, or where a wave's share of the keys is so short that the second
+    kernel costs more than the longer walk.
 
     A wave walks its keys one 32-key block after another, so few keys per wave shorten the chain when few requests
     decode, and long chunks save partial results (and time in the merging kernel) when many do.  Measured on
@@ -84,8 +91,10 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False
     heads; ``max_keys`` is rounded up to 256.
     """
     pairs = n_split * kv_heads
-    if whole_ok and pairs >= WHOLE_MIN_PAIRS:     # at 2,000 as at 32,000 keys (measured from 128 pairs on)
-        return 0, 8
+    if whole_ok:
+        walk = max_keys * head_size
+        if pairs >= WHOLE_MIN_PAIRS or any(pairs >= p and walk <= w for p, w in WHOLE_SHORT_WALKS):
+            return 0, 8
     tasks = n_split * -(-max_keys // CHUNK) * kv_heads
     if tasks <= 160:
         return 128, 1
@@ -168,7 +177,7 @@ def _tile_tasks(e: int, start: int, count: int, tok_base: int, group: int, windo
 
 def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int, bucket_keys: Optional[int] = None,
                 vectorized: bool = True, *, kv_heads: int, max_waves: int = 2, row_tiles: int = 1,
-                ) -> Tuple[np.ndarray, tuple]:
+                head_size: int = 64) -> Tuple[np.ndarray, tuple]:
     """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials, waves that
     share a task: two when a prompt tile walks many keys, else what ``chunk_for`` says for the split entries; pieces
     of 32 rows that a task which writes the output covers: ``row_tiles`` if the step has such tasks, walks at least
@@ -181,7 +190,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     """
     bucket = bucket_keys
     if vectorized and bucket is not None and len(counts) and int(counts.max()) == 1:
-        return _build_decode_tasks(starts, group, window, bucket, kv_heads, max_waves)
+        return _build_decode_tasks(starts, group, window, bucket, kv_heads, max_waves, head_size)
     # two pieces of rows a task where the prompt tiles of the step walk long key ranges (see the kernel), and the
     # head size allows it
     longest = int((starts + counts).max()) if len(starts) else 0
@@ -264,7 +273,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
 
 
 def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int, kv_heads: int,
-                        max_waves: int = 2):
+                        max_waves: int = 2, head_size: int = 64):
     """``build_tasks`` for a step in which every entry brings one token, without a Python loop over entries."""
     s = len(starts)
     starts = starts.astype(np.int64)
@@ -273,7 +282,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     row_chunks = -(-group // 32)
     # the bucket, not the step's longest request, decides between whole ranges and chunks: a graph holds one of them
     keys = bucket if window <= 0 else min(bucket, window + CHUNK)      # what a token can see
-    chunk, waves = chunk_for(s, keys, kv_heads, whole_ok=max_waves >= 8)
+    chunk, waves = chunk_for(s, keys, kv_heads, whole_ok=max_waves >= 8, head_size=head_size)
     waves = min(waves, max_waves)
     if chunk == 0:
         whole = np.zeros((s, row_chunks, 12), dtype=np.int32)

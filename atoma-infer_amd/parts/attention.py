@@ -95,7 +95,7 @@ class PagedAttention(Mixer):
                 lambda starts, counts, bucket: attention_bf16.build_tasks(
                     starts, counts, group, window, bucket, kv_heads=nkv,
                     max_waves=attention_bf16.max_waves_for(self.hd),
-                    row_tiles=attention_bf16.max_row_tiles_for(self.hd)))
+                    row_tiles=attention_bf16.max_row_tiles_for(self.hd), head_size=self.hd))
 
     # -- execution ------------------------------------------------------------------------------------
     accepts_begun = True

@@ -131,9 +131,22 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     arr, meta = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
     assert meta == (s * -(-group // 32), 0, 0, 8, 1)
     coverage(arr, meta, starts, counts, group, window)
-    # a head size that does not allow eight waves, or few pairs: chunks as before
+    # a head size that does not allow eight waves, or few pairs with many keys to walk: chunks as before
     assert A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=2)[1][1] > 0
-    assert A.build_tasks(starts[:8], counts[:8], group, window, bucket, kv_heads=8, max_waves=8)[1][1] > 0
+    far = np.full(8, 2999, dtype=np.int32)
+    assert A.build_tasks(far, counts[:8], group, 0, 3072, kv_heads=8, max_waves=8)[1][1] > 0
+    assert A.build_tasks(far, counts[:8], group, 0, 3072, kv_heads=8, max_waves=8, head_size=128)[1][1] > 0
+    # few pairs with few keys to walk: whole ranges again (the second kernel would cost more than the walk)
+    near = np.full(8, 999, dtype=np.int32)
+    arr2, meta2 = A.build_tasks(near, counts[:8], group, 0, 1024, kv_heads=8, max_waves=8)
+    assert meta2 == (8 * -(-group // 32), 0, 0, 8, 1)
+    coverage(arr2, meta2, near, counts[:8], group, 0)
+    assert A.build_tasks(near, counts[:8], group, 0, 1024, kv_heads=8, max_waves=8, head_size=128)[1][1] > 0
+    # twelve requests of 8 KV heads: whole ranges up to 8,192 keys of head size 64, 4,096 of head size 128
+    assert A.chunk_for(12, 8192, 8, whole_ok=True, head_size=64) == (0, 8)
+    assert A.chunk_for(12, 8192, 8, whole_ok=True, head_size=128)[0] > 0
+    assert A.chunk_for(12, 4096, 8, whole_ok=True, head_size=128) == (0, 8)
+    assert A.chunk_for(12, 32768, 8, whole_ok=True, head_size=64)[0] > 0
     # the merge of the waves' shares must fit the 160 KB of LDS of a CU: eight waves up to heads of 160, two beyond
     assert A.max_waves_for(64) == 8 and A.max_waves_for(128) == 8 and A.max_waves_for(160) == 8
     assert A.max_waves_for(176) == 2 and A.max_waves_for(256) == 2

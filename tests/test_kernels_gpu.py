@@ -4,6 +4,8 @@ import math
 import pytest
 import torch
 
+from util import force_chunked_decode
+
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
@@ -768,6 +770,8 @@ def test_decode_plans_with_large_groups(nh, nkv, hd, whole, monkeypatch):
         if attention_bf16.max_waves_for(hd) < 8:
             pytest.skip("eight waves a task do not fit this head size")
         monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 2)
+    else:
+        force_chunked_decode(monkeypatch)
     group, page = nh // nkv, 16
     starts = [700, 129, 15, 256, 511]
     counts = [1] * len(starts)
@@ -793,12 +797,18 @@ def test_decode_plans_with_large_groups(nh, nkv, hd, whole, monkeypatch):
         assert err < 2e-2, f"request {e} at {s}: {err:.3e}"
 
 
+@pytest.mark.parametrize("whole", [False, True])
 @pytest.mark.parametrize("window", [64, 200, 1000])
-def test_decode_plans_behind_a_window(window):
-    """Decoded tokens far behind a window, planned as the engine plans them: their requests own slots only for the
-    chunks a window can touch, the first of which is wherever the window begins."""
+def test_decode_plans_behind_a_window(window, whole, monkeypatch):
+    """Decoded tokens far behind a window, planned as the engine plans them: in chunks, their requests own slots only
+    for the chunks a window can touch, the first of which is wherever the window begins; as whole ranges, eight
+    waves begin where the window does."""
     import numpy as np
     from atoma_infer_amd.kernels import attention_bf16
+    if whole:
+        monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 2)
+    else:
+        force_chunked_decode(monkeypatch)
     nh, nkv, hd, page = 8, 2, 64, 16
     starts = [1500, 700, 300, 129, 5]
     counts = [1] * len(starts)
@@ -812,7 +822,10 @@ def test_decode_plans_behind_a_window(window):
     arr, meta = attention_bf16.build_tasks(np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32),
                                            nh // nkv, window, bucket, kv_heads=nkv,
                                            max_waves=attention_bf16.max_waves_for(hd))
-    assert 0 < meta[2] <= t * (window // 128 + 2)
+    if whole:
+        assert meta[1:4] == (0, 0, 8)
+    else:
+        assert 0 < meta[2] <= t * (window // 128 + 2)
     ctx.plans = {attention_bf16.plan_key(nh // nkv, window, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
     scale = 1.0 / math.sqrt(hd)
     assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, FakeCache(bt, page), scale, window, nh, nkv, hd)

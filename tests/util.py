@@ -109,3 +109,12 @@ def check_greedy_tokens(prompt: List[int], tokens: List[int], chosen_logits: Lis
             f"step {step}: the engine's logit {lg:.5f} of token {tok} is not the plain model's {float(row[tok]):.5f}"
         assert float(row.max() - row[tok]) <= 2 * tol * scale, \
             f"step {step}: token {tok} is no argmax of the plain model ({float(row[tok]):.5f} < {float(row.max()):.5f})"
+
+
+def force_chunked_decode(monkeypatch):
+    """Make the bfloat16 attention cut the keys of decoded tokens into chunks that a second kernel merges, as it does
+    at long contexts with few requests; at the tiny contexts of tests its planner would let eight waves walk whole
+    key ranges instead."""
+    from atoma_infer_amd.kernels import attention_bf16
+    monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 10 ** 9)
+    monkeypatch.setattr(attention_bf16, "WHOLE_SHORT_WALKS", ())
