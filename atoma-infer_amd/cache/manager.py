@@ -55,6 +55,10 @@ def _host():
         lib.cm_table.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_int]
         lib.cm_fill_step.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
                                      ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+        lib.cm_reserve_all.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                       ctypes.c_void_p, ctypes.c_void_p]
+        lib.cm_release_behind_all.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        lib.cm_pack_step.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 9 + [ctypes.c_int]
         _lib = lib
     return _lib
 
@@ -131,6 +135,24 @@ class CacheManager:
         if rc != 0:
             raise CacheError(f"reserve({request}, {length}) failed with code {rc}")
 
+    def reserve_all(self, ids: np.ndarray, starts: np.ndarray, counts: np.ndarray) -> None:
+        """``reserve(ids[e], starts[e] + counts[e])`` for every entry of a step, in one call."""
+        failed = ctypes.c_int(-1)
+        rc = self._lib.cm_reserve_all(self._h, len(ids), ids.ctypes.data, starts.ctypes.data, counts.ctypes.data,
+                                      ctypes.byref(failed))
+        if rc == 0:
+            return
+        e = failed.value
+        what = f"request {int(ids[e])}" if e >= 0 else "a request"
+        if rc == -1:
+            raise OutOfPages(f"{what}: not enough free pages to reach {int(starts[e]) + int(counts[e])} tokens")
+        raise CacheError(f"reserving for {what} failed with code {rc}")
+
+    def release_behind_all(self, ids: np.ndarray, done: np.ndarray) -> None:
+        """``release_behind(ids[e], done[e])`` for every entry of a step, in one call."""
+        if self._lib.cm_release_behind_all(self._h, len(ids), ids.ctypes.data, done.ctypes.data) != 0:
+            raise CacheError("a request of the step is not registered")
+
     def reserved_len(self, request: int) -> int:
         rc = self._lib.cm_reserved_len(self._h, request)
         if rc < 0:
@@ -187,3 +209,22 @@ class CacheManager:
             raise CacheError("a token of the step has no page (reserve before the step; was its page released?)")
         if rc != 0:
             raise CacheError(f"fill_step failed with code {rc}")
+
+    def pack_step(self, ids: np.ndarray, starts: np.ndarray, counts: np.ndarray, tokens: np.ndarray,
+                  feeds: np.ndarray, want_counts: np.ndarray, wants: np.ndarray, buf: np.ndarray,
+                  offsets: np.ndarray, max_blocks: int) -> int:
+        """Write a step's metadata into the int32 staging buffer ``buf``: token ids, positions, entry per token,
+        first row and length per entry, state slots, wanted rows, and per group the cache slots and block tables
+        (``fill_step``); ``offsets`` (int64) says where each array starts, in the order of ``cm_pack_step``.
+        Returns the number of (row, feed) pairs written."""
+        assert ids.dtype == np.int64 and offsets.dtype == np.int64 and buf.dtype == np.int32
+        for a in (starts, counts, tokens, feeds, want_counts, wants):
+            assert a.dtype == np.int32 and a.flags.c_contiguous
+        rc = self._lib.cm_pack_step(self._h, len(ids), ids.ctypes.data, starts.ctypes.data, counts.ctypes.data,
+                                    tokens.ctypes.data, feeds.ctypes.data, want_counts.ctypes.data, wants.ctypes.data,
+                                    buf.ctypes.data, offsets.ctypes.data, int(max_blocks))
+        if rc == -1:
+            raise CacheError("a token of the step has no page (reserve before the step; was its page released?)")
+        if rc < 0:
+            raise CacheError(f"packing the step failed with code {rc}")
+        return rc

@@ -284,6 +284,90 @@ int cm_fill_step(void* h, int group, int n, const int64_t* ids, const int32_t* s
   return CM_OK;
 }
 
+// One step's reservations in one call: every entry's request is made to cover its tokens.  Returns CM_OK, or the
+// code of the first reservation that failed, with that entry's index in *failed (earlier entries keep what they
+// got, as after a loop of cm_reserve calls).
+int cm_reserve_all(void* h, int n, const int64_t* ids, const int32_t* starts, const int32_t* counts, int* failed) {
+  for (int e = 0; e < n; ++e) {
+    const int rc = cm_reserve(h, ids[e], (int64_t)starts[e] + counts[e]);
+    if (rc != CM_OK) {
+      if (failed) *failed = e;
+      return rc;
+    }
+  }
+  return CM_OK;
+}
+
+// After a step: pages that a window has passed go back, for every entry; done[e] is what request ids[e] now holds.
+int cm_release_behind_all(void* h, int n, const int64_t* ids, const int32_t* done) {
+  for (int e = 0; e < n; ++e) {
+    const int rc = cm_release_behind(h, ids[e], done[e]);
+    if (rc < 0) return rc;
+  }
+  return CM_OK;
+}
+
+// The metadata of a step, written into one staging buffer of int32 (the layout is the caller's: off[] gives where
+// each array starts).  Entry e brings counts[e] tokens of request ids[e] at positions starts[e] ...; tokens holds
+// them one entry after the other; feeds[e] >= 0 names the row of a device array that supplies the entry's one token
+// instead; wants holds, per entry, want_counts[e] places among its tokens.  Written: token ids, positions and
+// entry index per token; first row per entry (n + 1 values); length after the step and state slot per entry; the
+// batch rows of the wanted places; per group, cache slot per token and padded block table per entry; and
+// (row, feed) pairs.  Returns the number of such pairs, or a negative code.
+//   off: tokens, positions, token->entry, first rows, lengths, state slots, wanted rows, slot mappings (groups one
+//   after the other, a step's tokens each), block tables (groups one after the other, n * max_blocks each), pairs
+int cm_pack_step(void* h, int n, const int64_t* ids, const int32_t* starts, const int32_t* counts,
+                 const int32_t* tokens, const int32_t* feeds, const int32_t* want_counts, const int32_t* wants,
+                 int32_t* buf, const int64_t* off, int max_blocks) {
+  Manager* m = static_cast<Manager*>(h);
+  if (n <= 0 || max_blocks <= 0) return CM_BAD_ARG;
+  int32_t* o_tok = buf + off[0];
+  int32_t* o_pos = buf + off[1];
+  int32_t* o_seq = buf + off[2];
+  int32_t* o_qs = buf + off[3];
+  int32_t* o_len = buf + off[4];
+  int32_t* o_slot = buf + off[5];
+  int32_t* o_want = buf + off[6];
+  int32_t* o_feed = buf + off[9];
+  int64_t row = 0, wi = 0;
+  int n_feed = 0;
+  for (int e = 0; e < n; ++e) {
+    auto it = m->requests.find(ids[e]);
+    if (it == m->requests.end()) return CM_UNKNOWN;
+    const int32_t c = counts[e];
+    if (c <= 0) return CM_BAD_ARG;
+    if (feeds[e] >= 0) {
+      if (c != 1) return CM_BAD_ARG;
+      o_feed[2 * n_feed] = (int32_t)row;
+      o_feed[2 * n_feed + 1] = feeds[e];
+      ++n_feed;
+    }
+    for (int32_t i = 0; i < c; ++i) {
+      o_tok[row + i] = tokens[row + i];
+      o_pos[row + i] = starts[e] + i;
+      o_seq[row + i] = e;
+    }
+    for (int32_t w = 0; w < want_counts[e]; ++w) {
+      const int32_t place = wants[wi + w];
+      if (place < 0 || place >= c) return CM_BAD_ARG;
+      o_want[wi + w] = (int32_t)row + place;
+    }
+    wi += want_counts[e];
+    o_qs[e] = (int32_t)row;
+    o_len[e] = starts[e] + c;
+    o_slot[e] = it->second.state_slot;
+    row += c;
+  }
+  o_qs[n] = (int32_t)row;
+  const int64_t t = row;
+  for (int g = 0; g < (int)m->groups.size(); ++g) {
+    const int rc = cm_fill_step(h, g, n, ids, starts, counts, buf + off[7] + (int64_t)g * t,
+                                buf + off[8] + (int64_t)g * n * max_blocks, max_blocks);
+    if (rc != CM_OK) return rc;
+  }
+  return n_feed;
+}
+
 // Consistency: every page is either free or held by exactly one table entry, and likewise every state slot.
 int cm_check(void* h) {
   Manager* m = static_cast<Manager*>(h);

@@ -18,6 +18,7 @@ second time.
 from __future__ import annotations
 
 import dataclasses
+import itertools
 from collections import OrderedDict
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
@@ -224,8 +225,16 @@ class ModelRunner:
             if e.feed >= 0 and n != 1:
                 raise StepError(f"request {e.request}: only an entry of one token can be fed from the device")
 
+    @staticmethod
+    def _arrays(entries: Sequence[StepEntry]) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+        """(request ids, first positions, token counts) of the entries."""
+        s = len(entries)
+        return (np.fromiter((e.request for e in entries), dtype=np.int64, count=s),
+                np.fromiter((e.start for e in entries), dtype=np.int32, count=s),
+                np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=s))
+
     def _build(self, entries: Sequence[StepEntry], stage: _Staging, bucket: Optional[int],
-               feed_src: Optional[torch.Tensor] = None) -> StepContext:
+               feed_src: Optional[torch.Tensor] = None, arrays=None) -> StepContext:
         """Fill ``stage`` with the step's metadata, start its copy to the device and describe it.
 
         With ``bucket`` (decode graphs) every size is a function of (entries, bucket) alone, so the layout, and
@@ -233,9 +242,7 @@ class ModelRunner:
         """
         mgr = self.manager
         s = len(entries)
-        counts = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=s)
-        starts = np.fromiter((e.start for e in entries), dtype=np.int32, count=s)
-        ids = np.fromiter((e.request for e in entries), dtype=np.int64, count=s)
+        ids, starts, counts = arrays if arrays is not None else self._arrays(entries)
         t = int(counts.sum())
         n_want = sum(len(e.want) for e in entries)
         n_groups = len(self.pool.plan.groups)
@@ -264,32 +271,17 @@ class ModelRunner:
             total += arr.size
         stage.wait()
         buf = stage.ensure(total)
-        q_start = np.zeros(s + 1, dtype=np.int32)
-        np.cumsum(counts, out=q_start[1:])
-        row = 0
-        wi = o_want
-        n_feed = 0
-        for i, e in enumerate(entries):
-            n = counts[i]
-            if e.feed >= 0:
-                buf[o_feed + 2 * n_feed] = row
-                buf[o_feed + 2 * n_feed + 1] = e.feed
-                n_feed += 1
-            buf[o_tok + row: o_tok + row + n] = e.tokens
-            buf[o_pos + row: o_pos + row + n] = np.arange(e.start, e.start + n, dtype=np.int32)
-            buf[o_seq + row: o_seq + row + n] = i
-            for w in e.want:
-                buf[wi] = row + w
-                wi += 1
-            row += n
-        buf[o_qs: o_qs + s + 1] = q_start
-        buf[o_len: o_len + s] = starts + counts
-        slots = np.fromiter((mgr.state_slot(e.request) for e in entries), dtype=np.int32, count=s)
-        buf[o_slot: o_slot + s] = slots
-        for g in range(n_groups):
-            sm = buf[o_sm + g * t: o_sm + (g + 1) * t]
-            bt = buf[o_bt + g * s * max_blocks: o_bt + (g + 1) * s * max_blocks].reshape(s, max_blocks)
-            mgr.fill_step(g, ids, starts, counts, sm, bt)
+        # the arrays that depend on the entries alone are written by the host library in one call
+        if t == s:
+            tokens = np.fromiter((e.tokens[0] for e in entries), dtype=np.int32, count=s)
+        else:
+            tokens = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries), dtype=np.int32, count=t)
+        feeds = np.fromiter((e.feed for e in entries), dtype=np.int32, count=s)
+        want_counts = np.fromiter((len(e.want) for e in entries), dtype=np.int32, count=s)
+        wants = np.fromiter(itertools.chain.from_iterable(e.want for e in entries), dtype=np.int32, count=n_want)
+        offsets = np.asarray((o_tok, o_pos, o_seq, o_qs, o_len, o_slot, o_want, o_sm, o_bt, o_feed), dtype=np.int64)
+        n_feed = mgr.pack_step(ids, starts, counts, tokens, feeds, want_counts, wants, buf, offsets, max_blocks)
+        slots = buf[o_slot: o_slot + s].copy()
         for off, (_, arr, _) in zip(ex_off, extras):
             buf[off: off + arr.size] = arr.reshape(-1)
         stage.upload(total)
@@ -307,8 +299,9 @@ class ModelRunner:
             block_tables=[dev[o_bt + g * s * max_blocks: o_bt + (g + 1) * s * max_blocks].view(s, max_blocks)
                           for g in range(n_groups)],
             pool=self.pool, decode_bucket=bucket,
-            wants_all_rows=n_want == t and all(len(e.want) == len(e.tokens) and
-                                               all(w == j for j, w in enumerate(e.want)) for e in entries))
+            wants_all_rows=n_want == t and (t == s or all(len(e.want) == len(e.tokens) and
+                                                          all(w == j for j, w in enumerate(e.want))
+                                                          for e in entries)))
         for off, (key, arr, meta) in zip(ex_off, extras):
             ctx.plans[key] = (dev[off: off + arr.size].view(arr.shape), meta)
         return ctx
@@ -316,15 +309,16 @@ class ModelRunner:
     def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
         """Check the entries, reserve their pages and build the step's metadata on the device."""
         self._validate(entries)
-        for e in entries:
-            self.manager.reserve(e.request, e.start + len(e.tokens))
-        return self._build(entries, self._stage, None)
+        arrays = self._arrays(entries)
+        self.manager.reserve_all(*arrays)
+        return self._build(entries, self._stage, None, arrays=arrays)
 
-    def _finish(self, entries: Sequence[StepEntry]) -> None:
-        for e in entries:
-            done = e.start + len(e.tokens)
-            self._computed[e.request] = done
-            self.manager.release_behind(e.request, done)
+    def _finish(self, entries: Sequence[StepEntry], arrays) -> None:
+        ids, starts, counts = arrays
+        done = starts + counts
+        for e, d in zip(entries, done.tolist()):
+            self._computed[e.request] = d
+        self.manager.release_behind_all(ids, done)
 
     def step(self, entries: Sequence[StepEntry], feed_src: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run one batch; returns float32 logits [wanted places, vocab] (order: entries, then ``want``) or None.
@@ -335,20 +329,20 @@ class ModelRunner:
         the same shape: use it (sample, copy) before stepping again.
         """
         self._validate(entries)
-        for e in entries:
-            self.manager.reserve(e.request, e.start + len(e.tokens))
+        arrays = self._arrays(entries)
+        self.manager.reserve_all(*arrays)
         logits = None
-        if self.use_graphs and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries):
-            logits = self._decode_with_graph(entries, feed_src)
+        if self.use_graphs and int(arrays[2].max()) == 1 and all(len(e.want) == 1 for e in entries):
+            logits = self._decode_with_graph(entries, feed_src, arrays)
         if logits is None:
-            ctx = self._build(entries, self._stage, None, feed_src)
+            ctx = self._build(entries, self._stage, None, feed_src, arrays)
             logits = self.model.forward(ctx)
-        self._finish(entries)
+        self._finish(entries, arrays)
         return logits
 
-    def _decode_with_graph(self, entries: Sequence[StepEntry], feed_src=None) -> Optional[torch.Tensor]:
+    def _decode_with_graph(self, entries: Sequence[StepEntry], feed_src, arrays) -> Optional[torch.Tensor]:
         s = len(entries)
-        max_seq = max(e.start for e in entries) + 1
+        max_seq = int(arrays[1].max()) + 1
         key = (s, -(-max_seq // DECODE_BUCKET))
         g = self._graphs.get(key)
         if g is None:
@@ -358,7 +352,7 @@ class ModelRunner:
                 self._graphs.popitem(last=False)
             return None
         self._graphs.move_to_end(key)
-        ctx = self._build(entries, g.stage, key[1], feed_src)
+        ctx = self._build(entries, g.stage, key[1], feed_src, arrays)
         if g.graph is None:
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()

@@ -221,3 +221,95 @@ def test_admission_with_a_window_counts_what_everyone_will_need():
     w.free(2)
     assert w.can_admit(100, 4) and w.can_admit(100, 16) and not w.can_admit(100, 17)
     w.check()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_a_step_packed_in_one_call_equals_the_arrays_made_one_by_one(seed):
+    """``reserve_all`` / ``pack_step`` / ``release_behind_all`` against per-entry calls and arrays filled here."""
+    rng = random.Random(seed)
+    groups = [GroupGeometry(4, 200), GroupGeometry(16, 60, window=rng.choice([None, 24]))]
+    one, two = CacheManager(groups, 8), CacheManager(groups, 8)
+    held = {}
+    for step in range(12):
+        ids = [r for r in range(6) if rng.random() < 0.7]
+        if not ids:
+            continue
+        rng.shuffle(ids)
+        for r in ids:
+            if r not in held:
+                held[r] = 0
+                assert one.add(r) == two.add(r)
+        counts = [rng.choice([1, 1, 2, 7, 20]) for _ in ids]
+        starts = [held[r] for r in ids]
+        wants = [sorted(rng.sample(range(c), rng.randint(0, min(c, 3)))) for c in counts]
+        feeds = [rng.randint(0, 9) if c == 1 and rng.random() < 0.3 else -1 for c in counts]
+        tokens = [[rng.randrange(1000) for _ in range(c)] for c in counts]
+        a_ids = np.asarray(ids, dtype=np.int64)
+        a_starts, a_counts = np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32)
+        for r, s0, c in zip(ids, starts, counts):
+            one.reserve(r, s0 + c)
+        two.reserve_all(a_ids, a_starts, a_counts)
+        s, t, n_want = len(ids), sum(counts), sum(len(w) for w in wants)
+        max_blocks = -(-max(s0 + c for s0, c in zip(starts, counts)) // 4)
+        # the layout of the engine's staging buffer, with gaps of three between the arrays to catch overruns
+        sizes = [t, t, t, s + 1, s, s, n_want, 2 * t, 2 * s * max_blocks, 2 * s]
+        offs, total = [], 0
+        for n in sizes:
+            offs.append(total)
+            total += n + 3
+        buf = np.full(total, -7, dtype=np.int32)
+        n_feed = two.pack_step(a_ids, a_starts, a_counts, np.asarray(sum(tokens, []), dtype=np.int32),
+                               np.asarray(feeds, dtype=np.int32), np.asarray([len(w) for w in wants], dtype=np.int32),
+                               np.asarray(sum(wants, []), dtype=np.int32), buf, np.asarray(offs, dtype=np.int64),
+                               max_blocks)
+        want = np.full(total, -7, dtype=np.int32)
+        row, wi, pairs = 0, 0, []
+        for e, (r, s0, c) in enumerate(zip(ids, starts, counts)):
+            want[offs[0] + row: offs[0] + row + c] = tokens[e]
+            want[offs[1] + row: offs[1] + row + c] = range(s0, s0 + c)
+            want[offs[2] + row: offs[2] + row + c] = e
+            want[offs[3] + e] = row
+            want[offs[4] + e] = s0 + c
+            want[offs[5] + e] = one.state_slot(r)
+            for w in wants[e]:
+                want[offs[6] + wi] = row + w
+                wi += 1
+            if feeds[e] >= 0:
+                pairs += [row, feeds[e]]
+            row += c
+        want[offs[3] + s] = row
+        want[offs[9]: offs[9] + len(pairs)] = pairs
+        for g in range(2):
+            sm = np.zeros(t, dtype=np.int32)
+            bt = np.zeros((s, max_blocks), dtype=np.int32)
+            one.fill_step(g, a_ids, a_starts, a_counts, sm, bt)
+            want[offs[7] + g * t: offs[7] + (g + 1) * t] = sm
+            want[offs[8] + g * s * max_blocks: offs[8] + (g + 1) * s * max_blocks] = bt.reshape(-1)
+        assert n_feed == len(pairs) // 2
+        assert np.array_equal(buf, want)
+        for r, s0, c in zip(ids, starts, counts):
+            held[r] = s0 + c
+            one.release_behind(r, held[r])
+        two.release_behind_all(a_ids, np.asarray([held[r] for r in ids], dtype=np.int32))
+        for g in range(2):
+            assert one.num_free_pages(g) == two.num_free_pages(g)
+            for r in held:
+                assert one.table(r, g) == two.table(r, g)
+        for r in [r for r in held if rng.random() < 0.2]:
+            one.free(r)
+            two.free(r)
+            del held[r]
+        one.check()
+        two.check()
+    # a reservation that does not fit names its request; a wanted place outside an entry is refused
+    big = CacheManager([GroupGeometry(4, 3)], 2)
+    big.add(5)
+    big.add(6)
+    with pytest.raises(OutOfPages, match="request 6"):
+        big.reserve_all(np.asarray([5, 6], dtype=np.int64), np.asarray([0, 0], dtype=np.int32),
+                        np.asarray([8, 8], dtype=np.int32))
+    with pytest.raises(CacheError):
+        big.pack_step(np.asarray([5], dtype=np.int64), np.asarray([0], dtype=np.int32), np.asarray([2], dtype=np.int32),
+                      np.asarray([1, 2], dtype=np.int32), np.asarray([-1], dtype=np.int32),
+                      np.asarray([1], dtype=np.int32), np.asarray([2], dtype=np.int32), np.zeros(64, dtype=np.int32),
+                      np.arange(0, 60, 6, dtype=np.int64), 2)
