@@ -202,6 +202,26 @@ def try_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Op
     return None
 
 
+def _probe_addmm_out_dtype() -> bool:
+    doc = getattr(torch.addmm, "__doc__", "") or ""
+    return "out_dtype" in doc
+
+
+_ADDMM_OUT_DTYPE = _probe_addmm_out_dtype()
+
+
+def try_addmm_resid(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor) -> bool:
+    """``resid += x @ w^T`` by the library (hipBLASLt with beta = 1: the float32 sums of the product are added to the
+    float32 rows in place, so the product's own result is never written or read again), for products of more rows
+    than the streaming kernels take; False, nothing done, where that is not the choice."""
+    m = x.shape[0]
+    if not (_ADDMM_OUT_DTYPE and m > SKINNY_MAX_M and x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16
+            and resid.dtype is torch.float32 and resid.is_contiguous() and tuple(resid.shape) == (m, w.shape[0])):
+        return False
+    torch.addmm(resid, x, w.t(), out_dtype=torch.float32, out=resid)
+    return True
+
+
 def linear_planes(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
     """For M <= 64: float32 planes [slices, M, N] whose sum is x @ w^T (K split over the grid), else None."""
     m, k = x.shape

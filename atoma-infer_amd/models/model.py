@@ -14,6 +14,7 @@ import torch
 from ..config.base import ModelConfig
 from ..config.registry import Architecture, load_model_config
 from ..kernels.gemm_bf16 import Begun
+from ..parts.linear import Normed
 from ..weights.loader import load_into, load_random_into
 from .spec import ModelSpec
 
@@ -55,6 +56,8 @@ class Model:
             return None
         if isinstance(pending, Begun):      # the final norm, begun by the last product, on every row
             return spec.head[1].forward(pending)
+        if isinstance(pending, Normed):     # ... or finished behind it
+            return spec.head[1].forward(pending.data)
         x = spec.final_norm[1].add_norm(resid, pending, rows=ctx.want_rows)
         return spec.head[1].forward(x)
 

@@ -95,7 +95,8 @@ class Norm(Part):
     # them (``kernels.gemm_bf16.Begun``), which saves the norm's own launch where launches are what a step costs.
     # A norm that cannot says None, and the caller runs ``add_norm``.
     def add_product(self, resid: torch.Tensor, x, w: torch.Tensor):
-        """``resid += x @ w^T`` in place with this norm of the new rows begun, as ``Begun``; or None, nothing done."""
+        """``resid += x @ w^T`` in place with this norm of the new rows begun (``kernels.gemm_bf16.Begun``) or
+        finished (``parts.linear.Normed``); or None, nothing done."""
         return None
 
     def embed(self, table: torch.Tensor, tokens: torch.Tensor):

@@ -10,7 +10,7 @@ from typing import Dict
 
 from ..kernels.gemm_bf16 import Begun
 from .base import Block, FeedForward, Mixer, Norm, WeightSpec, register_block
-from .linear import ResidualSink
+from .linear import Normed, ResidualSink
 
 
 class PreNormBlock(Block):
@@ -43,7 +43,11 @@ class PreNormBlock(Block):
     @staticmethod
     def _normed(norm, resid, pending, reader):
         """The input of ``reader``: ``pending`` is either a delta still to be added and normed, or ``norm`` already
-        begun by the product that made it (which has also added it to ``resid``)."""
+        begun or finished by the product that made it (which has also added it to ``resid``)."""
+        if isinstance(pending, Normed):
+            if pending.norm is not norm:
+                raise RuntimeError("a finished norm reached another norm than the one it was made for")
+            return pending.data
         if isinstance(pending, Begun):
             if pending.norm is not norm:
                 raise RuntimeError("a begun norm reached another norm than the one it was begun for")

@@ -26,6 +26,14 @@ class ResidualSink:
     norm: object
 
 
+@dataclasses.dataclass
+class Normed:
+    """What a product handed to a ``ResidualSink`` may return instead of a delta: the residual rows have the product
+    added already, and ``data`` is ``norm`` of the new rows, finished."""
+    data: torch.Tensor
+    norm: object
+
+
 def as_tensor(x) -> torch.Tensor:
     """``x`` as a tensor: a begun norm is finished."""
     return x.tensor() if isinstance(x, Begun) else x
@@ -47,8 +55,9 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
 def linear_delta(x, w: torch.Tensor, sink: Optional[ResidualSink] = None):
     """A product whose result is only ever added to the residual stream.
 
-    With a ``sink`` whose norm can, the product adds itself to the residual rows and begins that norm: the result
-    is then a ``Begun`` norm, not a delta, and the caller hands it on as it is.  Otherwise the delta comes back for
+    With a ``sink`` whose norm can, the product adds itself to the residual rows and begins that norm (few rows) or
+    the norm follows at once (many rows): the result is then a ``Begun`` norm or a ``Normed`` one, not a delta, and
+    the caller hands it on as it is.  Otherwise the delta comes back for
     ``Norm.add_norm``: for few rows as float32 planes [slices, M, N] of a K-split product, which ``add_norm`` sums
     (the split keeps the whole GPU busy on a small product and costs no extra kernel).
     """

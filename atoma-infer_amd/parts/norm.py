@@ -35,15 +35,20 @@ class RMSNorm(Norm):
     def add_norm(self, resid, delta, rows=None):
         return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.act_dtype, rows)
 
-    # the norm begun by its neighbours (bfloat16 steps of at most 16 rows): see kernels/gemm_bf16.py
+    # the norm begun by its neighbours (bfloat16 steps of at most 16 rows): see kernels/gemm_bf16.py; with many rows
+    # the library adds its product to the residual rows itself, and the norm reads them once
     def add_product(self, resid, x, w):
         if self.act_dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16:
             return None
         from ..kernels import gemm_bf16
+        from .linear import Normed, as_tensor
         y = gemm_bf16.try_linear_resid(x, w, resid, self.weight, self.eps)
         if y is not None:
             y.norm = self
-        return y
+            return y
+        if gemm_bf16.try_addmm_resid(as_tensor(x), w, resid):
+            return Normed(self.add_norm(resid, None), self)
+        return None
 
     def embed(self, table, tokens):
         if self.act_dtype is not torch.bfloat16 or tokens.numel() > 16 or table.shape[1] != self.width:
