@@ -482,11 +482,14 @@ extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M,
   }
   ATOMA_RESID(1, 1, 4, 4, false)
   ATOMA_RESID(1, 1, 8, 4, false)
+  ATOMA_RESID(1, 1, 8, 2, false)
+  ATOMA_RESID(1, 1, 8, 8, false)
   ATOMA_RESID(1, 4, 1, 4, false)
   ATOMA_RESID(1, 1, 4, 4, true)
   ATOMA_RESID(1, 1, 4, 8, true)
   ATOMA_RESID(1, 1, 8, 4, true)
   ATOMA_RESID(1, 1, 8, 8, true)
+  ATOMA_RESID(1, 1, 8, 2, true)
   ATOMA_RESID(1, 4, 1, 4, true)
 #undef ATOMA_RESID
   return ATOMA_ERR_SHAPE;

@@ -292,16 +292,21 @@ def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, c
 
 
 def resid_plan(m: int, n: int, k: int):
-    """(rows-of-16 per wave, waves splitting K, steps of K per batch of loads) of the product that adds into the residual stream: K is split over
-    the waves of a workgroup only (every sum has one owner, which also begins the norm), as many ways as K allows,
-    and a wave owns 8 rows of the weight, so that N = 2048 still makes 256 workgroups (measured at Llama 1B's o and
-    down products: 5.3 and 12.7 us against 5.9 and 15.0 with 16 rows a wave)."""
+    """(tiles of 16 rows of the weight per wave, waves splitting K, steps of K per batch of loads, half tiles) of the
+    product that adds into the residual stream: K is split over the waves of a workgroup only (every sum has one
+    owner, which also begins the norm), as many ways as K allows.  With N up to 2,048 a wave owns 8 rows of the
+    weight, not 16, so that 256 workgroups share the product (measured at Llama 1B's o and down products: 5.3 and
+    12.7 us against 5.9 and 15.0 with 16 rows a wave); wider outputs fill the GPU with whole tiles, and half tiles
+    cost them a third more (Llama 3B: 7.8 and 15.0 us against 10.5 and 21.4; 8B: 9.6 and 27.0 against 12.9 and 35.9)."""
     wk = 8
     while wk > 1 and k % (32 * wk):
         wk //= 2
     if wk == 2:
         wk = 1
-    return 1, wk, 4, 1
+    half = 1 if n <= 2048 else 0
+    depths = {(8, 1): (4, 2, 8), (8, 0): (8, 4, 2), (4, 1): (4, 8), (4, 0): (4,), (1, 1): (4,), (1, 0): (4,)}[(wk, half)]
+    depth = next((d for d in depths if k % (32 * wk * d) == 0), 4)
+    return 1, wk, depth, half
 
 
 def try_linear_resid(x, w: torch.Tensor, resid: torch.Tensor, gamma: torch.Tensor, eps: float) -> Optional[Begun]:

@@ -591,7 +591,7 @@ def _rms(x, g, eps):
 
 
 @pytest.mark.parametrize("m", [1, 5, 8, 16])
-@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (96, 64), (200, 96), (3072, 512)])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (96, 64), (200, 96), (3072, 512), (3072, 1024), (4096, 2048)])
 @pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
 def test_product_into_the_residual_begins_the_norm(m, n, k, gdt):
     """``resid += x w^T`` with the following RMSNorm begun in the product's epilogue (residual times norm weight and
