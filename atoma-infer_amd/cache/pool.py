@@ -7,8 +7,9 @@ backends/vllm/src/worker.rs:570-598).  Keys and values of an entry are [pages, k
 a (page, head) tile is contiguous, and the order of its elements is the one in which the MFMA attention kernel's
 lanes read them (``cache/layout.py`` and csrc/kernels/cache_layout.h state it).
 
-Mixers that declare a ``StateSpec`` get a float32 tensor [slots, *shape] per layer call, indexed by the
-request's state slot.
+Mixers that declare a ``StateSpec`` get a tensor [slots, *shape] (float32 unless the spec says otherwise) per layer
+call, indexed by the request's state slot.  A ``CacheSpec`` may ask for values of another width than the keys, or for
+no second tensor at all.
 """
 from __future__ import annotations
 
@@ -27,7 +28,7 @@ class GroupPlan:
     calls: List[int]          # run-order positions that own an entry of this group
 
     def bytes_per_token(self, elem: int) -> int:
-        return 2 * len(self.calls) * self.spec.kv_heads * self.spec.head_size * elem
+        return len(self.calls) * self.spec.kv_heads * (self.spec.head_size + self.spec.value_elements) * elem
 
 
 @dataclasses.dataclass
@@ -35,8 +36,8 @@ class CachePlan:
     groups: List[GroupPlan]
     #: run-order position -> (group, entry within group, writable); absent for calls whose mixer keeps no cache
     where: Dict[int, Tuple[int, int, bool]]
-    #: run-order position -> state shape
-    states: Dict[int, Tuple[int, ...]]
+    #: run-order position -> (state shape, dtype name)
+    states: Dict[int, Tuple[Tuple[int, ...], str]]
 
     def bytes_per_token(self, elem: int) -> int:
         return sum(g.bytes_per_token(elem) for g in self.groups)
@@ -46,12 +47,12 @@ def plan_cache(spec) -> CachePlan:
     groups: List[GroupPlan] = []
     index: Dict[CacheSpec, int] = {}
     where: Dict[int, Tuple[int, int, bool]] = {}
-    states: Dict[int, Tuple[int, ...]] = {}
+    states: Dict[int, Tuple[Tuple[int, ...], str]] = {}
     for pos, call in enumerate(spec.run_order):
         mixer = spec.layers[call.layer][1].mixer
         st = mixer.state_spec()
         if st is not None:
-            states[pos] = tuple(st.shape)
+            states[pos] = (tuple(st.shape), st.dtype)
         cs = mixer.cache_spec()
         if cs is None:
             continue
@@ -78,7 +79,7 @@ class LayerCache:
     group: int = -1
     slot_mapping: Optional[torch.Tensor] = None     # [T] int32: page * page_size + offset of each token
     block_tables: Optional[torch.Tensor] = None     # [S, blocks] int32
-    state: Optional[torch.Tensor] = None            # [slots, *shape] float32
+    state: Optional[torch.Tensor] = None            # [slots, *shape], float32 unless the StateSpec says otherwise
 
 
 class CachePool:
@@ -91,29 +92,31 @@ class CachePool:
         self.plan, self.page_size, self.dtype, self.device = plan, int(page_size), dtype, device
         self.num_state_slots = int(num_state_slots)
         self.k: List[torch.Tensor] = []
-        self.v: List[torch.Tensor] = []
+        self.v: List[Optional[torch.Tensor]] = []       # None for a group whose mixers keep one tensor only
         geometry = []
         for g, n in zip(plan.groups, num_pages):
             cs = g.spec
             # zero-filled, so that pages never written hold finite numbers
-            tile = page_size * cs.head_size
-            self.k.append(torch.zeros((len(g.calls), n, cs.kv_heads, tile), dtype=dtype, device=device))
-            self.v.append(torch.zeros((len(g.calls), n, cs.kv_heads, tile), dtype=dtype, device=device))
+            self.k.append(torch.zeros((len(g.calls), n, cs.kv_heads, page_size * cs.head_size), dtype=dtype,
+                                      device=device))
+            self.v.append(torch.zeros((len(g.calls), n, cs.kv_heads, page_size * cs.value_elements), dtype=dtype,
+                                      device=device) if cs.value_elements else None)
             geometry.append(GroupGeometry(page_size, n, cs.window))
-        self.states = {pos: torch.zeros((num_state_slots, *shape), dtype=torch.float32, device=device)
-                       for pos, shape in plan.states.items()}
+        self.states = {pos: torch.zeros((num_state_slots, *shape), dtype=getattr(torch, dt), device=device)
+                       for pos, (shape, dt) in plan.states.items()}
         self.manager = CacheManager(geometry, num_state_slots)
 
     def layer_cache(self, pos: int, slot_mappings, block_tables) -> LayerCache:
         lc = LayerCache(state=self.states.get(pos))
         if pos in self.plan.where:
             g, e, writable = self.plan.where[pos]
-            lc.k, lc.v, lc.page_size, lc.writable, lc.group = self.k[g][e], self.v[g][e], self.page_size, writable, g
+            lc.k, lc.page_size, lc.writable, lc.group = self.k[g][e], self.page_size, writable, g
+            lc.v = self.v[g][e] if self.v[g] is not None else None
             lc.slot_mapping, lc.block_tables = slot_mappings[g], block_tables[g]
         return lc
 
     def bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.k + self.v)
+        return sum(t.numel() * t.element_size() for t in self.k + self.v if t is not None)
 
 
 def pages_for_tokens(plan: CachePlan, page_size: int, max_tokens: int, max_requests: int) -> List[int]:

@@ -42,16 +42,36 @@ class CacheSpec:
 
     ``window``: None keeps every token; w keeps the last w.  Layers whose specs are equal share one
     group of pages and one block table per request.
+
+    ``value_size``: elements per head and token of the second tensor, when it is not as wide as the first: None
+    means ``head_size``; 0 means that the mixer keeps one tensor only (a latent vector per token, say) and its
+    ``LayerCache.v`` is None.  How a mixer orders the ``page_size * size`` elements of a (page, head) tile is its own
+    affair; the pool only hands out the tiles.
     """
     kv_heads: int
     head_size: int
     window: Optional[int] = None
+    value_size: Optional[int] = None
+
+    def __post_init__(self):
+        if self.kv_heads <= 0 or self.head_size <= 0 or (self.value_size is not None and self.value_size < 0):
+            raise ValueError(f"invalid cache spec: {self}")
+
+    @property
+    def value_elements(self) -> int:
+        return self.head_size if self.value_size is None else self.value_size
 
 
 @dataclasses.dataclass(frozen=True)
 class StateSpec:
-    """Per-request state of fixed size that a mixer keeps: ``shape`` float32 numbers per request."""
+    """Per-request state of fixed size that a mixer keeps: ``shape`` numbers per request, float32 unless ``dtype``
+    ("float32", "bfloat16", "int32") says otherwise; zero at admission."""
     shape: Tuple[int, ...]
+    dtype: str = "float32"
+
+    def __post_init__(self):
+        if self.dtype not in ("float32", "bfloat16", "int32"):
+            raise ValueError(f"state dtype must be float32, bfloat16 or int32, not {self.dtype!r}")
 
 
 WeightGetter = Callable[[str], torch.Tensor]

@@ -481,7 +481,7 @@ def test_toy_cache_plan(toy_dir):
     # attention calls 0, 3, 5 keep all keys (one group), call 2 keeps a window (a group of its own),
     # call 6 reads call 0's entry, calls 1 and 4 each have their own state
     assert [(g.spec.window, g.calls) for g in plan.groups] == [(None, [0, 3, 5]), (24, [2])]
-    assert plan.where[6] == (0, 0, False) and sorted(plan.states) == [1, 4] and plan.states[1] == (40,)
+    assert plan.where[6] == (0, 0, False) and sorted(plan.states) == [1, 4] and plan.states[1] == ((40,), "float32")
 
 
 def _toy_run(model, plan, reqs, schedule, pages):
@@ -803,3 +803,170 @@ def test_toy_state_survives_preemption(toy_dir):
     assert eng.stats["preemptions"] > 0
     assert [o.inference_outputs[0].token_ids for o in outs] == want
     assert eng.runner.manager.num_requests() == 0
+
+
+# ----------------------------------------------------------------------------------------------------------
+# a mixer whose cache is one latent vector per token, and whose state is a counter of integers
+
+
+def _latent_parts():
+    """Attention over cached latent vectors: a token leaves c = x Wc^T (``latent`` numbers, one head, no second
+    tensor) in its page; a query head scores the latents themselves and sums them, and Wo maps the heads' sums back.
+    The state counts, in int32, the tokens the request has brought."""
+    from atoma_infer_amd.parts import CacheSpec, Mixer, StateSpec, WeightSpec, register_mixer
+
+    class LatentMixer(Mixer):
+        def __init__(self, width: int, latent: int, heads: int):
+            self.width, self.latent, self.heads = width, latent, heads
+
+        def weight_specs(self):
+            return {"c_proj.weight": WeightSpec((self.latent, self.width)),
+                    "q_proj.weight": WeightSpec((self.heads * self.latent, self.width)),
+                    "o_proj.weight": WeightSpec((self.width, self.heads * self.latent))}
+
+        def load(self, get, device, act_dtype):
+            self.wc, self.wq, self.wo = (get(n + ".weight").to(device).float() for n in ("c_proj", "q_proj", "o_proj"))
+
+        def cache_spec(self):
+            return CacheSpec(kv_heads=1, head_size=self.latent, value_size=0)
+
+        def state_spec(self):
+            return StateSpec((1,), "int32")
+
+        def forward(self, x, ctx, cache):
+            assert cache.v is None and cache.state.dtype is torch.int32
+            L, page = self.latent, cache.page_size
+            xf = x.float()
+            lat = cache.k.view(-1, L)                     # this mixer's tile order: token after token
+            lat[cache.slot_mapping.long()] = (xf @ self.wc.T).to(lat.dtype)
+            q = (xf @ self.wq.T).view(-1, self.heads, L)
+            out = torch.empty_like(q)
+            row = 0
+            for e in range(ctx.n_entries):
+                start, n = int(ctx.h_starts[e]), int(ctx.h_counts[e])
+                slot = int(ctx.h_state_slots[e])
+                assert int(cache.state[slot, 0]) == start, "the counter follows the request, whatever its slot was"
+                cache.state[slot, 0] += n
+                total = start + n
+                pages = cache.block_tables[e, : -(-total // page)].long()
+                seen = cache.k.view(-1, page, L)[pages].reshape(-1, L)[:total].float()
+                s = torch.einsum("nhl,sl->hns", q[row: row + n], seen) / math.sqrt(L)
+                far = torch.arange(total, device=x.device)[None, :] > (start + torch.arange(n, device=x.device))[:, None]
+                p = torch.softmax(s.masked_fill(far[None], float("-inf")), dim=-1)
+                out[row: row + n] = torch.einsum("hns,sl->nhl", p, seen)
+                row += n
+            return (out.reshape(-1, self.heads * L) @ self.wo.T).to(x.dtype)
+
+    register_mixer("toy_latent", LatentMixer, replace=True)
+
+
+TOY_LATENT = {"architectures": ["ToyLatentForCausalLM"], "width": 80, "vocab": 211, "latent": 24, "heads": 3,
+              "attn_heads": 5, "attn_kv_heads": 1, "inter": 112, "depth": 3, "eps": 1e-5, "max_positions": 256}
+
+
+def _latent_architecture():
+    from atoma_infer_amd.config import ModelConfig, key, register_architecture
+    from atoma_infer_amd.config.base import as_float, as_positive_int
+    from atoma_infer_amd.models import ModelSpec
+    from atoma_infer_amd.parts import OutputHead, TokenEmbedding, make_part
+
+    @dataclasses.dataclass(frozen=True)
+    class LatentConfig(ModelConfig):
+        architectures = ("ToyLatentForCausalLM",)
+        width: int = key(convert=as_positive_int)
+        vocab: int = key(convert=as_positive_int)
+        latent: int = key(convert=as_positive_int)
+        heads: int = key(convert=as_positive_int)
+        attn_heads: int = key(convert=as_positive_int)
+        attn_kv_heads: int = key(convert=as_positive_int)
+        inter: int = key(convert=as_positive_int)
+        depth: int = key(convert=as_positive_int)
+        eps: float = key(convert=as_float)
+        max_positions: int = key(convert=as_positive_int)
+
+        def to_dict(self):
+            d = {f.name: getattr(self, f.name) for f in dataclasses.fields(self)}
+            d["architectures"] = ["ToyLatentForCausalLM"]
+            return d
+
+    def build(cfg: LatentConfig) -> ModelSpec:
+        norm = lambda: make_part("norm", "rmsnorm", width=cfg.width, eps=cfg.eps)
+        hd = cfg.width // cfg.attn_heads
+        layers = []
+        for i in range(cfg.depth):
+            if i % 2 == 0:
+                mixer = make_part("mixer", "toy_latent", width=cfg.width, latent=cfg.latent, heads=cfg.heads)
+            else:       # the framework's attention between them: its keys and values lie in a group of their own
+                pos = make_part("position", "rotary", head_size=hd, theta=10000.0, max_positions=cfg.max_positions)
+                mixer = make_part("mixer", "attention", width=cfg.width, num_heads=cfg.attn_heads,
+                                  num_kv_heads=cfg.attn_kv_heads, head_size=hd, position=pos)
+            ffn = make_part("feed_forward", "swiglu", width=cfg.width, intermediate=cfg.inter)
+            layers.append((f"lat.layers.{i}", make_part("block", "pre_norm", norm1=norm(), mixer=mixer, norm2=norm(),
+                                                        feed_forward=ffn, names=("n1", "mix", "n2", "ffn"))))
+        return ModelSpec(width=cfg.width, vocab_size=cfg.vocab, max_positions=cfg.max_positions,
+                         embedding=("lat.embed", TokenEmbedding(cfg.vocab, cfg.width)), layers=layers,
+                         final_norm=("lat.final_norm", norm()), head=("lat.head", OutputHead(cfg.width, cfg.vocab)))
+
+    register_architecture("ToyLatentForCausalLM", LatentConfig, build, replace=True)
+
+
+def latent_plain_forward(tokens: List[int], w: Dict[str, torch.Tensor], cfg: dict) -> torch.Tensor:
+    H, L, nh, t = cfg["width"], cfg["latent"], cfg["heads"], len(tokens)
+    ah, akv = cfg["attn_heads"], cfg["attn_kv_heads"]
+    hd = H // ah
+    rms = lambda x, g: x / torch.sqrt((x * x).mean(-1, keepdim=True) + cfg["eps"]) * g
+    c, s = P.rope_tables({"hidden_size": H, "num_attention_heads": ah, "rope_theta": 10000.0}, torch.arange(t))
+    x = w["lat.embed.weight"][torch.tensor(tokens)]
+    for i in range(cfg["depth"]):
+        p = f"lat.layers.{i}."
+        h = rms(x, w[p + "n1.weight"])
+        if i % 2 == 0:
+            lat = h @ w[p + "mix.c_proj.weight"].T
+            q = (h @ w[p + "mix.q_proj.weight"].T).view(t, nh, L).transpose(0, 1)
+            kv = lat[None].expand(nh, t, L)
+            o = P.attention_scores_softmax_pv(q, kv, kv, 1 / math.sqrt(L), True, None)
+            x = x + o.transpose(0, 1).reshape(t, nh * L) @ w[p + "mix.o_proj.weight"].T
+        else:
+            q = P.apply_rope((h @ w[p + "mix.q_proj.weight"].T).view(t, ah, hd), c, s)
+            k = P.apply_rope((h @ w[p + "mix.k_proj.weight"].T).view(t, akv, hd), c, s)
+            v = (h @ w[p + "mix.v_proj.weight"].T).view(t, akv, hd)
+            kk, vv = k.repeat_interleave(ah // akv, 1), v.repeat_interleave(ah // akv, 1)
+            o = P.attention_scores_softmax_pv(q.transpose(0, 1), kk.transpose(0, 1), vv.transpose(0, 1),
+                                              1 / math.sqrt(hd), True, None)
+            x = x + o.transpose(0, 1).reshape(t, H) @ w[p + "mix.o_proj.weight"].T
+        x = x + P.swiglu_mlp(rms(x, w[p + "n2.weight"]), w, p + "ffn.")
+    return rms(x, w["lat.final_norm.weight"]) @ w["lat.head.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_cache_of_latent_vectors_and_a_state_of_integers(tmp_path, dtype):
+    """A mixer that keeps one tensor per token, of a width of its own and in a tile order of its own, beside layers
+    of the framework's attention: the pool gives it pages of its own group and no second tensor, its state is
+    int32, and the steps (portions beside decoded tokens, pages reused) equal the whole-sequence formula."""
+    from atoma_infer_amd.cache import plan_cache
+    from atoma_infer_amd.config import unregister_architecture
+    from atoma_infer_amd.models import load_model
+    from atoma_infer_amd.parts import CacheSpec
+    from atoma_infer_amd.weights import write_random_model
+    _latent_parts()
+    _latent_architecture()
+    try:
+        d = write_random_model(str(tmp_path / "lat"), TOY_LATENT, seed=6, dtype="bfloat16", norm_jitter=0.1)
+        model = load_model(d, dtype)
+        plan = plan_cache(model.spec)
+        assert [(g.spec, g.calls) for g in plan.groups] == [
+            (CacheSpec(1, 24, None, 0), [0, 2]), (CacheSpec(1, 16, None), [1])]
+        elem = 2
+        assert plan.bytes_per_token(elem) == (2 * 24 + 2 * 16) * elem
+        assert plan.states == {0: ((1,), "int32"), 2: ((1,), "int32")}
+        w = plain_weights(d)
+        reqs = {n: random_tokens(ln, TOY_LATENT["vocab"], 70 + i) for i, (n, ln) in enumerate([("a", 90), ("b", 41), ("c", 60)])}
+        want = {n: latent_plain_forward(t, w, TOY_LATENT) for n, t in reqs.items()}
+        sched = [([("a", 50)], []), ([("a", 3), ("b", 30)], []), ([("a", 1), ("b", 1)], []), ([("b", 10), ("a", 36)], ["a", "b"]),
+                 ([("c", 17)], []), ([("c", 2)], []), ([("c", 1)], []), ([("c", 40)], ["c"])]
+        got, runner = _toy_run(model, plan, reqs, sched, [9, 9])
+        _toy_check(got, want, dtype)
+        assert runner.pool.v[0] is None and runner.pool.v[1] is not None
+        assert runner.manager.num_free_pages(0) == 9 and runner.manager.num_free_pages(1) == 9
+    finally:
+        unregister_architecture("ToyLatentForCausalLM")
