@@ -79,10 +79,10 @@ __device__ __forceinline__ bf16x8 pack8(const float* v) {
 //          second kernel (there are enough requests and KV heads to fill the GPU without cutting keys into tasks).
 // RT: pieces of 32 rows a wave works on, against the same keys: with two, every fragment of keys and values that a
 // wave fetches, and the page and loop arithmetic of a block, serve 64 rows.  A wave's pace is set by its vector
-// instructions (about a hundred a block and piece, of which some 35 are that arithmetic), so portions behind long
-// prefixes gain (2,048 tokens behind 30,720: 882 -> 755 us at head size 64); short prompts lose, because twice as
-// few waves, each with a chain twice as long, fill the GPU worse (2,048 tokens alone: 43 -> 54 us).  The host asks
-// for two pieces from 16,384 keys on.
+// instructions (about a hundred a block and piece, a third of their time the sixteen exponentials), so portions
+// behind long prefixes gain (2,048 tokens behind 30,720: 741 -> 682 us at head size 64, behind 63,488: 1,495 ->
+// 1,355, behind 14,336: 376 -> 363); short prompts lose, because twice as few waves, each with a chain twice as
+// long, fill the GPU worse.  The host asks for two pieces from 16,384 keys on.
 template <int TASKS, int KSPLIT, int RT = 1>
 __global__ void __launch_bounds__(64 * TASKS * KSPLIT)
 attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
@@ -90,7 +90,8 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
                       float* __restrict__ part_o, float* __restrict__ part_lse, const Task* __restrict__ tasks,
                       int n_tasks, const int32_t* __restrict__ block_tables, int max_blocks, float scale,
                       int window, int nh, int nkv) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // (a wave's number is the same in all its lanes; saying so keeps what follows from it in scalar registers)
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave % TASKS, part = wave / TASKS;   // which of the workgroup's tasks, which share of its keys
   // workgroups are numbered with the KV head running fastest: neighbours read the same block tables and finish
   // together, and the longest tasks (which come first) start first.  The GPU deals workgroups to its eight XCDs in
@@ -163,6 +164,8 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     p_lo = min(p_lo, __shfl_xor(p_lo, off, 64));
     lo_hi = max(lo_hi, __shfl_xor(lo_hi, off, 64));
   }
+  p_lo = __builtin_amdgcn_readfirstlane(p_lo);       // (all lanes hold the same by now)
+  lo_hi = __builtin_amdgcn_readfirstlane(lo_hi);
 
   const float sc2 = scale * kLog2e;
   float m[RT], l[RT];
@@ -179,11 +182,16 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const size_t kv_head_stride = (size_t)PAGE * HD;            // one (page, head) tile
   const size_t page_stride = (size_t)nkv * kv_head_stride;
 
+  // Page numbers are the same in all lanes, so a tile's address is scalar arithmetic and a lane adds its own
+  // offset, which never changes: tile order (cache_layout.h): keys: for each 16 columns, the 8-column pieces of all 16
+  // tokens side by side; values: this lane's eight key slots of column d are one 16-byte piece.
+  const uint16_t* const k_tiles = kcache + (size_t)kvh * kv_head_stride;
+  const uint16_t* const v_tiles = vcache + (size_t)kvh * kv_head_stride;
+  const uint32_t k_lane = (uint32_t)(hg * PAGE + (c & 15)) * 8;
   auto load_keys = [&](int p0, int p1, bf16x8* kf) {
-    const int pg = (c < 16) ? p0 : p1;
-    // tile order (cache_layout.h): for each 16 columns, the 8-column pieces of all 16 tokens side by side
-    const uint16_t* kp = kcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride +
-                         (size_t)(hg * PAGE + (c & 15)) * 8;
+    const uint16_t* const t0 = k_tiles + (size_t)__builtin_amdgcn_readfirstlane(p0) * page_stride;
+    const uint16_t* const t1 = k_tiles + (size_t)__builtin_amdgcn_readfirstlane(p1) * page_stride;
+    const uint16_t* kp = ((c < 16) ? t0 : t1) + k_lane;
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) kf[st] = *reinterpret_cast<const bf16x8*>(kp + st * (2 * PAGE * 8));
   };
@@ -191,17 +199,15 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   auto load_vals = [&](int p0, int p1, bf16x8 (*vf)[DTILES]) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int pg = j ? p1 : p0;
+      const uint16_t* const tile = v_tiles + (size_t)__builtin_amdgcn_readfirstlane(j ? p1 : p0) * page_stride;
 #pragma unroll
       for (int dt = 0; dt < DTILES; ++dt) {
         const int d = dt * 32 + c;
         if (HD % 32 == 0 || d < HD) {
-          // tile order (cache_layout.h): this lane's eight key slots of column d are one 16-byte piece
           constexpr int last_rows = HD % 32 == 0 ? 32 : HD % 32;
           const int rows = (HD % 32 == 0 || dt < DTILES - 1) ? 32 : last_rows;
-          const uint16_t* vp = vcache + (size_t)pg * page_stride + (size_t)kvh * kv_head_stride + dt * 512 +
-                               (size_t)(hg * rows + c) * 8;
-          vf[j][dt] = *reinterpret_cast<const bf16x8*>(vp);
+          const uint32_t v_lane = (uint32_t)(dt * 512 + (hg * rows + c) * 8);
+          vf[j][dt] = *reinterpret_cast<const bf16x8*>(tile + v_lane);
         } else {
 #pragma unroll
           for (int i = 0; i < 8; ++i) vf[j][dt][i] = (__bf16)0.f;
@@ -300,8 +306,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
         sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -m_use));
         psum += sv[i];
       }
-      psum += from_other_half(psum, hg != 0);
-      l[t] += psum;
+      l[t] += psum;      // this lane's half of the row's sum; the halves meet after the last block
 
       // O^T += V^T P^T
       const bf16x8 pf0 = pack8(sv), pf1 = pack8(sv + 8);
@@ -357,6 +362,10 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
       }
     }
   }
+
+  // a row's sum of weights: its two lanes have each summed the keys they hold (both scaled by the same m)
+#pragma unroll
+  for (int t = 0; t < RT; ++t) l[t] += from_other_half(l[t], hg != 0);
 
   // accumulator element i of tile dt is d = dt*32 + (i/4)*8 + hg*4 + i%4 of row c
   if (task.dest < 0) {
