@@ -7,7 +7,7 @@
 // kernels: csrc/src/lib.rs:69-100).  The four waves of a workgroup run four consecutive tasks; the host orders
 // tasks so that these read the same keys (the heads of one tile, or neighbouring key ranges of one request) and
 // meet in the L1 cache.  A task either covers all keys its rows may see and writes the output, or covers one
-// chunk of 64 to 256 keys and writes a partial result (normalised output and log-sum-exp) that the combine kernel merges:
+// chunk of 128 to 512 keys and writes a partial result (normalised output and log-sum-exp) that the combine kernel merges:
 // the split keeps the GPU busy when few rows face many keys (csrc/kernels/flash_fwd_kernel.h:1131-1310 is the
 // reference's combine).  Chunk borders are multiples of the chunk size, so a partial result covers the same keys
 // whatever else the batch holds.
