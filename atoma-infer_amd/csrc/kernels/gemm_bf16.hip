@@ -50,9 +50,13 @@ struct FuseArgs {
   float* ss_out;
 };
 
-// HALF (one tile of W, at most 16 rows of A, the residual epilogue): a wave owns 8 rows of W, not 16; the lanes of
-// the other 8 rows load nothing.  Twice as many workgroups then share a small N, and what a workgroup may have in
-// flight, not the matrix cores, is what bounds these products.
+// HALF (one tile of W, at most 16 rows of A, the residual epilogue): a wave owns 8 rows of W, not 16, so that twice
+// as many workgroups share a small N; what a workgroup may have in flight, not the matrix cores, is what bounds
+// these products.  The lanes of the tile's other 8 rows load the same 8 rows of W 32 values of K further on, so a
+// step covers 64 values of K and every lane's load is used: the step's two MFMAs take the one fragment of W
+// against the activations of its first and of its second 32 values, into two accumulators; rows 0..7 of the first
+// and rows 8..15 of the second are the wave's sums (the other halves are products of mismatched K and are dropped),
+// and they meet once, after the last step.
 template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false, bool ROPE = false, int UO = 0,
           bool HALF = false>
 __global__ void __launch_bounds__(64 * WN * WK)
@@ -67,8 +71,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   const int r16 = lane & 15, kg = lane >> 4;
   static_assert(!HALF || (RT == 1 && MT == 1 && !SWIGLU && !ROPE), "half tiles: one tile, residual epilogue");
   const int n_base = (blockIdx.x * WN + wn) * (HALF ? 8 : RT * 16);
-  const bool w_on = !HALF || r16 < 8;                 // this lane loads a row of W
-  const bool a_on = !HALF || M > 8 || r16 < 8;        // ... and a row of A
+  constexpr int KSTEP = HALF ? 64 : 32;               // values of K that a wave's step covers
   const int k_slices = gridDim.y * WK;
   const int k_len = K / k_slices;
   const int k_begin = (blockIdx.y * WK + wk) * k_len;
@@ -77,9 +80,9 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   const uint16_t* wp[RT];
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
-    int n = n_base + r * 16 + r16;
+    int n = n_base + r * 16 + (HALF ? (r16 & 7) : r16);
     if (n > N - 1) n = N - 1;
-    wp[r] = w + (size_t)n * ldw + k_begin + kg * 8;
+    wp[r] = w + (size_t)n * ldw + k_begin + kg * 8 + ((HALF && r16 >= 8) ? 32 : 0);
   }
   const uint16_t* ap[MT];
 #pragma unroll
@@ -94,6 +97,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   for (int r = 0; r < RT; ++r)
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[r][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 acc_hi = f32x4{0.f, 0.f, 0.f, 0.f};           // HALF: the sums over the second 32 values of every step
 
   // what the fused norm needs from memory is asked for first, so that it has arrived when the sums are done
   // The shares of the rows' sums of squares are added by all waves of the workgroup, up to sixteen per lane and row,
@@ -122,28 +126,30 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   }
 
   // two buffers of U steps each: while the MFMAs of one run, the loads of the other are in flight
-  bf16x8 wf[2][U][RT], af[2][U][MT];
+  bf16x8 wf[2][U][RT], af[2][U][MT], af_hi[2][U];
   auto load = [&](int buf, int k0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int r = 0; r < RT; ++r)
-        wf[buf][u][r] = w_on ? *reinterpret_cast<const bf16x8*>(wp[r] + k0 + u * 32) : bf16x8{};
+      for (int r = 0; r < RT; ++r) wf[buf][u][r] = *reinterpret_cast<const bf16x8*>(wp[r] + k0 + u * KSTEP);
 #pragma unroll
-      for (int m = 0; m < MT; ++m)
-        af[buf][u][m] = a_on ? *reinterpret_cast<const bf16x8*>(ap[m] + k0 + u * 32) : bf16x8{};
+      for (int m = 0; m < MT; ++m) af[buf][u][m] = *reinterpret_cast<const bf16x8*>(ap[m] + k0 + u * KSTEP);
+      if constexpr (HALF) af_hi[buf][u] = *reinterpret_cast<const bf16x8*>(ap[0] + k0 + u * KSTEP + 32);
     }
   };
   auto multiply = [&](int buf) {
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int r = 0; r < RT; ++r)
 #pragma unroll
         for (int m = 0; m < MT; ++m)
           acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[buf][u][r], af[buf][u][m], acc[r][m], 0, 0, 0);
+      if constexpr (HALF)
+        acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[buf][u][0], af_hi[buf][u], acc_hi, 0, 0, 0);
+    }
   };
-  constexpr int STEP = 32 * U;
+  constexpr int STEP = KSTEP * U;
   const int n_batches = k_len / STEP;
   int k = 0;
   if (n_batches > 0) {
@@ -159,17 +165,30 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
     if (b < n_batches) multiply(0);
     k = n_batches * STEP;
   }
-  for (; k < k_len; k += 32) {
+  for (; k < k_len; k += KSTEP) {
     bf16x8 wt[RT], at[MT];
 #pragma unroll
-    for (int r = 0; r < RT; ++r) wt[r] = w_on ? *reinterpret_cast<const bf16x8*>(wp[r] + k) : bf16x8{};
+    for (int r = 0; r < RT; ++r) wt[r] = *reinterpret_cast<const bf16x8*>(wp[r] + k);
 #pragma unroll
-    for (int m = 0; m < MT; ++m) at[m] = a_on ? *reinterpret_cast<const bf16x8*>(ap[m] + k) : bf16x8{};
+    for (int m = 0; m < MT; ++m) at[m] = *reinterpret_cast<const bf16x8*>(ap[m] + k);
 #pragma unroll
     for (int r = 0; r < RT; ++r)
 #pragma unroll
       for (int m = 0; m < MT; ++m)
         acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt[r], at[m], acc[r][m], 0, 0, 0);
+    if constexpr (HALF) {
+      const bf16x8 at_hi = *reinterpret_cast<const bf16x8*>(ap[0] + k + 32);
+      acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt[0], at_hi, acc_hi, 0, 0, 0);
+    }
+  }
+  if constexpr (HALF) {
+    // rows 0..7 of the tile (lanes kg < 2) take the sums of the second halves from rows 8..15 (the lane 32 further)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc_hi[i]), __float_as_uint(acc_hi[i]), false,
+                                                       false);
+      acc[0][0][i] += __uint_as_float(sw[1]);
+    }
   }
 
   if (scaled) {
@@ -458,7 +477,7 @@ extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M,
                                             int width_in, float* resid, const void* gamma, int gamma_dtype,
                                             void* u_out, float* ss_out, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 16 || K <= 0 || K % (32 * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K || (N & 3) ||
+  if (M > 16 || K <= 0 || K % ((half ? 64 : 32) * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K || (N & 3) ||
       ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || !resid || !gamma || !u_out || !ss_out ||
       ((uintptr_t)resid & 15) || ((uintptr_t)gamma & 15) || ((uintptr_t)u_out & 7) ||
       (gamma_dtype != kF32 && gamma_dtype != kBF16) || !fuse_in_ok(ss_in, parts_in, eps_in, width_in, M))
@@ -490,6 +509,9 @@ extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M,
   ATOMA_RESID(1, 1, 8, 4, true)
   ATOMA_RESID(1, 1, 8, 8, true)
   ATOMA_RESID(1, 1, 8, 2, true)
+  ATOMA_RESID(1, 1, 16, 4, true)
+  ATOMA_RESID(1, 1, 16, 2, true)
+  ATOMA_RESID(1, 1, 16, 4, false)
   ATOMA_RESID(1, 4, 1, 4, true)
 #undef ATOMA_RESID
   return ATOMA_ERR_SHAPE;

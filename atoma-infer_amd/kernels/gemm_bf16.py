@@ -302,17 +302,19 @@ def resid_plan(m: int, n: int, k: int):
     """(tiles of 16 rows of the weight per wave, waves splitting K, steps of K per batch of loads, half tiles) of the
     product that adds into the residual stream: K is split over the waves of a workgroup only (every sum has one
     owner, which also begins the norm), as many ways as K allows.  With N up to 2,048 a wave owns 8 rows of the
-    weight, not 16, so that 256 workgroups share the product (measured at Llama 1B's o and down products: 5.3 and
-    12.7 us against 5.9 and 15.0 with 16 rows a wave); wider outputs fill the GPU with whole tiles, and half tiles
-    cost them a third more (Llama 3B: 7.8 and 15.0 us against 10.5 and 21.4; 8B: 9.6 and 27.0 against 12.9 and 35.9)."""
+    weight, not 16, so that 256 workgroups share the product; the lanes of the other 8 rows fetch the same rows
+    further along K (measured at Llama 1B's o and down products with 8 rows of activations: 5.3 and 11.7 us against
+    5.9 and 15.0 with 16 rows a wave, and 12.7 when those lanes fetched nothing); wider outputs fill the GPU with
+    whole tiles, and half tiles cost them a third more (Llama 3B: 7.8 and 15.0 us against 10.5 and 21.4; 8B: 9.6 and
+    27.0 against 12.9 and 35.9)."""
     wk = 8
     while wk > 1 and k % (32 * wk):
         wk //= 2
     if wk == 2:
         wk = 1
-    half = 1 if n <= 2048 else 0
+    half = 1 if n <= 2048 and k % (64 * wk) == 0 else 0        # (a step of half tiles covers 64 values of K)
     depths = {(8, 1): (4, 2, 8), (8, 0): (8, 4, 2), (4, 1): (4, 8), (4, 0): (4,), (1, 1): (4,), (1, 0): (4,)}[(wk, half)]
-    depth = next((d for d in depths if k % (32 * wk * d) == 0), 4)
+    depth = next((d for d in depths if k % ((64 if half else 32) * wk * d) == 0), 4)
     return 1, wk, depth, half
 
 
