@@ -509,9 +509,6 @@ extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M,
   ATOMA_RESID(1, 1, 8, 4, true)
   ATOMA_RESID(1, 1, 8, 8, true)
   ATOMA_RESID(1, 1, 8, 2, true)
-  ATOMA_RESID(1, 1, 16, 4, true)
-  ATOMA_RESID(1, 1, 16, 2, true)
-  ATOMA_RESID(1, 1, 16, 4, false)
   ATOMA_RESID(1, 4, 1, 4, true)
 #undef ATOMA_RESID
   return ATOMA_ERR_SHAPE;
