@@ -91,11 +91,12 @@ class PagedAttention(Mixer):
         if cache_dtype is not torch.bfloat16 or page_size != attention_bf16.PAGE:
             return None
         group, window, nkv = self.nh // self.nkv, self.window or 0, self.nkv
+        cus = torch.cuda.get_device_properties(self.w_qkv.device).multi_processor_count
         return (attention_bf16.plan_key(group, window, nkv, self.hd),
                 lambda starts, counts, bucket: attention_bf16.build_tasks(
                     starts, counts, group, window, bucket, kv_heads=nkv,
                     max_waves=attention_bf16.max_waves_for(self.hd),
-                    row_tiles=attention_bf16.max_row_tiles_for(self.hd), head_size=self.hd))
+                    row_tiles=attention_bf16.max_row_tiles_for(self.hd), head_size=self.hd, compute_units=cus))
 
     # -- execution ------------------------------------------------------------------------------------
     accepts_begun = True

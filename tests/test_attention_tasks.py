@@ -183,3 +183,22 @@ def test_a_window_far_into_a_context_owns_few_slots():
         assert meta[2] <= 3 * (1000 // 128 + 2) and meta[0] <= meta[2] + 3
     without, meta_all = A.build_tasks(starts, counts, 4, 0, bucket, kv_heads=8, max_waves=2)
     assert meta_all[2] > 500
+
+
+def test_long_and_short_groups_meet_on_a_cu():
+    """Groups come longest first; every second round over the CUs is reversed, so that the workgroups which share a
+    CU's slots add up to about the same number of keys."""
+    order = A._serpentine(7, 8, 32)             # 4 groups a round
+    assert order.tolist() == [0, 1, 2, 3, 6, 5, 4]
+    assert A._serpentine(10, 8, 32).tolist() == list(range(10))            # more than two rounds: as it was
+    assert A._serpentine(5, 8, 256).tolist() == [0, 1, 2, 3, 4]            # less than a round: as it was
+    assert A._serpentine(7, 8, 32, head_size=128).tolist() == list(range(7))        # one workgroup a CU: as it was
+    for n, kv, cus in ((64, 8, 256), (7, 1, 4), (100, 3, 64)):
+        assert sorted(A._serpentine(n, kv, cus).tolist()) == list(range(n))
+    # a lone prompt of 2,048 tokens, 8 KV heads, 256 CUs: the keys of groups i and 63 - i... sum to the same
+    arr, meta = A.build_tasks(np.asarray([0], dtype=np.int32), np.asarray([2048], dtype=np.int32), 4, 0, kv_heads=8)
+    spans = (arr[: meta[0], 5] - arr[: meta[0], 4]).reshape(-1, 4).max(axis=1)
+    assert len(spans) == 64
+    sums = spans[:32] + spans[32:]
+    assert sums.max() - sums.min() <= 32
+    coverage(arr, meta, np.asarray([0]), np.asarray([2048]), 4, 0)
