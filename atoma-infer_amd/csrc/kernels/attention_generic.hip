@@ -8,7 +8,9 @@
 // Keys are visited in chunks of 64 starting at the first visible key, so the order of every reduction depends
 // only on (p, window): the result for a token does not depend on how the step was cut or batched.
 // Online softmax in float32 (csrc/kernels/softmax.h:128-186 of the reference); query head h reads KV head
-// h / (nh / nkv) (csrc/kernels/flash_fwd_kernel.h:593).
+// h / (nh / nkv) (csrc/kernels/flash_fwd_kernel.h:593).  With slopes (one per query head) the score of key j for the
+// token at p gains slopes[h] * (j - p), a bias that is linear in the distance (the reference's kernels take such
+// slopes too: csrc/kernels/mask.h:155-157, 179-186; its Llama passes none).
 #include "common.h"
 #include "cache_layout.h"
 
@@ -22,7 +24,8 @@ paged_attention_generic_kernel(const TQ* __restrict__ q, int q_stride, const TC*
                                const TC* __restrict__ vcache, TQ* __restrict__ out, int out_stride,
                                const int32_t* __restrict__ block_tables, int max_blocks,
                                const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
-                               float scale, int window, int page_size, int nh, int nkv, int hd) {
+                               float scale, int window, int page_size, int nh, int nkv, int hd,
+                               const float* __restrict__ slopes) {
   __shared__ float qs[kMaxHead];
   __shared__ float ps[kWave];
   __shared__ int32_t pg[kWave];
@@ -33,6 +36,7 @@ paged_attention_generic_kernel(const TQ* __restrict__ q, int q_stride, const TC*
   const int kvh = h / (nh / nkv);
   const int32_t* table = block_tables + (size_t)s * max_blocks;
   const int first = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const float slope = slopes ? slopes[h] : 0.f;
 
   for (int d = lane; d < hd; d += kWave) qs[d] = to_f32(q[(size_t)t * q_stride + (size_t)h * hd + d]);
   __syncthreads();
@@ -56,7 +60,7 @@ paged_attention_generic_kernel(const TQ* __restrict__ q, int q_stride, const TC*
 #pragma unroll
         for (int e = 0; e < 8; ++e) dot += qs[d0 + e] * to_f32(kr[e]);
       }
-      sc = dot * scale;
+      sc = dot * scale + slope * (float)(j - p);
     }
     const float m_new = fmaxf(m, wave_max(sc));
     const float corr = expf(m - m_new);  // exp(-inf) = 0 on the first chunk
@@ -93,7 +97,8 @@ extern "C" int atoma_paged_attention_generic(const void* q, int q_stride, const 
                                              void* out, int out_stride, int act_dtype, int cache_dtype,
                                              const int32_t* block_tables, int max_blocks, const int32_t* token_seq,
                                              const int32_t* positions, float scale, int window, int page_size,
-                                             int n_tokens, int nh, int nkv, int hd, hipStream_t stream) {
+                                             int n_tokens, int nh, int nkv, int hd, const float* slopes,
+                                             hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (hd <= 0 || hd > kMaxHead || nkv <= 0 || nh % nkv || page_size <= 0 || max_blocks <= 0 || nh > 65535)
     return ATOMA_ERR_SHAPE;
@@ -101,7 +106,7 @@ extern "C" int atoma_paged_attention_generic(const void* q, int q_stride, const 
 #define ATOMA_ATTN(TQ, TC)                                                                                       \
   hipLaunchKernelGGL((paged_attention_generic_kernel<TQ, TC>), grid, block, 0, stream, (const TQ*)q, q_stride, \
                      (const TC*)kcache, (const TC*)vcache, (TQ*)out, out_stride, block_tables, max_blocks,      \
-                     token_seq, positions, scale, window, page_size, nh, nkv, hd)
+                     token_seq, positions, scale, window, page_size, nh, nkv, hd, slopes)
   if (act_dtype == kF32 && cache_dtype == kF32) ATOMA_ATTN(float, float);
   else if (act_dtype == kBF16 && cache_dtype == kBF16) ATOMA_ATTN(bf16_t, bf16_t);
   else if (act_dtype == kF32 && cache_dtype == kBF16) ATOMA_ATTN(float, bf16_t);

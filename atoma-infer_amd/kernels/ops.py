@@ -202,11 +202,13 @@ def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[t
 
 def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, out: torch.Tensor,
                             block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
-                            scale: float, window: int, page_size: int, nh: int, nkv: int, hd: int) -> None:
+                            scale: float, window: int, page_size: int, nh: int, nkv: int, hd: int,
+                            slopes: Optional[torch.Tensor] = None) -> None:
     """Attention of every token of ``q`` [T, >= nh hd] (row stride free) over its request's cached keys.
 
     Token t belongs to row ``token_seq[t]`` of ``block_tables`` and sits at absolute position ``positions[t]``;
-    it sees keys max(0, p - window + 1) .. p (window 0: all).  ``out`` is [T, nh hd].
+    it sees keys max(0, p - window + 1) .. p (window 0: all).  ``out`` is [T, nh hd].  ``slopes`` (float32 [nh]):
+    head h's score of key j gains ``slopes[h] * (j - p)``.
     """
     _dev(q, kcache, vcache, out, block_tables, token_seq, positions)
     t = q.shape[0]
@@ -221,10 +223,14 @@ def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch
           "block_tables must be contiguous int32 [requests, blocks]")
     _i32(token_seq, "token_seq", t)
     _i32(positions, "positions", t)
+    if slopes is not None:
+        _dev(slopes)
+        _need(slopes.dtype is torch.float32 and slopes.is_contiguous() and slopes.numel() == nh,
+              "slopes must be contiguous float32, one per query head")
     _check(core().atoma_paged_attention_generic(
         _p(q), q.stride(0), _p(kcache), _p(vcache), _p(out), out.stride(0), _code(q, "q"), _code(kcache, "cache"),
         _p(block_tables), block_tables.shape[1], _p(token_seq), _p(positions), ctypes.c_float(scale), int(window),
-        page_size, t, nh, nkv, hd, _stream()), "paged_attention_generic")
+        page_size, t, nh, nkv, hd, _p(slopes), _stream()), "paged_attention_generic")
 
 
 def swiglu(gu: torch.Tensor, out: Optional[torch.Tensor] = None, block: int = 0) -> torch.Tensor:

@@ -45,6 +45,7 @@ class PagedAttention(Mixer):
         self.w_o: Optional[torch.Tensor] = None
         self.act_dtype = torch.float32
         self.paired = False      # q and k columns in pair order (set at load time)
+        self.slopes: Optional[torch.Tensor] = None      # per-head bias of the scores by distance, if the encoding has one
 
     # -- declaration ----------------------------------------------------------------------------------
     def graph_safe(self) -> bool:
@@ -65,6 +66,11 @@ class PagedAttention(Mixer):
         if self.position is not None:
             self.position.load(get, device, act_dtype)
         tables = self.position.rotary_tables() if self.position is not None else None
+        self.slopes = self.position.score_slopes(self.nh) if self.position is not None else None
+        if self.slopes is not None:
+            self.slopes = self.slopes.to(device=device, dtype=torch.float32).contiguous()
+            if self.slopes.numel() != self.nh:
+                raise ValueError(f"score_slopes gave {self.slopes.numel()} slopes for {self.nh} heads")
         self.paired = tables is not None and tables[2] == self.hd
         if self.paired:
             half = self.hd // 2
@@ -83,6 +89,8 @@ class PagedAttention(Mixer):
         kernels, built once per step on the host and shipped with the step's metadata.  ``bucket_tokens`` is None, or
         for a step that only decodes the context length its plan must serve (a multiple of the runner's bucket)."""
         from ..kernels import attention_bf16
+        if self.slopes is not None:
+            return None          # scores with a bias take the general kernel, which needs no plan
         if cache_dtype is torch.bfloat16 and page_size != attention_bf16.PAGE:
             import warnings
             warnings.warn(f"bfloat16 attention with pages of {page_size} tokens runs the general kernel (one wave per "
@@ -145,13 +153,14 @@ class PagedAttention(Mixer):
         return linear_delta(out, self.w_o, sink)
 
     def attend(self, q, k_cache, v_cache, out, ctx, cache) -> None:
-        if q.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16:
+        if self.slopes is None and q.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16:
             from ..kernels import attention_bf16
             if attention_bf16.try_attention(q, k_cache, v_cache, out, ctx, cache, self.scale, self.window or 0,
                                             self.nh, self.nkv, self.hd):
                 return
         ops.paged_attention_generic(q, k_cache, v_cache, out, cache.block_tables, ctx.token_seq, ctx.positions,
-                                    self.scale, self.window or 0, cache.page_size, self.nh, self.nkv, self.hd)
+                                    self.scale, self.window or 0, cache.page_size, self.nh, self.nkv, self.hd,
+                                    self.slopes)
 
 
 register_mixer("attention", PagedAttention)

@@ -139,6 +139,12 @@ class PositionEncoding(Part):
         """Encode in place: q [T, heads, hd], k [T, kv_heads, hd], positions [T] int32."""
         raise NotImplementedError
 
+    def score_slopes(self, num_heads: int) -> Optional[torch.Tensor]:
+        """float32 [num_heads] on the device, or None: an encoding that biases the attention scores by the distance,
+        head h's score of the key at j for the query at p gaining ``slopes[h] * (j - p)``.  Attention with such a
+        bias runs the general kernel (the matrix-core kernel has no bias)."""
+        return None
+
 
 class Mixer(Part):
     """Mixes information between the tokens of a request (attention here).

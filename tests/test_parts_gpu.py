@@ -155,6 +155,62 @@ def test_attention_part(act, nh, nkv, hd, width, window):
 
 
 @pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 24])
+def test_an_encoding_that_biases_scores_by_distance(act, window):
+    """A position encoding defined here that rotates nothing and gives each head a slope: the score of the key at j
+    for the query at p gains slope * (j - p).  The framework's attention takes it through its general kernel; the
+    plain formula is written out below (softmax over the visible keys of q.k * scale + slope * (j - p))."""
+    from atoma_infer_amd.cache.pool import LayerCache
+    from atoma_infer_amd.parts import PagedAttention, PositionEncoding
+
+    class Slopes(PositionEncoding):
+        def graph_safe(self):
+            return True
+
+        def apply(self, q, k, positions):
+            pass
+
+        def score_slopes(self, num_heads):
+            return torch.tensor([2.0 ** (-8.0 * (h + 1) / num_heads) for h in range(num_heads)])
+
+    nh, nkv, hd, width, n, page, pages = 6, 2, 32, 80, 70, 16, 8
+    g = torch.Generator().manual_seed(11)
+    ws = {name: (torch.randn(*sh, generator=g) * 0.2).to(torch.bfloat16) for name, sh in
+          (("q_proj.weight", (nh * hd, width)), ("k_proj.weight", (nkv * hd, width)),
+           ("v_proj.weight", (nkv * hd, width)), ("o_proj.weight", (width, nh * hd)))}
+    part = PagedAttention(width, nh, nkv, hd, Slopes(), window)
+    part.load(getter(ws), torch.device(DEV), act)
+    assert part.step_planner(page, act) is None              # the general kernel needs no plan
+    x = torch.randn(n, width, generator=g).to(act)
+    xf, w = x.double(), {k: v.double() for k, v in ws.items()}
+    q = (xf @ w["q_proj.weight"].T).view(n, nh, hd)
+    k = (xf @ w["k_proj.weight"].T).view(n, nkv, hd).repeat_interleave(nh // nkv, 1)
+    v = (xf @ w["v_proj.weight"].T).view(n, nkv, hd).repeat_interleave(nh // nkv, 1)
+    slopes = Slopes().score_slopes(nh).double()
+    dist = torch.arange(n)[None, :] - torch.arange(n)[:, None]                  # j - p
+    scores = torch.einsum("phd,jhd->hpj", q, k) / math.sqrt(hd) + slopes[:, None, None] * dist[None]
+    hidden = (dist > 0) | ((dist <= -window) if window else torch.zeros_like(dist, dtype=torch.bool))
+    probs = torch.softmax(scores.masked_fill(hidden[None], float("-inf")), dim=-1)
+    want = (torch.einsum("hpj,jhd->phd", probs, v).reshape(n, nh * hd) @ w["o_proj.weight"].T).float()
+    # the bias matters: without it the result is another
+    plain = torch.softmax((scores - slopes[:, None, None] * dist[None]).masked_fill(hidden[None], float("-inf")), dim=-1)
+    assert frob_err((torch.einsum("hpj,jhd->phd", plain, v).reshape(n, nh * hd) @ w["o_proj.weight"].T).float(), want) > 0.05
+    order = torch.randperm(pages, generator=g)[: -(-n // page)]
+    bt = order.int().view(1, -1).to(DEV)
+    kc = torch.zeros(pages, nkv, page * hd, dtype=act, device=DEV)
+    vc = torch.zeros(pages, nkv, page * hd, dtype=act, device=DEV)
+    got = []
+    for start, count in [(0, 37), (37, 20)] + [(i, 1) for i in range(57, n)]:
+        pos = torch.arange(start, start + count)
+        slots = (order[pos // page] * page + pos % page).int().to(DEV)
+        cache = LayerCache(k=kc, v=vc, page_size=page, writable=True, group=0, slot_mapping=slots, block_tables=bt)
+        y = part.forward(x[start:start + count].to(DEV), PartCtx(start, count), cache)
+        got.append((y.sum(0) if y.dim() == 3 else y).float().cpu())
+    err = frob_err(torch.cat(got), want)
+    assert err < (TOL_F32 if act is torch.float32 else TOL_BF16), err
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
 def test_pre_norm_block_part(act):
     """The arrangement alone: h = x + mixer(norm(x)), y = h + ffn(norm(h)), with the sums left to the next norm."""
     from atoma_infer_amd.cache.pool import LayerCache
