@@ -56,3 +56,22 @@ def test_library_thresholds():
     assert wins(17, 128256, 2048, torch.float32) == gemm_bf16._MM_OUT_DTYPE and not wins(16, 128256, 2048, torch.float32)
     # the head: eight waves splitting K up to 8 rows, then 64 rows of W a wave and four waves splitting K
     assert [gemm_bf16._plan(m, 128256, 2048, False) for m in (8, 9, 16)] == [(2, 8, 1), (4, 4, 1), (4, 4, 1)]
+
+
+# (tiles, waves splitting K, steps a batch of loads, half tiles) of the residual product in csrc/kernels/gemm_bf16.hip
+RESID = {(1, 4, 4, 0), (1, 8, 4, 0), (1, 8, 2, 0), (1, 8, 8, 0), (1, 1, 4, 0),
+         (1, 4, 4, 1), (1, 4, 8, 1), (1, 8, 4, 1), (1, 8, 8, 1), (1, 8, 2, 1), (1, 1, 4, 1)}
+
+
+def test_residual_products_name_kernels_that_exist():
+    for n, k in shapes():
+        for m in (1, 8, 16):
+            rt, wk, depth, half = gemm_bf16.resid_plan(m, n, k)
+            assert (rt, wk, depth, half) in RESID, (m, n, k)
+            assert k % (32 * wk) == 0
+            if half:            # a step of half tiles covers 64 values of K, and N is small
+                assert k % (64 * wk) == 0 and n <= 2048
+    # Llama 1B: 8 rows of the weight a wave; 3B and 8B: whole tiles, and as many steps a batch as K allows
+    assert gemm_bf16.resid_plan(8, 2048, 2048) == (1, 8, 4, 1) and gemm_bf16.resid_plan(8, 2048, 8192) == (1, 8, 4, 1)
+    assert gemm_bf16.resid_plan(8, 3072, 8192) == (1, 8, 8, 0) and gemm_bf16.resid_plan(8, 4096, 14336) == (1, 8, 8, 0)
+    assert gemm_bf16.resid_plan(8, 3072, 3072) == (1, 8, 4, 0)
