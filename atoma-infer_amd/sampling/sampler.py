@@ -44,6 +44,7 @@ class Pending:
 class Sampler:
     def __init__(self, device: torch.device):
         self.device = device
+        self._greedy_meta = {}        # rows -> the device copy of the parameters of that many greedy rows
 
     def launch(self, logits: torch.Tensor, plans: Sequence[SamplingPlan], steps: Sequence[int],
                contexts: Sequence[Sequence[int]]) -> Pending:
@@ -61,6 +62,16 @@ class Sampler:
                 uniq = set(contexts[i][-pl.repeat_last_n:])
                 pen_rows += [i] * len(uniq)
                 pen_toks += list(uniq)
+        # rows that all take the largest logit need no parameters of their own: one upload per batch size, ever
+        all_greedy = not pen_rows and all(pl.greedy for pl in plans)
+        if all_greedy and s in self._greedy_meta:
+            m = self._greedy_meta[s]
+            out = ops.sample_packed(logits, m[0], m[4].view(torch.int32), m[1], m[2])
+            host = torch.empty((2, s), dtype=torch.float32, pin_memory=True)
+            host.copy_(out, non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            return Pending(out[0].view(torch.int32), out[1], host, ev)
         # one packed upload: temperature, top_p, uniform, penalty (float32) and top_k (int32 bits)
         meta = torch.empty((5, s), dtype=torch.float32, pin_memory=True)
         mn = meta.numpy()
@@ -72,6 +83,9 @@ class Sampler:
             mn[3, i] = pl.repetition_penalty
             top_k[i] = pl.top_k
         m = meta.to(self.device, non_blocking=True)
+        if all_greedy:
+            # (top_p, penalty and top_k of a greedy row are never read; the copy kept is this batch's)
+            self._greedy_meta[s] = m
         if pen_rows:
             pen = torch.tensor([pen_rows, pen_toks], dtype=torch.int32).to(self.device)
             ops.repeat_penalty(logits, pen[0], pen[1], m[3])
