@@ -3,7 +3,7 @@
     python -m atoma_infer_amd generate --config-path engine.toml --requests requests.jsonl
     python -m atoma_infer_amd generate --model DIR --dtype bf16 --prompt-ids 1,2,3 --max-new-tokens 16
     python -m atoma_infer_amd random-weights --config config.json --out DIR --seed 0
-    python -m atoma_infer_amd replay --model DIR --dtype float32 --out DIR --max-tokens 4096 < trace.jsonl
+    python -m atoma_infer_amd replay --model DIR --dtype float32 --out DIR --max-tokens 4096 [--page-size P] [--max-live L] < trace.jsonl
 
 ``--config-path`` is the reference's one flag (server/src/main.rs:22-27): a TOML file with the sections
 [inference], [cache], [scheduler] and [validation].  A line of ``--requests`` is the reference's
@@ -79,8 +79,13 @@ def _cmd_random(args) -> int:
 
 
 def _cmd_replay(args) -> int:
-    from .engine.replay import make_runner, replay
-    return replay(make_runner(args.model, args.dtype, args.max_tokens), sys.stdin, args.out)
+    from .engine.replay import main as replay_main
+    argv = ["--model", args.model, "--dtype", args.dtype, "--out", args.out, "--max-tokens", str(args.max_tokens)]
+    if args.page_size is not None:
+        argv += ["--page-size", str(args.page_size)]
+    if args.max_live is not None:
+        argv += ["--max-live", str(args.max_live)]
+    return replay_main(argv)
 
 
 def main(argv=None) -> int:
@@ -125,6 +130,8 @@ def main(argv=None) -> int:
     t.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     t.add_argument("--out", required=True)
     t.add_argument("--max-tokens", type=int, required=True)
+    t.add_argument("--page-size", type=int, default=None, help="tokens a page of the cache (bin/trace_run's default)")
+    t.add_argument("--max-live", type=int, default=None, help="most requests live at a time (bin/trace_run's default)")
     t.set_defaults(fn=_cmd_replay)
 
     args = ap.parse_args(argv)

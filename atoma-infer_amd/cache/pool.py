@@ -121,10 +121,10 @@ class CachePool:
 
 def pages_for_tokens(plan: CachePlan, page_size: int, max_tokens: int, max_requests: int) -> List[int]:
     """Pages per group that hold ``max_tokens`` tokens of at most ``max_requests`` live requests, where the caller
-    has rounded each request's count up to a multiple of 64.  Pages of up to 64 tokens then need no more than
-    ``max_tokens / page_size`` pages; larger pages round each request up further, by less than a page each."""
+    has rounded each request's count up to a multiple of 64.  Page sizes that divide 64 then need no more than
+    ``max_tokens / page_size`` pages; any other size rounds each request up further, by less than a page each."""
     per_group = -(-max_tokens // page_size)
-    if page_size > 64:
+    if 64 % page_size:
         per_group += max_requests
     return [max(per_group, 1) for _ in plan.groups]
 

@@ -239,8 +239,10 @@ void* sc_create(void* cache_manager, int max_tokens, int max_seqs, int max_model
                 double delay_factor, int chunk_align) {
   if (!cache_manager || max_tokens <= 0 || max_seqs <= 0 || max_model_len <= 0 || max_chunk < 0 || chunk_align <= 0)
     return nullptr;
-  // a cut prompt needs room for one aligned portion
-  if (chunked && chunk_align > 1 && (max_tokens < chunk_align || (max_chunk > 0 && max_chunk < chunk_align)))
+  // a cut prompt needs room for one aligned portion, also in a step in which every other request decodes a token
+  // (decoding requests are planned first: with less room a prompt would stand still for as long as they run)
+  if (chunked && chunk_align > 1 &&
+      (max_tokens < chunk_align + max_seqs - 1 || (max_chunk > 0 && max_chunk < chunk_align)))
     return nullptr;
   Sched* s = new Sched();
   s->cm = cache_manager;

@@ -511,11 +511,21 @@ constexpr bool kSplit8Fits = kMerge8Bytes <= kLdsBytes;
 // merge of two waves a task (twice as large) lets two workgroups share a CU
 constexpr bool kTwoPieces = HD <= 64;
 
-// A kernel that wants more than 64 KB of LDS at launch must be told so once (per device).
+// A kernel that wants more than 64 KB of LDS at launch must be told so once per device: every instance of the
+// template keeps, per device, whether it has been (a driver call per launch would sit on the path of every layer of
+// every step, and inside the recording of decode graphs).  An instance always asks for the same number of bytes.
+constexpr int kMaxDevices = 64;
 template <typename K> static int allow_lds(K kernel, size_t bytes) {
   if (bytes <= 65536) return 0;
-  return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)bytes);
+  static bool told[kMaxDevices] = {};
+  int dev = 0;
+  const hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev >= 0 && dev < kMaxDevices && told[dev]) return 0;
+  const int rc = (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (rc == 0 && dev >= 0 && dev < kMaxDevices) told[dev] = true;
+  return rc;
 }
 
 extern "C" int atoma_attention_mfma_head_size() { return HD; }

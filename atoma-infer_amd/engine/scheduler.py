@@ -111,7 +111,10 @@ class Scheduler:
                                       config.max_model_len, int(config.enable_chunked_prefill),
                                       config.max_prefill_chunk, float(config.delay_factor), int(chunk_alignment))
         if not self._h:
-            raise SchedulerError(f"the native scheduler refused {config} with portions aligned to {chunk_alignment}")
+            raise SchedulerError(f"the native scheduler refused {config} with portions aligned to {chunk_alignment} "
+                                 f"(a cut prompt needs max_num_batched_tokens >= alignment + max_num_sequences - 1, so "
+                                 f"that an aligned portion fits beside the decoding requests, and max_prefill_chunk, "
+                                 f"if set, >= alignment)")
         self._requests: Dict[int, Request] = {}
         self._running: Dict[int, Request] = {}
         self._adopted = getattr(cache, "adopted", None)

@@ -299,7 +299,9 @@ class ModelRunner:
             block_tables=[dev[o_bt + g * s * max_blocks: o_bt + (g + 1) * s * max_blocks].view(s, max_blocks)
                           for g in range(n_groups)],
             pool=self.pool, decode_bucket=bucket,
-            wants_all_rows=n_want == t and (t == s or all(len(e.want) == len(e.tokens) and
+            # (one token an entry: every entry must want its one place, once; two wanting [0, 0] and [] do not)
+            wants_all_rows=n_want == t and (bool((want_counts == 1).all()) if t == s else
+                                            all(len(e.want) == len(e.tokens) and
                                                           all(w == j for j, w in enumerate(e.want))
                                                           for e in entries)))
         for off, (key, arr, meta) in zip(ex_off, extras):

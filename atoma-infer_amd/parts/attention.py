@@ -32,9 +32,10 @@ class PagedAttention(Mixer):
                  scale: Optional[float] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot be grouped over {num_kv_heads} KV heads")
-        if head_size % 16 or not 16 <= head_size <= 256:
-            raise ValueError(f"head size {head_size} is not supported: the attention kernels take multiples of 16 "
-                             f"from 16 to 256")
+        # every multiple of 8 up to 256, as the reference's kernels take (csrc/src/lib.rs:136-143, 790)
+        if head_size % 8 or not 8 <= head_size <= 256:
+            raise ValueError(f"head size {head_size} is not supported: the attention kernels take multiples of 8 "
+                             f"from 8 to 256")
         if window is not None and window <= 0:
             raise ValueError("window must be positive")
         self.width, self.nh, self.nkv, self.hd = int(width), int(num_heads), int(num_kv_heads), int(head_size)
@@ -91,6 +92,12 @@ class PagedAttention(Mixer):
         from ..kernels import attention_bf16
         if self.slopes is not None:
             return None          # scores with a bias take the general kernel, which needs no plan
+        if cache_dtype is torch.bfloat16 and self.hd % 16:
+            import warnings
+            warnings.warn(f"bfloat16 attention with heads of {self.hd} columns runs the general kernel (one wave per "
+                          f"token and head), many times slower than the matrix-core kernel, which takes head sizes "
+                          f"that are multiples of 16", stacklevel=2)
+            return None
         if cache_dtype is torch.bfloat16 and page_size != attention_bf16.PAGE:
             import warnings
             warnings.warn(f"bfloat16 attention with pages of {page_size} tokens runs the general kernel (one wave per "

@@ -313,3 +313,28 @@ def test_a_step_packed_in_one_call_equals_the_arrays_made_one_by_one(seed):
                       np.asarray([1, 2], dtype=np.int32), np.asarray([-1], dtype=np.int32),
                       np.asarray([1], dtype=np.int32), np.asarray([2], dtype=np.int32), np.zeros(64, dtype=np.int32),
                       np.arange(0, 60, 6, dtype=np.int64), 2)
+
+
+@pytest.mark.parametrize("page_size", [4, 16, 24, 32, 48, 64, 80, 128])
+def test_a_pool_sized_for_rounded_tokens_holds_them_at_every_page_size(page_size):
+    """What the replay program promises: a pool made for N tokens holds any live requests whose counts, each rounded
+    up to a multiple of 64, add up to N -- also with pages of 24 or 48 tokens, which do not divide 64."""
+    from atoma_infer_amd.cache.pool import CachePlan, pages_for_tokens
+    plan = CachePlan(groups=[None], where={}, states={})
+    live, max_tokens = 16, 16 * 64
+    (pages,) = pages_for_tokens(plan, page_size, max_tokens, live)
+    m = CacheManager([GroupGeometry(page_size, pages)], live)
+    for r in range(live):
+        m.add(r)
+        m.reserve(r, 64)                   # sixteen requests of 64 rounded tokens each
+    m.check()
+    for r in range(live):
+        m.free(r)
+    # a few long requests beside short ones
+    counts = [448, 320, 192, 64]
+    (pages,) = pages_for_tokens(plan, page_size, sum(counts), live)
+    m = CacheManager([GroupGeometry(page_size, pages)], live)
+    for r, n in enumerate(counts):
+        m.add(r)
+        m.reserve(r, n)
+    m.check()

@@ -19,7 +19,7 @@ DTYPES = ["float32", "bfloat16"]
 # ranges walked by eight waves, where the head size allows them), or in chunks merged by a second kernel, as it does
 # at long contexts with few requests; the float32 attention has one way only
 DTYPE_TASKS = [(d, "planned") for d in DTYPES] + [("bfloat16", "chunks")]
-PAGE = {"A": 4, "B": 16, "C": 16, "D": 16, "E": 16}
+PAGE = {"A": 4, "B": 16, "C": 16, "D": 16, "E": 16, "F": 16}
 
 
 @pytest.fixture(scope="module")
@@ -102,7 +102,7 @@ def check_against_plain(model_dir, requests, got, dtype):
 
 def lengths(name):
     return {"A": [100, 37, 64, 5], "B": [200, 1, 77, 130], "C": [150, 48, 97, 16], "D": [900, 300, 150, 40],
-            "E": [600, 290, 33, 129]}[name]
+            "E": [600, 290, 33, 129], "F": [180, 61, 16, 99]}[name]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -160,7 +160,7 @@ def test_mixed_batches_with_few_pages(model_dirs, name, dtype, tasks, monkeypatc
     vocab = TINY[name]["vocab_size"]
     lens = {"A": [60, 33, 47, 21, 58, 40, 9, 52], "B": [120, 1, 77, 90, 45, 130, 18, 66],
             "C": [90, 48, 97, 16, 70, 33, 80, 25], "D": [700, 48, 97, 530, 70, 33, 80, 25],
-            "E": [300, 48, 97, 610, 70, 33, 80, 25]}[name]
+            "E": [300, 48, 97, 610, 70, 33, 80, 25], "F": [110, 48, 97, 16, 70, 33, 80, 25]}[name]
     requests = {f"r{i}": random_tokens(n, vocab, 300 + i) for i, n in enumerate(lens)}
     page = PAGE[name]
     rng = random.Random(5)
@@ -195,6 +195,34 @@ def test_mixed_batches_with_few_pages(model_dirs, name, dtype, tasks, monkeypatc
     assert len(got) == sum(lens)
     check_against_plain(model_dirs[name], requests, got, dtype)
     assert runner.manager.num_free_pages(0) == need and runner.manager.num_requests() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_place_wanted_twice_beside_an_entry_that_wants_nothing(model_dirs, dtype):
+    """Two decoded tokens, the first entry wanting its place twice, the second nothing: as many wanted rows as
+    tokens, but not "every row once" (the bfloat16 path that lets the last product begin the final norm on all rows
+    must not take it)."""
+    from atoma_infer_amd.engine import StepEntry
+    name = "D"
+    vocab = TINY[name]["vocab_size"]
+    a, b = random_tokens(40, vocab, 41), random_tokens(23, vocab, 42)
+    runner = make_runner(model_dirs[name], dtype, PAGE[name], 16)
+    runner.add_request(0)
+    runner.add_request(1)
+    assert runner.step([StepEntry(0, a[:39], 0, []), StepEntry(1, b[:22], 0, [])]) is None
+    logits = runner.step([StepEntry(0, a[39:], 39, [0, 0]), StepEntry(1, b[22:], 22, [])]).cpu()
+    assert logits.shape == (2, vocab)
+    assert torch.equal(logits[0], logits[1])
+    check_against_plain(model_dirs[name], {"a": a}, {("a", 39): logits[0]}, dtype)
+    # ... and the other way round: the second entry's row, not the first's
+    runner.free_request(0)
+    runner.free_request(1)
+    runner.add_request(0)
+    runner.add_request(1)
+    runner.step([StepEntry(0, a[:39], 0, []), StepEntry(1, b[:22], 0, [])])
+    logits = runner.step([StepEntry(0, a[39:], 39, []), StepEntry(1, b[22:], 22, [0, 0])]).cpu()
+    assert torch.equal(logits[0], logits[1])
+    check_against_plain(model_dirs[name], {"b": b}, {("b", 22): logits[0]}, dtype)
 
 
 def test_pages_the_matrix_core_attention_refuses_are_announced(model_dirs):
@@ -509,7 +537,24 @@ def _random_configuration(rng):
 @pytest.mark.parametrize("seed", range(16))
 def test_random_configurations_step_like_the_plain_model(tmp_path, seed):
     rng = random.Random(7000 + seed)
+    _step_a_random_schedule(tmp_path, _random_configuration(rng), rng, seed)
+
+
+@pytest.mark.parametrize("hd", [8, 24, 40, 72, 88, 104, 120, 136, 200, 248])
+def test_head_sizes_that_are_odd_multiples_of_eight(tmp_path, hd):
+    """The reference's attention takes every head size that is a multiple of 8 up to 256 (csrc/src/lib.rs:136-143,
+    790); here those that are no multiple of 16 run the general attention kernel, in both dtypes."""
+    rng = random.Random(9000 + hd)
     cfg = _random_configuration(rng)
+    nkv = rng.choice([1, 2, 3])
+    nh = nkv * rng.choice([1, 2, 4])
+    while nh * hd > 1024 and nh > nkv:
+        nh //= 2
+    cfg.update(hidden_size=nh * hd, num_attention_heads=nh, num_key_value_heads=nkv)
+    _step_a_random_schedule(tmp_path, cfg, rng, hd)
+
+
+def _step_a_random_schedule(tmp_path, cfg, rng, seed):
     model_dir = make_model_dir(str(tmp_path / "m"), cfg, seed=seed, dtype="bfloat16", norm_jitter=0.1)
     vocab = cfg["vocab_size"]
     la, lb, lc = rng.randint(150, 400), rng.randint(20, 200), rng.randint(2, 70)

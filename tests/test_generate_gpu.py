@@ -289,10 +289,16 @@ def test_repeat_penalty_kernel_and_temperature_limit():
 # bin/trace_run as a program
 
 
-def run_trace(model_dir, dtype, steps, out_dir, max_tokens, extra=(), ok=True):
+def run_trace(model_dir, dtype, steps, out_dir, max_tokens, extra=(), ok=True, program="bin/trace_run"):
+    """``program``: bin/trace_run, or the package's own ``replay`` command (the two are one function)."""
     env = dict(os.environ)
-    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype",
-                           dtype, "--out", out_dir, "--max-tokens", str(max_tokens), *extra],
+    if program == "bin/trace_run":
+        head = [sys.executable, os.path.join(ROOT, "bin", "trace_run")]
+    else:
+        head = [sys.executable, "-m", "atoma_infer_amd", "replay"]
+        env["PYTHONPATH"] = ROOT + os.pathsep + env.get("PYTHONPATH", "")
+    proc = subprocess.run([*head, "--model", model_dir, "--dtype", dtype, "--out", out_dir, "--max-tokens",
+                           str(max_tokens), *extra],
                           input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
                           env=env, timeout=300)
     if not ok:
@@ -302,10 +308,11 @@ def run_trace(model_dir, dtype, steps, out_dir, max_tokens, extra=(), ok=True):
     return proc
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run_with_pages_of_four_tokens(model_dirs, tmp_path, dtype):
+@pytest.mark.parametrize("dtype,program", [("float32", "bin/trace_run"), ("bfloat16", "python -m atoma_infer_amd replay")])
+def test_trace_run_with_pages_of_four_tokens(model_dirs, tmp_path, dtype, program):
     """Tiny A with its own block size of 4 through the program's --page-size, three requests with two live at a time
-    in a pool of 128 tokens; then a third live request beyond --max-live ends the program with a clear message."""
+    in a pool of 128 tokens; then a third live request beyond --max-live ends the program with a clear message.
+    Once through bin/trace_run and once through the package's ``replay`` command, which takes the same options."""
     d = model_dirs["A"]
     vocab = TINY["A"]["vocab_size"]
     a, b, c = random_tokens(50, vocab, 1), random_tokens(9, vocab, 2), random_tokens(30, vocab, 3)
@@ -318,7 +325,7 @@ def test_trace_run_with_pages_of_four_tokens(model_dirs, tmp_path, dtype):
         {"step": 3, "entries": [{"id": "c", "tokens": c[2:], "want": [27]}], "end": ["c"]},
     ]
     out = str(tmp_path / "out")
-    run_trace(d, dtype, steps, out, 128, extra=("--page-size", "4", "--max-live", "2"))
+    run_trace(d, dtype, steps, out, 128, extra=("--page-size", "4", "--max-live", "2"), program=program)
     w, cfg = plain_weights(d), plain_config(d)
     pa, pb, pc = (plain_llama.forward(t, w, cfg) for t in (a, b, c))
     want = {0: torch.stack([pa[20], pb[4]]), 1: torch.stack([pb[8], pa[21], pa[49]]), 2: pc[1][None], 3: pc[29][None]}

@@ -202,6 +202,63 @@ def test_whole_model_invariants(cfg):
     assert torch.allclose(P.forward(toks, w3, cfg), want, atol=1e-6)
 
 
+def test_one_token_block_in_closed_form():
+    """A sequence of one token: the softmax over one key is 1, so attention returns v whatever q, k and the rotation
+    are, and the block is h + mlp(norm2(h)) with h = x + Wo . repeat(Wv . norm1(x)) (models/src/llama.rs:401-409).
+    Written out here with matrix products only; a block that adds the feed-forward to x instead of h, norms after
+    the mixer, or feeds the mixer the unnormed rows fails it."""
+    cfg = {"hidden_size": 24, "num_attention_heads": 3, "num_key_value_heads": 1, "rope_theta": 1e4,
+           "rms_norm_eps": 1e-5}
+    g = torch.Generator().manual_seed(21)
+    r = lambda *shape: torch.randn(*shape, generator=g) * 0.5
+    p = "model.layers.0."
+    w = {p + "input_layernorm.weight": 1 + r(24), p + "post_attention_layernorm.weight": 1 + r(24),
+         p + "self_attn.q_proj.weight": r(24, 24), p + "self_attn.k_proj.weight": r(8, 24),
+         p + "self_attn.v_proj.weight": r(8, 24), p + "self_attn.o_proj.weight": r(24, 24),
+         p + "mlp.gate_proj.weight": r(40, 24), p + "mlp.up_proj.weight": r(40, 24), p + "mlp.down_proj.weight": r(24, 40)}
+    x = r(1, 24)
+
+    def norm(t, gamma):
+        return t / torch.sqrt((t * t).sum() / 24 + 1e-5) * gamma
+
+    v = norm(x, w[p + "input_layernorm.weight"]) @ w[p + "self_attn.v_proj.weight"].T          # [1, 8]: the one KV head
+    h = x + v.repeat(1, 3) @ w[p + "self_attn.o_proj.weight"].T                                  # all three heads read it
+    n2 = norm(h, w[p + "post_attention_layernorm.weight"])
+    gate, up = n2 @ w[p + "mlp.gate_proj.weight"].T, n2 @ w[p + "mlp.up_proj.weight"].T
+    want = h + (gate / (1 + torch.exp(-gate)) * up) @ w[p + "mlp.down_proj.weight"].T
+    for pos in (0, 5):      # one key: the position cannot matter either
+        got = P.block(x, w, 0, cfg, torch.tensor([pos]))
+        assert torch.allclose(got, want, atol=1e-5), (got - want).abs().max()
+    # the pin bites: the feed-forward's share and the mixer's share are both far from nothing
+    assert (want - h).abs().max() > 1e-2 and (h - x).abs().max() > 1e-2
+
+
+def test_two_token_attention_by_hand():
+    """Two tokens, one head of four columns.  Columns 0 and 2 (the pair that turns by one radian a position whatever
+    theta is) are zero in q and k, and theta is so large that the other pair's angle at position 1 is below 1e-14, so
+    the rotation changes nothing and token 1's weights are softmax([q1.k0, q1.k1] / sqrt(4)), worked out with exp
+    by hand (models/src/llama.rs:342).  A scale of 1/hd, no scale, or a scale applied after the softmax fails it."""
+    cfg = {"hidden_size": 4, "num_attention_heads": 1, "num_key_value_heads": 1, "rope_theta": 1e30}
+    eye = torch.eye(4)
+    wv = torch.tensor([[1.0, 0.5, 0.0, 0.0], [0.0, 1.0, 0.0, 2.0], [3.0, 0.0, 1.0, 0.0], [0.0, -1.0, 0.0, 1.0]])
+    w = {"q_proj.weight": eye, "k_proj.weight": eye, "v_proj.weight": wv, "o_proj.weight": eye}
+    x = torch.tensor([[0.0, 2.0, 0.0, -1.0], [0.0, 1.0, 0.0, 3.0]])
+    out = P.self_attention(x, w, "", cfg, torch.arange(2))
+    v = x @ wv.T
+    # token 0 sees itself only
+    assert torch.allclose(out[0], v[0], atol=1e-6)
+    s0, s1 = float(x[1] @ x[0]) / 2.0, float(x[1] @ x[1]) / 2.0          # (2 - 3) / 2 = -0.5, (1 + 9) / 2 = 5
+    assert (s0, s1) == (-0.5, 5.0)
+    a0 = math.exp(s0) / (math.exp(s0) + math.exp(s1))
+    want = a0 * v[0] + (1 - a0) * v[1]
+    assert torch.allclose(out[1], want, atol=1e-6)
+    # what the plausible slips would give is far from it
+    for wrong_scale in (1.0 / 4.0, 1.0):
+        t0, t1 = float(x[1] @ x[0]) * wrong_scale, float(x[1] @ x[1]) * wrong_scale
+        b0 = math.exp(t0) / (math.exp(t0) + math.exp(t1))
+        assert float(((b0 - a0) * (v[0] - v[1])).abs().max()) > 1e-3
+
+
 def test_grouping_maps_query_heads_to_kv_heads_in_blocks():
     """Query head h reads KV head h // (nh/nkv) (csrc/kernels/flash_fwd_kernel.h:593), not h % nkv."""
     cfg = {"hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2, "rope_theta": 1e4}

@@ -318,6 +318,30 @@ def test_portions_end_where_the_model_allows():
     with pytest.raises(SchedulerError):                              # no aligned portion fits such a budget
         Scheduler(SchedulerConfig(max_num_batched_tokens=6, max_num_sequences=4, max_model_len=256), cache,
                   chunk_alignment=8)
+    # ... nor one that an aligned portion fits only while nothing decodes: the prompt would stand still meanwhile
+    with pytest.raises(SchedulerError, match="alignment"):
+        Scheduler(SchedulerConfig(max_num_batched_tokens=8, max_num_sequences=2, max_model_len=256), cache,
+                  chunk_alignment=8)
+
+
+def test_an_aligned_portion_fits_beside_every_decoding_request():
+    """The smallest budget the scheduler takes with aligned portions (alignment + requests - 1): one request decodes,
+    another is in its prompt, and the prompt moves on by an aligned portion in every step."""
+    cache = CacheManager([GroupGeometry(4, 64)], 4)
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=9, max_num_sequences=2, max_model_len=256), cache,
+                  chunk_alignment=8)
+    a, b = make_request(0, 5, max_new=12), make_request(1, 40, max_new=2)
+    s.add(a)
+    run_step(s, s.schedule())                                        # a's prompt; a decodes from here on
+    s.add(b)
+    starts = []
+    for _ in range(5):
+        out = s.schedule()
+        plan = {e.request.uid: (e.start, e.num_tokens) for e in out.entries}
+        assert plan[0][1] == 1 and plan[1][1] == 8, plan           # a decodes, b takes 8 of its 40
+        starts.append(plan[1][0])
+        run_step(s, out)
+    assert starts == [0, 8, 16, 24, 32]
 
 
 def test_max_prefill_chunk_caps_portions():
@@ -382,6 +406,8 @@ def _random_world(seed):
     if not lim.cut:
         lim.max_tokens = max(lim.max_tokens, lim.max_model_len)      # the configuration demands it
     lim.max_tokens = max(lim.max_tokens, lim.max_requests, lim.align)
+    if lim.cut and lim.align > 1:
+        lim.max_tokens = max(lim.max_tokens, lim.align + lim.max_requests - 1)   # room for an aligned portion
     if lim.max_portion:
         lim.max_portion = max(lim.max_portion, lim.align)
     now = [0.0]

@@ -78,3 +78,57 @@ def test_sampling_without_allocation_refuses_what_does_not_fit():
                                  _ptr(dummy), _ptr(dummy), stream)
     assert rc == TOO_LARGE
     torch.cuda.synchronize()
+
+
+def test_sampling_without_allocation_allocates_nothing_and_can_be_captured():
+    """What the entry point is for.  Around a call, after the set-up call, the device's free memory (hipMemGetInfo)
+    and torch's own books stay as they were; and the call is recorded into a graph, where an allocating call is an
+    error, and replayed with eager work and synchronisation between the replays, every replay checked against the
+    workspace entry point."""
+    from atoma_infer_amd.kernels.library import load_hip_module
+    lib = load_hip_module("core")
+    for f in (lib.atoma_sample, lib.atoma_sample_static, lib.atoma_sample_static_init):
+        f.restype = ctypes.c_int
+    assert lib.atoma_sample_static_init() == 0
+    rows, vocab = 6, 7001
+    logits, temperature, top_k, top_p, uniform = _inputs(rows, vocab, 9)
+    tok = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
+    lg = torch.zeros((rows,), dtype=torch.float32, device="cuda")
+    work = torch.empty((rows, vocab), dtype=torch.float32, device="cuda")
+    tok_w, lg_w = torch.empty_like(tok), torch.empty_like(lg)
+    torch.cuda.synchronize()
+
+    def static_call():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        return lib.atoma_sample_static(_ptr(logits), vocab, rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                       _ptr(uniform), _ptr(tok), _ptr(lg), stream)
+
+    def workspace_call():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        assert lib.atoma_sample(_ptr(logits), vocab, rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                _ptr(uniform), _ptr(work), _ptr(tok_w), _ptr(lg_w), stream) == 0
+
+    before = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    assert static_call() == 0
+    torch.cuda.synchronize()
+    after = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    assert after == before, f"memory moved around the call: {before} -> {after}"
+    workspace_call()
+    torch.cuda.synchronize()
+    assert torch.equal(tok, tok_w) and torch.equal(lg, lg_w)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        assert static_call() == 0
+    g = torch.Generator().manual_seed(10)
+    for replay in range(4):
+        # new inputs in the same buffers, eager work of the program's own, then the replay
+        logits.copy_((torch.randn((rows, vocab), generator=g) * 3.0).cuda())
+        uniform.copy_(torch.rand((rows,), generator=g).cuda())
+        tok.fill_(-1)
+        workspace_call()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(tok, tok_w) and torch.equal(lg, lg_w), f"replay {replay}"
+        assert int(tok[0]) == int(logits[0].argmax())          # row 0 is greedy

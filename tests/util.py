@@ -50,8 +50,19 @@ TINY_E = {
     "num_attention_heads": 3, "num_key_value_heads": 1, "rms_norm_eps": 3e-6, "rope_theta": 250000.0,
     "max_position_embeddings": 1024, "tie_word_embeddings": False,
 }
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
-NORM_JITTER = {"A": 0.0, "B": 0.1, "C": 0.1, "D": 0.1, "E": 0.1}
+# heads of 40 columns: a multiple of 8 that is no multiple of 16, which the reference's attention kernels take too
+# (csrc/src/lib.rs:136-143, 790); here the general attention kernel runs them in both dtypes, while the bfloat16
+# products with their rotary and SiLU epilogues still apply (widths that are multiples of 32)
+TINY_F = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 160, "intermediate_size": 224, "vocab_size": 613, "num_hidden_layers": 2,
+    "num_attention_heads": 4, "num_key_value_heads": 2, "rms_norm_eps": 2e-5, "rope_theta": 10000.0,
+    "rope_scaling": {"factor": 4.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 128, "rope_type": "llama3"},
+    "max_position_embeddings": 512, "tie_word_embeddings": True,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
+NORM_JITTER = {"A": 0.0, "B": 0.1, "C": 0.1, "D": 0.1, "E": 0.1, "F": 0.1}
 
 
 def make_model_dir(path: str, cfg: dict, seed: int, dtype: str, norm_jitter: float = 0.0) -> str:
