@@ -57,8 +57,13 @@ struct FuseArgs {
 // against the activations of its first and of its second 32 values, into two accumulators; rows 0..7 of the first
 // and rows 8..15 of the second are the wave's sums (the other halves are products of mismatched K and are dropped),
 // and they meet once, after the last step.
+// PACK (half tiles, at most 8 rows of A): the activations are packed the same way, lanes 8..15 holding rows 0..7 of
+// A 32 values of K further on, so one fragment of A and one MFMA a step serve both halves: the quadrant (rows 0..7 of
+// W, rows 0..7 of A) holds the sums over the first 32 values of every step, the quadrant (8..15, 8..15) those over the
+// second, and they meet once, after the last step.  Half as many loads of the activations, which every workgroup
+// fetches whole.
 template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false, bool ROPE = false, int UO = 0,
-          bool HALF = false>
+          bool HALF = false, bool PACK = false>
 __global__ void __launch_bounds__(64 * WN * WK)
 gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
                    int K, int lda, int ldw, int ldc, size_t plane, RopeArgs ra, FuseArgs fa) {
@@ -70,6 +75,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   const int wn = wave % WN, wk = wave / WN;
   const int r16 = lane & 15, kg = lane >> 4;
   static_assert(!HALF || (RT == 1 && MT == 1 && !SWIGLU && !ROPE), "half tiles: one tile, residual epilogue");
+  static_assert(!PACK || HALF, "packed activations go with half tiles");
   const int n_base = (blockIdx.x * WN + wn) * (HALF ? 8 : RT * 16);
   constexpr int KSTEP = HALF ? 64 : 32;               // values of K that a wave's step covers
   const int k_slices = gridDim.y * WK;
@@ -87,9 +93,9 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   const uint16_t* ap[MT];
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
-    int row = m * 16 + r16;
+    int row = m * 16 + (PACK ? (r16 & 7) : r16);
     if (row > M - 1) row = M - 1;
-    ap[m] = a + (size_t)row * lda + k_begin + kg * 8;
+    ap[m] = a + (size_t)row * lda + k_begin + kg * 8 + ((PACK && r16 >= 8) ? 32 : 0);
   }
 
   f32x4 acc[RT][MT];
@@ -134,7 +140,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
       for (int r = 0; r < RT; ++r) wf[buf][u][r] = *reinterpret_cast<const bf16x8*>(wp[r] + k0 + u * KSTEP);
 #pragma unroll
       for (int m = 0; m < MT; ++m) af[buf][u][m] = *reinterpret_cast<const bf16x8*>(ap[m] + k0 + u * KSTEP);
-      if constexpr (HALF) af_hi[buf][u] = *reinterpret_cast<const bf16x8*>(ap[0] + k0 + u * KSTEP + 32);
+      if constexpr (HALF && !PACK) af_hi[buf][u] = *reinterpret_cast<const bf16x8*>(ap[0] + k0 + u * KSTEP + 32);
     }
   };
   auto multiply = [&](int buf) {
@@ -145,7 +151,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
 #pragma unroll
         for (int m = 0; m < MT; ++m)
           acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[buf][u][r], af[buf][u][m], acc[r][m], 0, 0, 0);
-      if constexpr (HALF)
+      if constexpr (HALF && !PACK)
         acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[buf][u][0], af_hi[buf][u], acc_hi, 0, 0, 0);
     }
   };
@@ -176,12 +182,16 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
 #pragma unroll
       for (int m = 0; m < MT; ++m)
         acc[r][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt[r], at[m], acc[r][m], 0, 0, 0);
-    if constexpr (HALF) {
+    if constexpr (HALF && !PACK) {
       const bf16x8 at_hi = *reinterpret_cast<const bf16x8*>(ap[0] + k + 32);
       acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt[0], at_hi, acc_hi, 0, 0, 0);
     }
   }
-  if constexpr (HALF) {
+  if constexpr (PACK) {
+    // (row n of W, row r of A), n and r below 8: the lane of (n + 8, r + 8), 32 + 8 lanes further, has the other half
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[0][0][i] += __shfl(acc[0][0][i], (lane + 40) & 63, 64);
+  } else if constexpr (HALF) {
     // rows 0..7 of the tile (lanes kg < 2) take the sums of the second halves from rows 8..15 (the lane 32 further)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -493,9 +503,14 @@ extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M,
   if (rt == R && wk == WK_ && depth == U_ && (half != 0) == H_) {                                                  \
     const int cols = H_ ? WN_ * 8 : WN_ * R * 16;                                                                  \
     dim3 grid((N + cols - 1) / cols, 1), block(64 * WN_ * WK_);                                                    \
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN_, WK_, float, false, false, U_, H_>), grid, block, 0, stream,  \
-                       (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0, RopeArgs{}, \
-                       fa);                                                                                        \
+    if (H_ && M <= 8)                                                                                              \
+      hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN_, WK_, float, false, false, U_, H_, H_>), grid, block, 0,    \
+                         stream, (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0,   \
+                         RopeArgs{}, fa);                                                                          \
+    else                                                                                                           \
+      hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN_, WK_, float, false, false, U_, H_>), grid, block, 0,        \
+                         stream, (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0,   \
+                         RopeArgs{}, fa);                                                                          \
     ATOMA_LAUNCH_CHECK();                                                                                          \
     return 0;                                                                                                      \
   }
