@@ -7,7 +7,8 @@
 // kernels: csrc/src/lib.rs:69-100).  The four waves of a workgroup run four consecutive tasks; the host orders
 // tasks so that these read the same keys (the heads of one tile, or neighbouring key ranges of one request) and
 // meet in the L1 cache.  A task either covers all keys its rows may see and writes the output, or covers one
-// chunk of 128 to 512 keys and writes a partial result (normalised output and log-sum-exp) that the combine kernel merges:
+// chunk of 128 to 512 keys and writes a partial result (normalised output and log-sum-exp); the wave that finishes a
+// row piece's last chunk merges them (or, without counters, the combine kernel does):
 // the split keeps the GPU busy when few rows face many keys (csrc/kernels/flash_fwd_kernel.h:1131-1310 is the
 // reference's combine).  Chunk borders are multiples of the chunk size, so a partial result covers the same keys
 // whatever else the batch holds.
@@ -48,7 +49,8 @@ struct Task {
   int32_t k_begin;  // keys [k_begin, k_end) by absolute position; k_begin is a multiple of 32
   int32_t k_end;
   int32_t dest;     // < 0: write the output; else index of the partial result
-  int32_t n_parts;  // combine tasks: number of partial results starting at dest
+  int32_t n_parts;  // combine tasks: number of partial results starting at dest; tasks that leave a partial result:
+                    // index of their combine task (the record that says where the row piece's parts start and how many)
   int32_t tok_base; // row of the entry's first token in the step's batch
   int32_t count;    // tokens of the entry in this step
   int32_t pos0;     // absolute position of the entry's first token
@@ -66,6 +68,88 @@ __device__ __forceinline__ bf16x8 pack8(const float* v) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) r[i] = (__bf16)v[i];
   return r;
+}
+
+
+// Stores and loads that go through to memory, past the L2 of this wave's XCD (which the other XCDs' waves do not
+// see): what a wave hands to a wave of another workgroup inside one launch.
+__device__ __forceinline__ void store_through(float* p, float4 v) {
+  unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+  const unsigned long long lo = (unsigned long long)__float_as_uint(v.x) | ((unsigned long long)__float_as_uint(v.y) << 32);
+  const unsigned long long hi = (unsigned long long)__float_as_uint(v.z) | ((unsigned long long)__float_as_uint(v.w) << 32);
+  __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(q + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_through(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float4 load_through(const float* p) {
+  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
+  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return make_float4(__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)), __uint_as_float((unsigned)hi),
+                     __uint_as_float((unsigned)(hi >> 32)));
+}
+__device__ __forceinline__ float load_through1(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Merge the partial results of one piece of 32 rows, by one wave: out = sum_s w_s O_s / sum_s w_s with
+// w_s = exp2(lse_s - max).  The live rows' values are dealt to the lanes four at a time; a lane walks the parts in the
+// order of their index, BATCH in flight (each round a trip to memory: the fewer rounds the better, but the parts in
+// flight need registers, and the launches that prompts use must not pay for them with a wave less a SIMD), and follows the
+// running maximum as the attention loop does, so the result depends on the parts alone.  comb: the piece's combine record (dest: first part, n_parts: how many).
+template <int BATCH>
+__device__ __forceinline__ void merge_parts(const float* __restrict__ part_o, const float* __restrict__ part_lse,
+                                            uint16_t* __restrict__ out, int out_stride, const Task& comb, int kvh,
+                                            int nh, int nkv, int lane) {
+  constexpr int Q = HD / 4;                        // pieces of four values in a row
+  const int g = nh / nkv;
+  const size_t part_stride = (size_t)nkv * 32;     // rows between two parts of the same (KV head, row)
+  const size_t base0 = ((size_t)comb.dest * nkv + kvh) * 32;
+  const int n_parts = comb.n_parts;
+  for (int idx = lane; idx < 32 * Q; idx += 64) {
+    const int c = idx / Q, d = (idx % Q) * 4;
+    const int r = comb.row0 + c;
+    const int hq = r / comb.qt, tok = comb.tok0 + r % comb.qt;
+    if (hq >= g || tok >= comb.count) continue;
+    const float* pl = part_lse + base0 + c;
+    const float* po = part_o + (base0 + c) * HD + d;
+    float m = -INFINITY, wsum = 0.f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s0 = 0; s0 < n_parts; s0 += BATCH) {
+      float ls[BATCH];
+      float4 v[BATCH];
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        const int sp = s0 + u < n_parts ? s0 + u : n_parts - 1;
+        ls[u] = load_through1(pl + (size_t)sp * part_stride);
+        v[u] = load_through(po + (size_t)sp * part_stride * HD);
+      }
+      float mb = m;
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u)
+        if (s0 + u < n_parts) mb = fmaxf(mb, ls[u]);
+      const float m_use = (mb == -INFINITY) ? 0.f : mb;
+      const float corr = __builtin_amdgcn_exp2f(m - m_use);      // exp2(-inf) = 0 on the first round
+      wsum *= corr;
+      acc.x *= corr, acc.y *= corr, acc.z *= corr, acc.w *= corr;
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        if (s0 + u < n_parts) {
+          const float w = __builtin_amdgcn_exp2f(ls[u] - m_use);
+          wsum += w;
+          acc.x += w * v[u].x, acc.y += w * v[u].y, acc.z += w * v[u].z, acc.w += w * v[u].w;
+        }
+      }
+      m = mb;
+    }
+    const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+    uint2 pk;
+    pk.x = (uint32_t)f32_to_bf16_bits(acc.x * inv) | ((uint32_t)f32_to_bf16_bits(acc.y * inv) << 16);
+    pk.y = (uint32_t)f32_to_bf16_bits(acc.z * inv) | ((uint32_t)f32_to_bf16_bits(acc.w * inv) << 16);
+    *reinterpret_cast<uint2*>(out + (size_t)(comb.tok_base + tok) * out_stride + (size_t)(kvh * g + hq) * HD + d) = pk;
+  }
 }
 
 // KSPLIT waves share a task: wave h of them takes the blocks of 32 keys number h, h + KSPLIT, ... of the task's
@@ -89,7 +173,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
                       const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
                       float* __restrict__ part_o, float* __restrict__ part_lse, const Task* __restrict__ tasks,
                       int n_tasks, const int32_t* __restrict__ block_tables, int max_blocks, float scale,
-                      int window, int nh, int nkv) {
+                      int window, int nh, int nkv, int32_t* __restrict__ counters) {
   // (a wave's number is the same in all its lanes; saying so keeps what follows from it in scalar registers)
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave % TASKS, part = wave / TASKS;   // which of the workgroup's tasks, which share of its keys
@@ -391,9 +475,10 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     }
   } else {
     // a partial result is one piece of 32 rows (the host gives such tasks one piece, whatever RT is);
-    // rows that are not live are never read by the combine kernel (their log-sum-exp is, and says -inf)
+    // rows that are not live are never read by the merge (their log-sum-exp is, and says -inf)
     const float inv = l[0] > 0.f ? 1.0f / l[0] : 0.f;
     float* po = part_o + (((size_t)task.dest * nkv + kvh) * 32 + c) * HD;
+    const bool merge_here = counters != nullptr;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
 #pragma unroll
@@ -402,18 +487,43 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
         if (row_ok[0] && (HD % 32 == 0 || d < HD)) {
           float4 v = make_float4(o[0][dt][q4 * 4 + 0] * inv, o[0][dt][q4 * 4 + 1] * inv, o[0][dt][q4 * 4 + 2] * inv,
                                  o[0][dt][q4 * 4 + 3] * inv);
-          *reinterpret_cast<float4*>(po + d) = v;
+          if (merge_here) store_through(po + d, v);
+          else *reinterpret_cast<float4*>(po + d) = v;
         }
       }
-    if (hg == 0)
-      part_lse[((size_t)task.dest * nkv + kvh) * 32 + c] = l[0] > 0.f ? m[0] + __builtin_amdgcn_logf(l[0]) : -INFINITY;
+    const float lse = l[0] > 0.f ? m[0] + __builtin_amdgcn_logf(l[0]) : -INFINITY;
+    float* pl = part_lse + ((size_t)task.dest * nkv + kvh) * 32 + c;
+    if (hg == 0) {
+      if (merge_here) store_through(pl, lse);
+      else *pl = lse;
+    }
+    if (merge_here) {
+      // The wave that finishes the last chunk of a row piece merges all of its chunks.  The parts go through to memory
+      // (stores and loads that pass the L2 of this wave's XCD, which other XCDs do not see), this wave's stores have
+      // arrived before it counts itself in, and the counter is a device-wide atomic: no fence that would write back or
+      // invalidate a whole cache is needed.  The parts are added in the order of their index, whoever comes last.
+      const Task comb = tasks[n_tasks + task.n_parts];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_s_waitcnt(0);
+      int32_t* counter = counters + (size_t)task.n_parts * nkv + kvh;
+      int before = 0;
+      if (lane == 0) before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      before = __builtin_amdgcn_readfirstlane(before);
+      if (before + 1 == comb.n_parts) {
+        if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        // (a wave a task: the launches of decoded tokens alone, which have registers to spare)
+        merge_parts<(KSPLIT == 1 ? 16 : 8)>(part_o, part_lse, out, out_stride, comb, kvh, nh, nkv, lane);
+      }
+    }
   }
 }
 
 // Merge partial results: out = sum_s w_s O_s / sum_s w_s with w_s = exp2(lse_s - max lse).
-// A kernel of its own on purpose: letting the last wave to finish a row's chunks merge them needs device-scope
-// fences around a counter, and on this GPU those write back and invalidate the L2 of the wave's XCD, which
-// measured far dearer (a decode step 1.6 times as long) than this second launch.
+// The kernel of its own, for callers that bring no counters (the attention kernel then leaves the parts to it).
+// With counters the last wave to finish a row piece's chunks merges them inside the attention kernel: done with
+// device-scope fences around the counter that measured far dearer than this second launch (a decode step 1.6 times as
+// long: such fences write back and invalidate the L2 of the wave's XCD), done with stores and loads that go through
+// to memory it saves the launch.
 // One block per (combine task, KV head).  The log-sum-exps of all parts are first brought into LDS by all
 // threads at once and turned into weights there; then the valid rows of the task (group x tokens, at most 32)
 // times HD output values are spread over the 256 threads, and each adds its parts in order of their index with
@@ -532,11 +642,14 @@ extern "C" int atoma_attention_mfma_head_size() { return HD; }
 extern "C" int atoma_attention_mfma_max_ksplit() { return kSplit8Fits ? 8 : kSplit2Fits ? 2 : 1; }
 extern "C" int atoma_attention_mfma_max_row_tiles() { return kTwoPieces ? 2 : 1; }
 
-// tasks: device array of n_tasks Task records (main kernel), followed by n_combine records for the combine kernel.
+// tasks: device array of n_tasks Task records (main kernel), followed by n_combine records of the row pieces whose
+// keys are cut into chunks.  counters: null, or n_combine * nkv zeros (left as zeros again): the attention kernel then
+// merges the chunks itself and the combine kernel does not run.
 extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kcache, const void* vcache, void* out,
                                     int out_stride, float* part_o, float* part_lse, const int32_t* tasks, int n_tasks,
                                     int n_combine, const int32_t* block_tables, int max_blocks, float scale,
-                                    int window, int nh, int nkv, int ksplit, int row_tiles, hipStream_t stream) {
+                                    int window, int nh, int nkv, int ksplit, int row_tiles, int32_t* counters,
+                                    hipStream_t stream) {
   if (n_tasks <= 0) return 0;
   // row_tiles: 1, or 2: the tasks that write the output cover 64 rows (Task::tiles says so), two waves a task
   if (row_tiles != 1 && !(row_tiles == 2 && kTwoPieces && ksplit == 2)) return ATOMA_ERR_SHAPE;
@@ -554,7 +667,7 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
                        dim3(64 * T * KS), BYTES,                                                                   \
                        stream, (const uint16_t*)q, q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,     \
                        (uint16_t*)out, out_stride, part_o, part_lse, t, n_tasks, block_tables, max_blocks, scale,  \
-                       window, nh, nkv);                                                                           \
+                       window, nh, nkv, counters);                                                                 \
   } while (0)
   if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
   else if (ksplit == 2 && row_tiles == 2) ATOMA_ATTN(4, 2, 2 * kMerge2Bytes, (kTwoPieces ? 2 : 1));
@@ -563,7 +676,7 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
   else return ATOMA_ERR_SHAPE;
 #undef ATOMA_ATTN
   ATOMA_LAUNCH_CHECK();
-  if (n_combine > 0) {
+  if (n_combine > 0 && counters == nullptr) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(n_combine, nkv), dim3(256), 0, stream, part_o, part_lse,
                        (uint16_t*)out, out_stride, t + n_tasks, nh, nkv);
     ATOMA_LAUNCH_CHECK();

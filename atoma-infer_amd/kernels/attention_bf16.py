@@ -74,6 +74,18 @@ WHOLE_SHORT_WALKS = ((96, 8192 * 64), (32, 1536 * 64), (1, 1024 * 64))
 LONG_KEYS = 16384
 
 
+# Contexts up to which the chunks of a row piece are merged by the attention kernel itself (the wave that finishes the
+# last chunk does it; at most 18 chunks then): measured on MI355X, 0.5 to 1 us quicker than the merging kernel at
+# 1,024 keys and equal at 2,048 for the pair alone, and 10 to 27 us quicker over the 16 layers of a decode step of 8
+# requests or of 1; from 4,096 keys on one wave's walk over the parts costs more than the second launch.
+MERGE_MAX_KEYS = 2304
+MERGE_IN_KERNEL = True        # False: always the merging kernel (tests run both)
+
+
+def merges_in_kernel(max_keys: int) -> bool:
+    return MERGE_IN_KERNEL and max_keys <= MERGE_MAX_KEYS
+
+
 def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False, head_size: int = 64,
               ) -> Tuple[int, int]:
     """(keys per partial task, waves that share a task) for the entries of a step that are split along their keys;
@@ -96,6 +108,9 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False
         if pairs >= WHOLE_MIN_PAIRS or any(pairs >= p and walk <= w for p, w in WHOLE_SHORT_WALKS):
             return 0, 8
     tasks = n_split * -(-max_keys // CHUNK) * kv_heads
+    if merges_in_kernel(max_keys):
+        # (with the chunks merged by the attention kernel itself; measured at 1,024 and 2,048 keys, 1 to 16 requests)
+        return (128, 1) if tasks <= 300 else (CHUNK, 2)
     if tasks <= 160:
         return 128, 1
     if tasks <= 540 and max_keys <= 4096:
@@ -202,7 +217,8 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     """Task records [n, 12] int32 (main tasks, then combine tasks), and (n_main, n_combine, n_partials, waves that
     share a task: two when a prompt tile walks many keys, else what ``chunk_for`` says for the split entries; pieces
     of 32 rows that a task which writes the output covers: ``row_tiles`` if the step has such tasks, walks at least
-    ``TWO_PIECES_MIN_KEYS`` keys and two waves may share a task, else 1).
+    ``TWO_PIECES_MIN_KEYS`` keys and two waves may share a task, else 1; whether the attention kernel merges the
+    chunks itself: ``merges_in_kernel``).
 
     Main tasks are padded to a multiple of 4 (one workgroup runs 4) and ordered so that tasks sharing keys are
     neighbours and long tasks come first.  With ``bucket_keys`` (decode steps: one token per entry; the context
@@ -231,13 +247,14 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
                                       and int(starts[e]) + int(counts[e]) - first_key >= SPLIT_MIN_KEYS)
 
     split_entries = [e for e in range(len(starts)) if splits(e)]
-    chunk, waves = CHUNK, 1
+    chunk, waves, merge = CHUNK, 1, False
     if split_entries:
         most = bucket if bucket is not None else max(int(starts[e]) + int(counts[e]) for e in split_entries)
         if bucket is not None and window > 0:
             most = min(most, window + CHUNK)
         chunk, waves = chunk_for(len(split_entries), most, kv_heads)
         waves = min(waves, max_waves)
+        merge = merges_in_kernel(most)
     for e in range(len(starts)):
         start, count = int(starts[e]), int(counts[e])
         qt = min(qt_max, count)
@@ -260,11 +277,13 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
                 # slot j holds chunk c_first + j
                 slots = _chunk_slots(bucket, chunk, window) if bucket is not None else c_last - c_first + 1
                 for row0 in live:
+                    piece_index = len(combine)       # a chunk's task names the record of its row piece
                     combine.append((e, tok0, qt, row0, 0, 0, n_part, c_last - c_first + 1) + tail)
                     for j in range(slots):
                         c = c_first + j
                         if c <= c_last:
-                            split.append((e, tok0, qt, row0, c * chunk, min((c + 1) * chunk, k_end), n_part + j, 0) + tail)
+                            split.append((e, tok0, qt, row0, c * chunk, min((c + 1) * chunk, k_end), n_part + j,
+                                          piece_index) + tail)
                         elif bucket is not None:
                             split.append(null)
                     n_part += slots
@@ -291,7 +310,7 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
         waves = 2
     if row_tiles > 1 and len(head):
         waves = 2                     # tasks of two pieces run in the launch of two waves a task only
-    return arr, (len(head) + len(split), len(combine), n_part, waves, row_tiles if len(head) else 1)
+    return arr, (len(head) + len(split), len(combine), n_part, waves, row_tiles if len(head) else 1, merge)
 
 
 def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int, kv_heads: int,
@@ -317,7 +336,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
         whole[..., 8] = np.arange(s)[:, None]
         whole[..., 9] = 1
         whole[..., 10] = starts[:, None]
-        return whole.reshape(-1, 12), (s * row_chunks, 0, 0, waves, 1)
+        return whole.reshape(-1, 12), (s * row_chunks, 0, 0, waves, 1, False)
     slots = _chunk_slots(bucket, chunk, window)
     j = np.arange(slots, dtype=np.int64)
     c_first, c_last = lo // chunk, (k_end - 1) // chunk
@@ -334,6 +353,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     main[..., 5] = np.where(v, np.minimum((c + 1) * chunk, k_end[:, None])[:, None, :], 0)
     part = (e[:, None, None] * row_chunks + rc[None, :, None]) * slots + j[None, None, :]
     main[..., 6] = np.where(v, part, -1)
+    main[..., 7] = np.where(v, e[:, None, None] * row_chunks + rc[None, :, None], 0)      # the row piece's record
     main[..., 8] = np.where(v, e[:, None, None], 0)
     main[..., 9] = np.where(v, 1, 0)
     main[..., 10] = np.where(v, starts[:, None, None], 0)
@@ -353,11 +373,29 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     comb[..., 9] = 1
     comb[..., 10] = starts[:, None]
     arr = np.concatenate([main, comb.reshape(-1, 12)])
-    return arr, (len(main), s * row_chunks, s * row_chunks * slots, waves, 1)
+    return arr, (len(main), s * row_chunks, s * row_chunks * slots, waves, 1, merges_in_kernel(keys))
 
 
 def plan_key(group: int, window: int, kv_heads: int, hd: int):
     return ("attention_mfma_tasks", group, window, kv_heads, hd)
+
+
+# Counters of the chunks that have finished, one per (row piece whose keys are cut into chunks, KV head): zeros that
+# the attention kernel leaves as zeros.  One array per device, made at first use (a step's first run is never
+# inside a recording); a step with more row pieces than it holds leaves its chunks to the merging kernel.
+MERGE_COUNTERS = 1 << 16
+_counters: Dict[torch.device, torch.Tensor] = {}
+
+
+def _merge_counters(device: torch.device, needed: int) -> Optional[torch.Tensor]:
+    if needed > MERGE_COUNTERS:
+        return None
+    t = _counters.get(device)
+    if t is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        t = _counters[device] = torch.zeros(MERGE_COUNTERS, dtype=torch.int32, device=device)
+    return t
 
 
 def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, hd) -> bool:
@@ -379,7 +417,7 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
                                     max_waves=max_waves_for(hd), row_tiles=max_row_tiles_for(hd))
             plan = (torch.from_numpy(arr).to(q.device), meta)
             ctx.scratch[key] = plan
-    tasks, (n_main, n_comb, n_part, waves, row_tiles) = plan
+    tasks, (n_main, n_comb, n_part, waves, row_tiles, merge) = plan
     ksplit = min(waves, lib(hd).atoma_attention_mfma_max_ksplit())
     part_o = part_lse = None
     if n_part:
@@ -391,8 +429,10 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
             ctx.scratch[ws_key] = ws
         part_o, part_lse = ws
     bt = cache.block_tables
+    counters = _merge_counters(q.device, n_comb * nkv) if n_comb and merge else None
     _check(lib(hd).atoma_attention_mfma(_p(q), q.stride(0), _p(k_cache), _p(v_cache), _p(out), out.stride(0),
                                         _p(part_o), _p(part_lse), _p(tasks), n_main, n_comb, _p(bt), bt.shape[1],
-                                        ctypes.c_float(scale), int(window), nh, nkv, ksplit, row_tiles, _stream()),
+                                        ctypes.c_float(scale), int(window), nh, nkv, ksplit, row_tiles, _p(counters),
+                                        _stream()),
            "attention_mfma")
     return True

@@ -7,7 +7,7 @@ from atoma_infer_amd.kernels import attention_bf16 as A
 
 
 def coverage(arr, meta, starts, counts, group, window):
-    n_main, n_comb, n_part, waves, tiles = meta
+    n_main, n_comb, n_part, waves, tiles, merge = meta
     assert waves in (1, 2, 8) and tiles in (1, 2) and (tiles == 1 or waves == 2)
     main, comb = arr[:n_main], arr[n_main:]
     assert len(comb) == n_comb and (n_main % 4 == 0 or waves == 8)    # (eight waves: one task a workgroup)
@@ -129,7 +129,7 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     counts = np.ones(s, dtype=np.int32)
     bucket = -(-int(starts.max() + 1) // 256) * 256
     arr, meta = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
-    assert meta == (s * -(-group // 32), 0, 0, 8, 1)
+    assert meta == (s * -(-group // 32), 0, 0, 8, 1, False)
     coverage(arr, meta, starts, counts, group, window)
     # a head size that does not allow eight waves, or few pairs with many keys to walk: chunks as before
     assert A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=2)[1][1] > 0
@@ -139,7 +139,7 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     # few pairs with few keys to walk: whole ranges again (the second kernel would cost more than the walk)
     near = np.full(8, 999, dtype=np.int32)
     arr2, meta2 = A.build_tasks(near, counts[:8], group, 0, 1024, kv_heads=8, max_waves=8)
-    assert meta2 == (8 * -(-group // 32), 0, 0, 8, 1)
+    assert meta2 == (8 * -(-group // 32), 0, 0, 8, 1, False)
     coverage(arr2, meta2, near, counts[:8], group, 0)
     assert A.build_tasks(near, counts[:8], group, 0, 1024, kv_heads=8, max_waves=8, head_size=128)[1][1] > 0
     # twelve requests of 8 KV heads: whole ranges up to 8,192 keys of head size 64, 4,096 of head size 128

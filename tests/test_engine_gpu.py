@@ -17,8 +17,9 @@ pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
 # how the bfloat16 attention plans decoded tokens: as its planner decides (at the contexts of these tests: whole key
 # ranges walked by eight waves, where the head size allows them), or in chunks merged by a second kernel, as it does
-# at long contexts with few requests; the float32 attention has one way only
-DTYPE_TASKS = [(d, "planned") for d in DTYPES] + [("bfloat16", "chunks")]
+# at long contexts with few requests (merged by the attention kernel itself, or by a second kernel); the float32
+# attention has one way only
+DTYPE_TASKS = [(d, "planned") for d in DTYPES] + [("bfloat16", "chunks"), ("bfloat16", "chunks, second kernel")]
 PAGE = {"A": 4, "B": 16, "C": 16, "D": 16, "E": 16, "F": 16}
 
 
@@ -120,8 +121,8 @@ def test_whole_prompts(model_dirs, name, dtype):
 @pytest.mark.parametrize("dtype,tasks", DTYPE_TASKS)
 @pytest.mark.parametrize("name", list(TINY))
 def test_last_32_one_by_one(model_dirs, name, dtype, tasks, monkeypatch):
-    if tasks == "chunks":
-        force_chunked_decode(monkeypatch)
+    if tasks.startswith("chunks"):
+        force_chunked_decode(monkeypatch, second_kernel=tasks.endswith("second kernel"))
     vocab = TINY[name]["vocab_size"]
     n = lengths(name)[0]
     requests = {"r": random_tokens(n, vocab, 7)}
@@ -155,8 +156,8 @@ def test_portions_of_changing_size(model_dirs, name, dtype):
 def test_mixed_batches_with_few_pages(model_dirs, name, dtype, tasks, monkeypatch):
     """Up to four live requests, portions of some beside decoded tokens of others; the pool is so small that
     pages freed by finished requests are used again at once."""
-    if tasks == "chunks":
-        force_chunked_decode(monkeypatch)
+    if tasks.startswith("chunks"):
+        force_chunked_decode(monkeypatch, second_kernel=tasks.endswith("second kernel"))
     vocab = TINY[name]["vocab_size"]
     lens = {"A": [60, 33, 47, 21, 58, 40, 9, 52], "B": [120, 1, 77, 90, 45, 130, 18, 66],
             "C": [90, 48, 97, 16, 70, 33, 80, 25], "D": [700, 48, 97, 530, 70, 33, 80, 25],
@@ -235,8 +236,8 @@ def test_pages_the_matrix_core_attention_refuses_are_announced(model_dirs):
 @pytest.mark.parametrize("dtype,tasks", DTYPE_TASKS)
 def test_first_tokens_and_long_decoding(model_dirs, dtype, tasks, monkeypatch):
     """A one-token prompt, then everything decoded token by token up to the model's last position."""
-    if tasks == "chunks":
-        force_chunked_decode(monkeypatch)
+    if tasks.startswith("chunks"):
+        force_chunked_decode(monkeypatch, second_kernel=tasks.endswith("second kernel"))
     name = "A"
     vocab, n = TINY[name]["vocab_size"], TINY[name]["max_position_embeddings"]
     requests = {"r": random_tokens(n, vocab, 9)}

@@ -724,7 +724,7 @@ def test_attention_whole_ranges_with_eight_waves(window, more):
     ctx, cache = FakeCtx(starts, counts), FakeCache(bt, page)
     bucket = -(-max(lens) // 256) * 256
     arr, meta = A.build_tasks(ctx.h_starts, ctx.h_counts, nh // nkv, window, bucket, kv_heads=nkv, max_waves=8)
-    assert meta[1:] == (0, 0, 8, 1)
+    assert meta[1:] == (0, 0, 8, 1, False)
     ctx.plans = {A.plan_key(nh // nkv, window, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
     scale = 1.0 / math.sqrt(hd)
     assert A.try_attention(q, kc, vc, out, ctx, cache, scale, window, nh, nkv, hd)
@@ -758,20 +758,24 @@ def test_tokens_outside_the_table_and_rows_of_nan_do_no_harm():
             assert tok[0] == int(torch.argmax(logits[0])) and tok[3] == 0
 
 
-@pytest.mark.parametrize("whole", [False, True])
+PLANS = ["chunks", "chunks, second kernel", "whole"]
+
+
+@pytest.mark.parametrize("plan", PLANS)
 @pytest.mark.parametrize("nh,nkv,hd", [(40, 1, 64), (33, 1, 32), (6, 2, 112), (64, 2, 64), (3, 3, 208)])
-def test_decode_plans_with_large_groups(nh, nkv, hd, whole, monkeypatch):
+def test_decode_plans_with_large_groups(nh, nkv, hd, plan, monkeypatch):
     """The task lists of decode steps as the engine builds them (every request owns its bucket's chunk slots), for
-    groups of more than 32 heads, which take several pieces of rows: chunks merged by the second kernel, and whole
-    key ranges walked by eight waves."""
+    groups of more than 32 heads, which take several pieces of rows: chunks merged by the wave that finishes the last
+    one or by the second kernel, and whole key ranges walked by eight waves."""
     import numpy as np
     from atoma_infer_amd.kernels import attention_bf16
+    whole = plan == "whole"
     if whole:
         if attention_bf16.max_waves_for(hd) < 8:
             pytest.skip("eight waves a task do not fit this head size")
         monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 2)
     else:
-        force_chunked_decode(monkeypatch)
+        force_chunked_decode(monkeypatch, second_kernel=plan.endswith("second kernel"))
     group, page = nh // nkv, 16
     starts = [700, 129, 15, 256, 511]
     counts = [1] * len(starts)
@@ -784,6 +788,7 @@ def test_decode_plans_with_large_groups(nh, nkv, hd, whole, monkeypatch):
     arr, meta = attention_bf16.build_tasks(np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32),
                                            group, 0, 3 * 256, kv_heads=nkv, max_waves=attention_bf16.max_waves_for(hd))
     assert (meta[1] == 0) == whole                       # no merge records with whole ranges
+    assert meta[5] == (plan == "chunks")
     ctx.plans = {attention_bf16.plan_key(group, 0, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
     scale = 1.0 / math.sqrt(hd)
     # the block tables of a bucket of three cover 768 keys
@@ -797,18 +802,19 @@ def test_decode_plans_with_large_groups(nh, nkv, hd, whole, monkeypatch):
         assert err < 2e-2, f"request {e} at {s}: {err:.3e}"
 
 
-@pytest.mark.parametrize("whole", [False, True])
+@pytest.mark.parametrize("plan", PLANS)
 @pytest.mark.parametrize("window", [64, 200, 1000])
-def test_decode_plans_behind_a_window(window, whole, monkeypatch):
+def test_decode_plans_behind_a_window(window, plan, monkeypatch):
     """Decoded tokens far behind a window, planned as the engine plans them: in chunks, their requests own slots only
     for the chunks a window can touch, the first of which is wherever the window begins; as whole ranges, eight
     waves begin where the window does."""
     import numpy as np
     from atoma_infer_amd.kernels import attention_bf16
+    whole = plan == "whole"
     if whole:
         monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 2)
     else:
-        force_chunked_decode(monkeypatch)
+        force_chunked_decode(monkeypatch, second_kernel=plan.endswith("second kernel"))
     nh, nkv, hd, page = 8, 2, 64, 16
     starts = [1500, 700, 300, 129, 5]
     counts = [1] * len(starts)

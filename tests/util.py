@@ -122,10 +122,13 @@ def check_greedy_tokens(prompt: List[int], tokens: List[int], chosen_logits: Lis
             f"step {step}: token {tok} is no argmax of the plain model ({float(row[tok]):.5f} < {float(row.max()):.5f})"
 
 
-def force_chunked_decode(monkeypatch):
-    """Make the bfloat16 attention cut the keys of decoded tokens into chunks that a second kernel merges, as it does
-    at long contexts with few requests; at the tiny contexts of tests its planner would let eight waves walk whole
-    key ranges instead."""
+def force_chunked_decode(monkeypatch, second_kernel: bool = False):
+    """Make the bfloat16 attention cut the keys of decoded tokens into chunks, as it does at long contexts with few
+    requests; at the tiny contexts of tests its planner would let eight waves walk whole key ranges instead.  The
+    chunks are merged by the wave that finishes the last one, as at contexts up to about 2,000 keys, or with
+    ``second_kernel`` by the merging kernel, as beyond."""
     from atoma_infer_amd.kernels import attention_bf16
     monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 10 ** 9)
     monkeypatch.setattr(attention_bf16, "WHOLE_SHORT_WALKS", ())
+    if second_kernel:
+        monkeypatch.setattr(attention_bf16, "MERGE_IN_KERNEL", False)
