@@ -19,11 +19,13 @@ def value_index(page_size: int, head_size: int) -> torch.Tensor:
     """int64 [head_size, page_size]: offset of (column d, token t) inside a value tile."""
     d = torch.arange(head_size)[:, None]
     t = torch.arange(page_size)[None, :]
-    if page_size != 16:
+    if page_size % 16:
         return d * page_size + t
+    # runs of 16 tokens, each laid out as a page of 16 tokens
+    run, t = (t // 16) * 16 * head_size, t % 16
     tile, c = d // 32, d % 32
     rows = torch.clamp(head_size - tile * 32, max=32)
-    return tile * 512 + (((t % 8) // 4) * rows + c) * 8 + (t // 8) * 4 + t % 4
+    return run + tile * 512 + (((t % 8) // 4) * rows + c) * 8 + (t // 8) * 4 + t % 4
 
 
 def pack_keys(k: torch.Tensor) -> torch.Tensor:

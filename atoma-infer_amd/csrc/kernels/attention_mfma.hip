@@ -1,5 +1,6 @@
 // bfloat16 attention over the paged cache on the matrix cores, for prompts, portions and decoded tokens alike.
-// Compiled once per head size: -DATOMA_HD=<multiple of 16, at most 256>.  Pages hold 16 tokens.
+// Compiled once per head size and page size: -DATOMA_HD=<multiple of 16, at most 256>, -DATOMA_PAGE=<tokens a page, a
+// multiple of 16; 16 if not given>.
 //
 // Work is cut on the host into tasks, one per wave: 32 query rows against a range of keys.  A row is a
 // (token, query head) pair of one request and one KV head: row r of a tile is head r / qt, token tok0 + r % qt,
@@ -13,7 +14,8 @@
 // reference's combine).  Chunk borders are multiples of the chunk size, so a partial result covers the same keys
 // whatever else the batch holds.
 //
-// Per block of 32 keys (two pages), with v_mfma_f32_32x32x16_bf16:
+// Per block of 32 keys (two runs of 16 tokens: two pages of 16 tokens, or two runs of one or of two larger pages),
+// with v_mfma_f32_32x32x16_bf16:
 //   S^T[key, row] = K[key, :] . Q[row, :]     K page rows are the A operand straight from global memory,
 //                                             Q the B operand, kept in registers for the whole task;
 //   online softmax down the keys of each row in float32 (exp2 with the scale folded in), masked by the row's
@@ -33,7 +35,12 @@ constexpr int HD = ATOMA_HD;
 static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
 constexpr int KSTEPS = HD / 16;        // MFMA steps over the head dimension for S
 constexpr int DTILES = (HD + 31) / 32; // 32-row tiles of O^T
-constexpr int PAGE = 16;
+#ifndef ATOMA_PAGE
+#define ATOMA_PAGE 16
+#endif
+constexpr int PAGE = ATOMA_PAGE;       // tokens a page
+static_assert(PAGE % 16 == 0 && PAGE >= 16, "pages hold a multiple of 16 tokens");
+constexpr int RUNS = PAGE / 16;        // runs of 16 tokens a page; a run of values is laid out as a page of 16 (cache_layout.h)
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kSlack = 8.0f;   // see the softmax in the kernel
 
@@ -213,15 +220,19 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
 #pragma unroll
   for (int t = 0; t < RT; ++t) piece_on[t] = RT == 1 || __ballot(row_ok[t]) != 0;
 
-  // page numbers: lane i asks for the page of block (kb / 16 + i) of the task's request; lanes 0 and 1 hold the two
-  // pages of the block of 32 keys at kb.  Asked for at the top of every turn for the next one, before anything else,
-  // so that waiting for the answer leaves the loads of fragments behind it in flight.
+  // page numbers: lane i asks for page (kb / PAGE + i) of the task's request; lanes 0 and 1 hold the pages that the two
+  // runs of 16 keys of the block at kb may lie in (with pages of 32, 64, ... tokens both in lane 0's).  Asked for at the
+  // top of every turn for the next one, before anything else, so that waiting for the answer leaves the loads of
+  // fragments behind it in flight.
   const int32_t* table = block_tables + (size_t)entry * max_blocks;
   auto page_window = [&](int kb) {
     int b = kb / PAGE + lane;
     if (b > max_blocks - 1) b = max_blocks - 1;
     return table[b];
   };
+  // the second run's page among those lanes, and each run's place in its page (all the same in every lane)
+  auto second_lane = [&](int kb) { return RUNS == 1 ? 1 : (kb + 16) / PAGE - kb / PAGE; };
+  auto run_of = [&](int key) { return RUNS == 1 ? 0 : (key / 16) % RUNS; };
 
   // Q fragments: B operand, lane (row c, k half hg) holds 8 consecutive d per step
   bf16x8 qf[RT][KSTEPS];
@@ -272,18 +283,20 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const uint16_t* const k_tiles = kcache + (size_t)kvh * kv_head_stride;
   const uint16_t* const v_tiles = vcache + (size_t)kvh * kv_head_stride;
   const uint32_t k_lane = (uint32_t)(hg * PAGE + (c & 15)) * 8;
-  auto load_keys = [&](int p0, int p1, bf16x8* kf) {
-    const uint16_t* const t0 = k_tiles + (size_t)__builtin_amdgcn_readfirstlane(p0) * page_stride;
-    const uint16_t* const t1 = k_tiles + (size_t)__builtin_amdgcn_readfirstlane(p1) * page_stride;
+  auto load_keys = [&](int kb, int p0, int p1, bf16x8* kf) {
+    // (a key's 8-column pieces lie PAGE * 8 elements apart, the tokens of a piece side by side: a run starts 16 * 8 in)
+    const uint16_t* const t0 = k_tiles + (size_t)__builtin_amdgcn_readfirstlane(p0) * page_stride + run_of(kb) * 128;
+    const uint16_t* const t1 = k_tiles + (size_t)__builtin_amdgcn_readfirstlane(p1) * page_stride + run_of(kb + 16) * 128;
     const uint16_t* kp = ((c < 16) ? t0 : t1) + k_lane;
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) kf[st] = *reinterpret_cast<const bf16x8*>(kp + st * (2 * PAGE * 8));
   };
   // V^T fragments of both pages: lane (d = dt*32 + c, key slots hg*4..+4 and 8 + hg*4..+4 of each page)
-  auto load_vals = [&](int p0, int p1, bf16x8 (*vf)[DTILES]) {
+  auto load_vals = [&](int kb, int p0, int p1, bf16x8 (*vf)[DTILES]) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const uint16_t* const tile = v_tiles + (size_t)__builtin_amdgcn_readfirstlane(j ? p1 : p0) * page_stride;
+      const uint16_t* const tile = v_tiles + (size_t)__builtin_amdgcn_readfirstlane(j ? p1 : p0) * page_stride +
+                                   run_of(kb + 16 * j) * (16 * HD);
 #pragma unroll
       for (int dt = 0; dt < DTILES; ++dt) {
         const int d = dt * 32 + c;
@@ -314,14 +327,14 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   if (k_first < k_end) {
     const int pw = page_window(k_first);
     p0 = __builtin_amdgcn_readlane(pw, 0);
-    p1 = __builtin_amdgcn_readlane(pw, 1);
-    load_keys(p0, p1, kf);
+    p1 = __builtin_amdgcn_readlane(pw, second_lane(k_first));
+    load_keys(k_first, p0, p1, kf);
   }
   auto turn = [&](int kb, auto more) {
     constexpr bool MORE = decltype(more)::value;
     int pw = 0;
     if constexpr (MORE) pw = page_window(kb + STRIDE);
-    load_vals(p0, p1, vf);
+    load_vals(kb, p0, p1, vf);
     // (no instruction: it keeps the compiler from moving these loads down to where their values are used)
     asm volatile("" ::: "memory");
     // S^T = K Q^T, for each piece of rows against the same fragments of the keys
@@ -338,8 +351,8 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
     }
     if constexpr (MORE) {
       p0 = __builtin_amdgcn_readlane(pw, 0);
-      p1 = __builtin_amdgcn_readlane(pw, 1);
-      load_keys(p0, p1, kf);
+      p1 = __builtin_amdgcn_readlane(pw, second_lane(kb + STRIDE));
+      load_keys(kb + STRIDE, p0, p1, kf);
       asm volatile("" ::: "memory");
     }
 
@@ -639,6 +652,7 @@ template <typename K> static int allow_lds(K kernel, size_t bytes) {
 }
 
 extern "C" int atoma_attention_mfma_head_size() { return HD; }
+extern "C" int atoma_attention_mfma_page_size() { return PAGE; }
 extern "C" int atoma_attention_mfma_max_ksplit() { return kSplit8Fits ? 8 : kSplit2Fits ? 2 : 1; }
 extern "C" int atoma_attention_mfma_max_row_tiles() { return kTwoPieces ? 2 : 1; }
 

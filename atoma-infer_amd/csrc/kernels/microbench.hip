@@ -7,18 +7,25 @@ using namespace atoma;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-// every thread reads 16-byte words with a stride of the whole grid, four in flight; what is read is folded into one
-// word that is stored only if it has a value it practically never has
+// every thread reads 16-byte words with a stride of the whole grid, U in flight; all of what is read is folded into
+// one word (so that the loads stay 16 bytes wide) that is stored only if it has a value it practically never has
+template <int U>
 __global__ void __launch_bounds__(256)
 probe_read_kernel(const uint4* __restrict__ src, size_t n16, uint32_t* __restrict__ sink) {
   uint32_t acc = 0;
   const size_t stride = (size_t)gridDim.x * 256;
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
-    acc ^= a.x ^ b.y ^ c.z ^ d.w;
+  for (; i + (U - 1) * stride < n16; i += U * stride) {
+    uint4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = src[i + u * stride];
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
   }
-  for (; i < n16; i += stride) acc ^= src[i].x;
+  for (; i < n16; i += stride) {
+    const uint4 a = src[i];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  }
   if (acc == 0x9e3779b9u) sink[0] = acc;
 }
 
@@ -55,11 +62,19 @@ probe_mfma_kernel(int iters, float* __restrict__ sink) {
   if (s == -1.0f) sink[0] = s;      // sums of non-negative products: never
 }
 
-// grid: workgroups of 256 threads.  src (and dst) hold `bytes` bytes, a multiple of 16.
-extern "C" int atoma_probe_read(const void* src, size_t bytes, int grid, void* sink, hipStream_t stream) {
+// grid: workgroups of 256 threads.  src (and dst) hold `bytes` bytes, a multiple of 16.  in_flight: 4, 8 or 16
+// loads of 16 bytes a thread.
+extern "C" int atoma_probe_read(const void* src, size_t bytes, int grid, int in_flight, void* sink,
+                                hipStream_t stream) {
   if (grid <= 0 || bytes % 16 || ((uintptr_t)src & 15)) return ATOMA_ERR_SHAPE;
-  hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, (const uint4*)src, bytes / 16,
-                     (uint32_t*)sink);
+#define ATOMA_READ(U)                                                                                          \
+  hipLaunchKernelGGL(probe_read_kernel<U>, dim3(grid), dim3(256), 0, stream, (const uint4*)src, bytes / 16,   \
+                     (uint32_t*)sink)
+  if (in_flight == 4) ATOMA_READ(4);
+  else if (in_flight == 8) ATOMA_READ(8);
+  else if (in_flight == 16) ATOMA_READ(16);
+  else return ATOMA_ERR_SHAPE;
+#undef ATOMA_READ
   ATOMA_LAUNCH_CHECK();
   return 0;
 }

@@ -1,7 +1,8 @@
 """bfloat16 attention over the paged cache on the matrix cores: task lists on the host, kernels per head size.
 
-``try_attention`` runs ``attention_mfma.hip`` (compiled for the model's head size on first use) when the cache
-has 16-token pages; otherwise it returns False and the caller runs the general kernel.
+``try_attention`` runs ``attention_mfma.hip`` (compiled for the model's head size and the cache's page size on
+first use) when the cache's pages hold a multiple of 16 tokens; otherwise it returns False and the caller runs the
+general kernel.
 
 The step's entries are cut into tasks of 32 query rows (row = token x query head of one KV group) against a key
 range.  An entry with few tokens and many keys (a decoded token, a short portion late in a prompt) is split into
@@ -20,27 +21,39 @@ import torch
 from .library import load_hip_module
 from .ops import _check, _p, _stream
 
-PAGE = 16
+PAGE = 16            # the page size that the build check compiles every head size for; others on first use
 CHUNK = 256          # keys per partial task, at most; fewer when few requests are split (see chunk_for)
 MAX_SPLIT_TASKS = 1024
 SPLIT_MAX_TOKENS = 16  # entries with at most this many tokens may be split along the keys
 SPLIT_MIN_KEYS = 2 * CHUNK
 SPLIT_WAVES_MIN_KEYS = 128   # a task of at least this many keys is walked by two waves, every other block each
-_libs: Dict[int, ctypes.CDLL] = {}
+_libs: Dict[Tuple[int, int], ctypes.CDLL] = {}
 
 
-def module_name(hd: int) -> str:
-    return f"attention_hd{hd}"
+def page_ok(page_size: int) -> bool:
+    """Pages that the matrix-core kernel reads: any multiple of 16 tokens (the reference's kernel takes the same:
+    csrc/src/lib.rs:778-785)."""
+    return page_size >= 16 and page_size % 16 == 0
 
 
-def lib(hd: int, force_build: bool = False) -> ctypes.CDLL:
-    if hd not in _libs or force_build:
-        _libs[hd] = load_hip_module(module_name(hd), ("attention_mfma.hip",), (f"ATOMA_HD={hd}",),
-                                    force_build=force_build)
-        assert _libs[hd].atoma_attention_mfma_head_size() == hd
-        assert _libs[hd].atoma_attention_mfma_max_ksplit() == max_waves_for(hd)
-        assert _libs[hd].atoma_attention_mfma_max_row_tiles() == max_row_tiles_for(hd)
-    return _libs[hd]
+def module_name(hd: int, page: int = PAGE) -> str:
+    return f"attention_hd{hd}" if page == PAGE else f"attention_hd{hd}_page{page}"
+
+
+def module_defines(hd: int, page: int = PAGE) -> Tuple[str, ...]:
+    return (f"ATOMA_HD={hd}",) if page == PAGE else (f"ATOMA_HD={hd}", f"ATOMA_PAGE={page}")
+
+
+def lib(hd: int, force_build: bool = False, page: int = PAGE) -> ctypes.CDLL:
+    key = (hd, page)
+    if key not in _libs or force_build:
+        _libs[key] = load_hip_module(module_name(hd, page), ("attention_mfma.hip",), module_defines(hd, page),
+                                     force_build=force_build)
+        assert _libs[key].atoma_attention_mfma_head_size() == hd
+        assert _libs[key].atoma_attention_mfma_page_size() == page
+        assert _libs[key].atoma_attention_mfma_max_ksplit() == max_waves_for(hd)
+        assert _libs[key].atoma_attention_mfma_max_row_tiles() == max_row_tiles_for(hd)
+    return _libs[key]
 
 
 def max_waves_for(hd: int) -> int:
@@ -400,11 +413,12 @@ def _merge_counters(device: torch.device, needed: int) -> Optional[torch.Tensor]
 
 def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, hd) -> bool:
     """Run the fast kernels if they take this shape; False sends the caller to the general kernel."""
-    if cache.page_size != PAGE or hd % 16 or not 16 <= hd <= 256:
+    page = cache.page_size
+    if not page_ok(page) or hd % 16 or not 16 <= hd <= 256:
         return False
     if q.stride(0) % 8 or q.data_ptr() % 16 or out.stride(0) % 4:
         return False
-    if tuple(k_cache.shape[1:]) != (nkv, PAGE * hd) or tuple(v_cache.shape[1:]) != (nkv, PAGE * hd):
+    if tuple(k_cache.shape[1:]) != (nkv, page * hd) or tuple(v_cache.shape[1:]) != (nkv, page * hd):
         raise ValueError("cache tensors must be [pages, nkv, page_size * hd] tiles")
     group = nh // nkv
     plan = getattr(ctx, "plans", {}).get(plan_key(group, window, nkv, hd))
@@ -418,7 +432,7 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
             plan = (torch.from_numpy(arr).to(q.device), meta)
             ctx.scratch[key] = plan
     tasks, (n_main, n_comb, n_part, waves, row_tiles, merge) = plan
-    ksplit = min(waves, lib(hd).atoma_attention_mfma_max_ksplit())
+    ksplit = min(waves, lib(hd, page=page).atoma_attention_mfma_max_ksplit())
     part_o = part_lse = None
     if n_part:
         ws_key = ("attention_partials", nkv, hd)
@@ -430,7 +444,7 @@ def try_attention(q, k_cache, v_cache, out, ctx, cache, scale, window, nh, nkv, 
         part_o, part_lse = ws
     bt = cache.block_tables
     counters = _merge_counters(q.device, n_comb * nkv) if n_comb and merge else None
-    _check(lib(hd).atoma_attention_mfma(_p(q), q.stride(0), _p(k_cache), _p(v_cache), _p(out), out.stride(0),
+    _check(lib(hd, page=page).atoma_attention_mfma(_p(q), q.stride(0), _p(k_cache), _p(v_cache), _p(out), out.stride(0),
                                         _p(part_o), _p(part_lse), _p(tasks), n_main, n_comb, _p(bt), bt.shape[1],
                                         ctypes.c_float(scale), int(window), nh, nkv, ksplit, row_tiles, _p(counters),
                                         _stream()),

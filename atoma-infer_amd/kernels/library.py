@@ -54,6 +54,9 @@ _module_locks: Dict[str, threading.Lock] = {}
 # head sizes whose attention module the build check compiles ahead of time: every one the kernel takes (a few
 # seconds each); a model compiles only its own when it is first used and no built module is there
 STANDARD_HEAD_SIZES = tuple(range(16, 257, 16))
+# (head size, tokens a page) beyond pages of 16 tokens that the build check compiles too: the head sizes of the Llamas
+# with pages of 32 and 64 tokens, and what the tests run; any other pair is compiled when a cache first has it
+LARGER_PAGE_MODULES = tuple((hd, page) for hd in (32, 48, 64, 128) for page in (32, 64)) + ((64, 48), (80, 48))
 
 
 def _lock_for(name: str) -> threading.Lock:
@@ -210,7 +213,10 @@ def build_all(head_sizes: Sequence[int] = STANDARD_HEAD_SIZES) -> List[str]:
     load_host_library(force_build=True)
     built.append("host")
     jobs = [(name, None, ()) for name in HIP_MODULES]
-    jobs += [(attention_bf16.module_name(hd), ("attention_mfma.hip",), (f"ATOMA_HD={hd}",)) for hd in head_sizes]
+    jobs += [(attention_bf16.module_name(hd), ("attention_mfma.hip",), attention_bf16.module_defines(hd))
+             for hd in head_sizes]
+    jobs += [(attention_bf16.module_name(hd, page), ("attention_mfma.hip",), attention_bf16.module_defines(hd, page))
+             for hd, page in LARGER_PAGE_MODULES]
     with ThreadPoolExecutor(min(8, len(jobs))) as pool:
         futs = [pool.submit(load_hip_module, n, src, d, force_build=True) for n, src, d in jobs]
         for (n, _, _), f in zip(jobs, futs):

@@ -98,12 +98,12 @@ class PagedAttention(Mixer):
                           f"token and head), many times slower than the matrix-core kernel, which takes head sizes "
                           f"that are multiples of 16", stacklevel=2)
             return None
-        if cache_dtype is torch.bfloat16 and page_size != attention_bf16.PAGE:
+        if cache_dtype is torch.bfloat16 and not attention_bf16.page_ok(page_size):
             import warnings
             warnings.warn(f"bfloat16 attention with pages of {page_size} tokens runs the general kernel (one wave per "
-                          f"token and head), many times slower than the matrix-core kernel, which needs pages of "
-                          f"{attention_bf16.PAGE} tokens ([cache] block_size = {attention_bf16.PAGE})", stacklevel=2)
-        if cache_dtype is not torch.bfloat16 or page_size != attention_bf16.PAGE:
+                          f"token and head), many times slower than the matrix-core kernel, which needs pages of a "
+                          f"multiple of 16 tokens ([cache] block_size = 16, 32, 64, ...)", stacklevel=2)
+        if cache_dtype is not torch.bfloat16 or not attention_bf16.page_ok(page_size):
             return None
         group, window, nkv = self.nh // self.nkv, self.window or 0, self.nkv
         cus = torch.cuda.get_device_properties(self.w_qkv.device).multi_processor_count

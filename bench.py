@@ -288,6 +288,7 @@ def main() -> int:
     if peaks:
         # what the probes reached on this GPU, beside the published peaks that the fractions above are of
         roofline["measured_peak"] = peaks["hbm_read_gbs"]
+        roofline["measured_how"] = peaks.get("hbm_read_how", "")
         roofline["measured_copy"] = peaks["hbm_copy_gbs"]
         roofline["frac_of_measured"] = round(achieved / peaks["hbm_read_gbs"], 4)
         prefill["measured_peak_tflops"] = peaks["mfma_bf16_tflops"]
@@ -297,8 +298,11 @@ def main() -> int:
     if not args.no_points:
         for b, st in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
             log(f"decode at batch {b} ...")
-            d, _ = decode_run(model, b, args.prompt_len, st, min(args.warmup, 4), args.context, sampling=sampling)
+            d, ctx_b = decode_run(model, b, args.prompt_len, st, min(args.warmup, 4), args.context, sampling=sampling)
             points[f"decode_b{b}"] = round(b * st / d, 1)
+            # the same roofline fraction as the headline's, with this batch's own mean context
+            bytes_b = model.weight_bytes() + kv_bytes_per_token * ctx_b * b
+            points[f"decode_b{b}_frac"] = round(bytes_b / (d / st) / 1e9 / HBM_PEAK_GBS, 4)
 
     line = {
         "metric": f"decode tok/s at batch {args.batch} ({name} sizes, {args.prompt_len}-token prompts); "

@@ -179,7 +179,8 @@ def test_plan_cache_groups_layers_by_their_needs():
         spec.__post_init__()
 
 
-@pytest.mark.parametrize("page,head", [(16, 64), (16, 48), (16, 16), (4, 16), (16, 256), (16, 80), (8, 32), (1, 32)])
+@pytest.mark.parametrize("page,head", [(16, 64), (16, 48), (16, 16), (4, 16), (16, 256), (16, 80), (8, 32), (1, 32),
+                                       (32, 64), (64, 128), (48, 80), (24, 32)])
 def test_tile_layout_is_a_permutation_and_serves_the_mfma_lanes(page, head):
     import torch
     from atoma_infer_amd.cache.layout import (key_index, pack_keys, pack_values, unpack_keys, unpack_values,
@@ -190,15 +191,20 @@ def test_tile_layout_is_a_permutation_and_serves_the_mfma_lanes(page, head):
     k, v = torch.randn(3, page, head), torch.randn(3, head, page)
     assert torch.equal(unpack_keys(pack_keys(k), page, head), k)
     assert torch.equal(unpack_values(pack_values(v), page, head), v)
-    # a lane's 8 columns of a key are contiguous; with 16-token pages a lane's 8 key slots of a value column too
+    # a lane's 8 columns of a key are contiguous; with pages of 16, 32, 48, ... tokens a lane's 8 key slots of a value
+    # column too, in every run of 16 tokens, and a run is laid out as a page of 16 tokens
     for t in range(page):
         for d0 in range(0, head, 8):
             assert ki[t, d0:d0 + 8].tolist() == list(range(int(ki[t, d0]), int(ki[t, d0]) + 8))
-    if page == 16:
-        for d in range(head):
-            for hg in (0, 1):
-                slots = [int(vi[d, hg * 4 + i]) for i in range(4)] + [int(vi[d, 8 + hg * 4 + i]) for i in range(4)]
-                assert slots == list(range(slots[0], slots[0] + 8)) and slots[0] % 8 == 0
+    if page % 16 == 0:
+        v16 = value_index(16, head)
+        for run in range(page // 16):
+            assert torch.equal(vi[:, run * 16: run * 16 + 16], v16 + run * 16 * head)
+            for d in range(head):
+                for hg in (0, 1):
+                    slots = [int(vi[d, run * 16 + hg * 4 + i]) for i in range(4)] + \
+                            [int(vi[d, run * 16 + 8 + hg * 4 + i]) for i in range(4)]
+                    assert slots == list(range(slots[0], slots[0] + 8)) and slots[0] % 8 == 0
 
 
 def test_admission_with_a_window_counts_what_everyone_will_need():

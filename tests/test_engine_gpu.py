@@ -226,6 +226,46 @@ def test_a_place_wanted_twice_beside_an_entry_that_wants_nothing(model_dirs, dty
     check_against_plain(model_dirs[name], {"b": b}, {("b", 22): logits[0]}, dtype)
 
 
+@pytest.mark.parametrize("page", [32, 64])
+@pytest.mark.parametrize("name", ["B", "D", "E"])
+def test_larger_pages_run_on_the_matrix_cores(model_dirs, name, page, monkeypatch):
+    """bfloat16 with pages of 32 and 64 tokens (the reference takes every multiple of 16: csrc/src/lib.rs:778-785):
+    portions of changing size, the last tokens one by one, then requests mixed in a pool so small that pages are used
+    again; the general attention kernel must not be called."""
+    from atoma_infer_amd.kernels import ops
+
+    def refuse(*a, **k):
+        raise AssertionError("the general attention kernel ran")
+
+    monkeypatch.setattr(ops, "paged_attention_generic", refuse)
+    force_chunked_decode(monkeypatch)
+    vocab = TINY[name]["vocab_size"]
+    lens = {"B": [120, 1, 77, 90, 45, 130], "D": [700, 48, 97, 530, 70, 33], "E": [300, 48, 97, 610, 70, 33]}[name]
+    requests = {f"r{i}": random_tokens(n, vocab, 500 + i) for i, n in enumerate(lens)}
+    need = sum(sorted(-(-n // page) for n in lens)[-3:])
+    runner = make_runner(model_dirs[name], "bfloat16", page, need, slots=3)
+    rng = random.Random(page + len(name))
+    waiting, live, done, steps = list(requests), [], {r: 0 for r in requests}, []
+    while waiting or live:
+        while waiting and len(live) < 3:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in live:
+            left = len(requests[r]) - done[r]
+            n = 1 if left <= 12 else min(rng.choice([2, 5, 16, 31, 33, 70]), left - 12)
+            entries.append((r, n))
+            done[r] += n
+            if done[r] == len(requests[r]):
+                end.append(r)
+        rng.shuffle(entries)
+        steps.append((entries, end))
+        live = [r for r in live if r not in end]
+    got = run_schedule(runner, requests, steps)
+    assert len(got) == sum(lens)
+    check_against_plain(model_dirs[name], requests, got, "bfloat16")
+    assert runner.manager.num_free_pages(0) == need
+
+
 def test_pages_the_matrix_core_attention_refuses_are_announced(model_dirs):
     """bfloat16 with pages of 4 tokens is right (the tests above run it) but takes the general attention kernel:
     building the runner says so once."""

@@ -260,6 +260,15 @@ ATTN_CASES = [
     # decoded tokens with so many keys that their chunks are 512 keys long
     (8, 8, 64, 16, 0, [(20000, 1), (16500, 1), (3, 2)]),
     (4, 4, 128, 16, 9000, [(17000, 1), (30000, 1), (16385, 1)]),
+    # pages of 32, 64 and 48 tokens (a block of 32 keys is then one page, half a page, or lies across two): prompts,
+    # portions, decoded tokens whose keys are cut into chunks, a window
+    (8, 2, 64, 32, 0, [(0, 130), (600, 1), (1030, 3), (511, 1), (512, 1)]),
+    (8, 2, 64, 64, 0, [(0, 1100), (900, 150), (2047, 1)]),
+    (6, 2, 48, 64, 0, [(0, 33), (100, 20), (77, 1)]),
+    (4, 4, 80, 48, 0, [(10, 50), (0, 97), (200, 1)]),
+    (16, 2, 128, 32, 0, [(0, 64), (700, 1), (4000, 70)]),
+    (4, 2, 32, 64, 600, [(0, 100), (900, 1), (640, 5)]),
+    (8, 2, 64, 48, 100, [(0, 300), (1500, 1), (95, 2)]),
 ]
 
 
@@ -279,6 +288,7 @@ def test_paged_attention(nh, nkv, hd, page, window, entries, kind):
     scale = 1.0 / math.sqrt(hd)
     if kind == "mfma":
         assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, cache, scale, window, nh, nkv, hd)
+        assert attention_bf16.lib(hd, page=page).atoma_attention_mfma_page_size() == page
     else:
         ops.paged_attention_generic(qkv, kc, vc, out, bt, ctx.token_seq, ctx.positions, scale, window, page, nh,
                                     nkv, hd)
@@ -397,6 +407,7 @@ def test_attention_when_one_key_stands_out(window, entries, key, kind):
     scale = 1.0 / math.sqrt(hd)
     if kind == "mfma":
         assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, cache, scale, window, nh, nkv, hd)
+        assert attention_bf16.lib(hd, page=page).atoma_attention_mfma_page_size() == page
     else:
         ops.paged_attention_generic(qkv, kc, vc, out, bt, ctx.token_seq, ctx.positions, scale, window, page, nh,
                                     nkv, hd)
