@@ -31,6 +31,48 @@ struct RopeArgs {
   int page_size, nh, nkv, hd;
 };
 
+// Outputs n0 .. n0 + 3 of row `row` of the fused q, k, v projection (float32 sums x0 .. x3), with the rows of every q
+// and k head ordered so that the members of rotary pair i = (column i, column i + hd/2) are outputs 2i and 2i + 1 of
+// the head: the four are two whole pairs, i and i + 1.  They are rotated here and go to their own columns: q to
+// q_out [M, nh * hd], k into the row's slot of the paged cache (the order inside a tile: cache_layout.h); v heads are
+// copied into theirs.  The same arithmetic as the rotary kernel (csrc/kernels/rotary.h:116-131 of the reference), on
+// the float32 sums before they are rounded.
+__device__ __forceinline__ void rope_store4(float x0, float x1, float x2, float x3, int row, int n0, const RopeArgs& ra,
+                                            uint16_t* __restrict__ q_out, int ldq) {
+  const int hd = ra.hd, half = hd >> 1;
+  const int head = n0 / hd, d0 = n0 % hd;
+  if (head >= ra.nh + ra.nkv) {
+    const int slot = ra.slot_mapping[row];
+    if (slot < 0) return;
+    const int page = slot / ra.page_size, off = slot % ra.page_size;
+    uint16_t* tile = ra.vcache + ((size_t)page * ra.nkv + (head - ra.nh - ra.nkv)) * ra.page_size * hd;
+    tile[value_offset(d0, off, hd, ra.page_size)] = f32_to_bf16_bits(x0);
+    tile[value_offset(d0 + 1, off, hd, ra.page_size)] = f32_to_bf16_bits(x1);
+    tile[value_offset(d0 + 2, off, hd, ra.page_size)] = f32_to_bf16_bits(x2);
+    tile[value_offset(d0 + 3, off, hd, ra.page_size)] = f32_to_bf16_bits(x3);
+    return;
+  }
+  const int i = d0 >> 1;                       // even: columns i, i + 1 and their partners lie together
+  const size_t at = (size_t)ra.positions[row] * half + i;
+  const float c0 = ra.cos_t[at], s0 = ra.sin_t[at], c1 = ra.cos_t[at + 1], s1 = ra.sin_t[at + 1];
+  const uint32_t lo = (uint32_t)f32_to_bf16_bits(x0 * c0 - x1 * s0) |
+                      ((uint32_t)f32_to_bf16_bits(x2 * c1 - x3 * s1) << 16);      // columns i, i + 1
+  const uint32_t hi = (uint32_t)f32_to_bf16_bits(x1 * c0 + x0 * s0) |
+                      ((uint32_t)f32_to_bf16_bits(x3 * c1 + x2 * s1) << 16);      // i + half, i + half + 1
+  if (head < ra.nh) {
+    uint16_t* q = q_out + (size_t)row * ldq + (size_t)head * hd;
+    *reinterpret_cast<uint32_t*>(q + i) = lo;
+    *reinterpret_cast<uint32_t*>(q + i + half) = hi;
+    return;
+  }
+  const int slot = ra.slot_mapping[row];
+  if (slot < 0) return;
+  const int page = slot / ra.page_size, off = slot % ra.page_size;
+  uint16_t* tile = ra.kcache + ((size_t)page * ra.nkv + (head - ra.nh)) * ra.page_size * hd;
+  *reinterpret_cast<uint32_t*>(tile + key_offset(off, i, ra.page_size)) = lo;
+  *reinterpret_cast<uint32_t*>(tile + key_offset(off, i + half, ra.page_size)) = hi;
+}
+
 // A norm that is finished by its neighbours (at most 16 rows of activations).
 //   In: the rows of A are residual rows times the norm's weight, not yet divided by their root mean square; the
 //   sums of squares of the residual rows arrive as ss_in [parts_in][16] (a part per producing wave), and every sum
@@ -316,54 +358,18 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   }
 
   if constexpr (ROPE) {
-    // W is the fused q, k, v projection with the rows of every q and k head ordered so that the members of
-    // rotary pair i = (column i, column i + hd/2) are outputs 2i and 2i + 1 of the head: a lane's four outputs are
-    // two whole pairs, i and i + 1.  They are rotated here and go to their own columns: q to C [M, nh * hd], k
-    // into the row's slot of the paged cache (the order inside a tile: cache_layout.h); v heads are copied into
-    // theirs.  The same arithmetic as the rotary kernel (csrc/kernels/rotary.h:116-131 of the reference), on the
-    // float32 sums before they are rounded.
+    // the fused q, k, v projection: rotate q and k, store k and v in the cache (rope_store4)
     static_assert(!ROPE || sizeof(TC) == 2, "the rotary epilogue writes bfloat16");
-    const int hd = ra.hd, half = hd >> 1;
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
       const int n0 = n_base + r * 16 + kg * 4;
       if (n0 + 3 >= N) continue;
-      const int head = n0 / hd, d0 = n0 % hd;
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         const int row = m * 16 + r16;
         if (row >= M) continue;
-        const float x0 = acc[r][m][0], x1 = acc[r][m][1], x2 = acc[r][m][2], x3 = acc[r][m][3];
-        if (head >= ra.nh + ra.nkv) {
-          const int slot = ra.slot_mapping[row];
-          if (slot < 0) continue;
-          const int page = slot / ra.page_size, off = slot % ra.page_size;
-          uint16_t* tile = ra.vcache + ((size_t)page * ra.nkv + (head - ra.nh - ra.nkv)) * ra.page_size * hd;
-          tile[value_offset(d0, off, hd, ra.page_size)] = f32_to_bf16_bits(x0);
-          tile[value_offset(d0 + 1, off, hd, ra.page_size)] = f32_to_bf16_bits(x1);
-          tile[value_offset(d0 + 2, off, hd, ra.page_size)] = f32_to_bf16_bits(x2);
-          tile[value_offset(d0 + 3, off, hd, ra.page_size)] = f32_to_bf16_bits(x3);
-          continue;
-        }
-        const int i = d0 >> 1;                       // even: columns i, i + 1 and their partners lie together
-        const size_t at = (size_t)ra.positions[row] * half + i;
-        const float c0 = ra.cos_t[at], s0 = ra.sin_t[at], c1 = ra.cos_t[at + 1], s1 = ra.sin_t[at + 1];
-        const uint32_t lo = (uint32_t)f32_to_bf16_bits(x0 * c0 - x1 * s0) |
-                            ((uint32_t)f32_to_bf16_bits(x2 * c1 - x3 * s1) << 16);      // columns i, i + 1
-        const uint32_t hi = (uint32_t)f32_to_bf16_bits(x1 * c0 + x0 * s0) |
-                            ((uint32_t)f32_to_bf16_bits(x3 * c1 + x2 * s1) << 16);      // i + half, i + half + 1
-        if (head < ra.nh) {
-          uint16_t* q = reinterpret_cast<uint16_t*>(c) + (size_t)row * ldc + (size_t)head * hd;
-          *reinterpret_cast<uint32_t*>(q + i) = lo;
-          *reinterpret_cast<uint32_t*>(q + i + half) = hi;
-          continue;
-        }
-        const int slot = ra.slot_mapping[row];
-        if (slot < 0) continue;
-        const int page = slot / ra.page_size, off = slot % ra.page_size;
-        uint16_t* tile = ra.kcache + ((size_t)page * ra.nkv + (head - ra.nh)) * ra.page_size * hd;
-        *reinterpret_cast<uint32_t*>(tile + key_offset(off, i, ra.page_size)) = lo;
-        *reinterpret_cast<uint32_t*>(tile + key_offset(off, i + half, ra.page_size)) = hi;
+        rope_store4(acc[r][m][0], acc[r][m][1], acc[r][m][2], acc[r][m][3], row, n0, ra,
+                    reinterpret_cast<uint16_t*>(c), ldc);
       }
     }
     return;
@@ -622,4 +628,42 @@ extern "C" int atoma_gemm_bf16_skinny_rope(const void* a, const void* w, void* c
     case 3: return launch_rope_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, fa, stream);
     default: return launch_rope_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, fa, stream);
   }
+}
+
+// The fused q, k, v projection of 17 to 64 rows as float32 planes of a K-split product (which about 256 workgroups
+// share, each fetching an eighth of the activations, where the product with the rotary epilogue has 192 that each
+// fetch all of them), summed here in the order of the planes, rotated and stored: a thread takes four outputs of a row.
+__global__ void __launch_bounds__(256)
+rope_from_planes_kernel(const float* __restrict__ planes, int slices, size_t plane, int M, int N, uint16_t* __restrict__ q_out,
+                        int ldq, RopeArgs ra) {
+  const int row = blockIdx.x;
+  const int n0 = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (n0 + 3 >= N) return;
+  const float* p = planes + (size_t)row * N + n0;
+  f32x4 sum = *reinterpret_cast<const f32x4*>(p);
+  for (int s = 1; s < slices; ++s) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(p + (size_t)s * plane);
+    sum[0] += v[0], sum[1] += v[1], sum[2] += v[2], sum[3] += v[3];
+  }
+  rope_store4(sum[0], sum[1], sum[2], sum[3], row, n0, ra, q_out, ldq);
+}
+
+// planes [slices][M][N] float32 with N = (nh + 2 nkv) hd, the columns of q and k heads in pair order; q_out
+// [M, ldq >= nh hd] bfloat16.  hd % 4 == 0.
+extern "C" int atoma_rope_from_planes(const float* planes, int slices, int M, void* q_out, int ldq,
+                                      const int32_t* positions, const float* cos_t, const float* sin_t, void* kcache,
+                                      void* vcache, const int32_t* slot_mapping, int page_size, int nh, int nkv, int hd,
+                                      hipStream_t stream) {
+  if (M <= 0) return 0;
+  const int N = (nh + 2 * nkv) * hd;
+  if (slices <= 0 || M > 65535 || ldq < nh * hd || (ldq & 1) || ((uintptr_t)planes & 15) || ((uintptr_t)q_out & 3) ||
+      (hd & 3) || nh <= 0 || nkv <= 0 || page_size <= 0 || !positions || !cos_t || !sin_t || !kcache || !vcache ||
+      !slot_mapping || ((uintptr_t)kcache & 3))
+    return ATOMA_ERR_SHAPE;
+  const RopeArgs ra{positions, cos_t, sin_t, (uint16_t*)kcache, (uint16_t*)vcache, slot_mapping, page_size, nh, nkv, hd};
+  dim3 grid(M, (N / 4 + 255) / 256);
+  hipLaunchKernelGGL(rope_from_planes_kernel, grid, dim3(256), 0, stream, planes, slices, (size_t)M * N, M, N,
+                     (uint16_t*)q_out, ldq, ra);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
 }

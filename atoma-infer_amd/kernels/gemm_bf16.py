@@ -264,6 +264,10 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
 
 
 ROPE_MAX_M = SKINNY_MAX_M
+# Rows beyond which the q, k, v product is split along K into planes and a second kernel sums, rotates and stores
+# (measured on MI355X over the 16 layers of a Llama 1B decode step: 1 to 2 % slower steps at 17 to 32 rows, 1 % quicker
+# at 48, 2 % at 64: 16.3 us become 8 + 6)
+ROPE_PLANES_MIN_M = 40
 
 
 def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
@@ -285,12 +289,23 @@ def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, c
             or cos.dtype is not torch.float32 or cos.shape[1] != hd // 2 or not cos.is_contiguous()
             or not sin.is_contiguous() or not kcache.is_contiguous() or not vcache.is_contiguous()):
         return None
+    out = torch.empty((m, nh * hd), dtype=torch.bfloat16, device=x.device)
+    if m > ROPE_PLANES_MIN_M and begun[1] == 0:
+        # more rows than one tile: K split over the grid into float32 planes (every workgroup then fetches a slice of
+        # the activations, not all of them), summed, rotated and stored by a second kernel
+        rt, wk, slices = _plan(m, n, k, True)
+        if slices > 1:
+            planes = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+            skinny(x, w, planes, slices, rt, wk)
+            _check(lib().atoma_rope_from_planes(_p(planes), slices, m, _p(out), nh * hd, _p(positions), _p(cos), _p(sin),
+                                                _p(kcache), _p(vcache), _p(slot_mapping), int(page_size), nh, nkv, hd,
+                                                _stream()), "rope_from_planes")
+            return out
     rt, wk, _ = _plan(m, n, k, False)
     if rt > 2:
         rt = 2
     if 8 < m <= 16 and rt == 1 and wk == 4 and n >= 5120:
         rt = 2          # (9 to 16 rows at Llama 3B's and 8B's sizes: 14.1 and 17.1 us against 15.3 and 18.9)
-    out = torch.empty((m, nh * hd), dtype=torch.bfloat16, device=x.device)
     _check(lib().atoma_gemm_bf16_skinny_rope(_p(x), _p(w), _p(out), m, k, x.stride(0) if m > 1 else k, w.stride(0),
                                              nh * hd, rt, wk, _p(positions), _p(cos), _p(sin), _p(kcache), _p(vcache),
                                              _p(slot_mapping), int(page_size), nh, nkv, hd, *begun, _stream()),

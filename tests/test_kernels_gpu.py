@@ -552,10 +552,18 @@ def test_gemm_with_swiglu_epilogue(m, inter, k):
 @pytest.mark.parametrize("m", [1, 8, 16, 23, 40, 64])
 @pytest.mark.parametrize("nh,nkv,hd,k", [(8, 2, 64, 256), (3, 1, 16, 64), (32, 8, 64, 2048), (5, 5, 48, 96),
                                          (24, 8, 128, 256), (32, 8, 128, 512), (3, 1, 128, 384)])
-def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k):
-    """The q, k, v projection that rotates and stores in its epilogue against product, rotation and store done
-    apart."""
+@pytest.mark.parametrize("planes", [False, True])
+def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k, planes, monkeypatch):
+    """The q, k, v projection that rotates and stores in its epilogue (or, with ``planes`` and more than 16 rows, as
+    a K-split product whose planes a second kernel sums, rotates and stores, as the planner has it from 41 rows on)
+    against product, rotation and store done apart."""
     from atoma_infer_amd.kernels import gemm_bf16, ops
+    if planes:
+        if m <= 16:
+            pytest.skip("one tile of rows: the epilogue always")
+        monkeypatch.setattr(gemm_bf16, "ROPE_PLANES_MIN_M", 16)
+    else:
+        monkeypatch.setattr(gemm_bf16, "ROPE_PLANES_MIN_M", 64)
     from atoma_infer_amd.cache.layout import pack_keys, pack_values
     page, pages = 16, 6
     n = (nh + 2 * nkv) * hd
