@@ -196,12 +196,12 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
 
 // The same for rows of at most 4096 columns, a multiple of 4, with 16-byte aligned rows: every thread keeps its
 // values in registers between the two passes and all loads of a pass are issued together.
-template <typename TD, typename TW, typename TO>
+// MAXJ: pieces of four columns a thread (1, 2 or 4: rows of up to 1024, 2048, 4096 columns).
+template <typename TD, typename TW, typename TO, int MAXJ>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(float* __restrict__ resid, const TD* __restrict__ delta, const TW* __restrict__ w,
                        TO* __restrict__ out, const int32_t* __restrict__ rows, int width, float eps, int planes,
                        size_t plane_stride) {
-  constexpr int MAXJ = 4;
   __shared__ float scratch[4];
   const int r = blockIdx.x;
   const size_t src = (size_t)(rows ? rows[r] : r) * width, dst = (size_t)r * width;
@@ -214,19 +214,31 @@ add_rmsnorm_vec_kernel(float* __restrict__ resid, const TD* __restrict__ delta, 
     if (c < n4) v[j] = load4(resid + src + 4 * c);
   }
   if (delta) {
-    for (int p = 0; p < planes; ++p) {
-      f4 d[MAXJ];
+    // the planes of a K-split product: the loads of up to eight planes are issued together (each is a trip to memory,
+    // and a plane at a time would make as many trips as there are planes); they are added in the order of their index
+    constexpr int PB = MAXJ <= 2 ? 8 : 4;
+    for (int p0 = 0; p0 < planes; p0 += PB) {
+      f4 d[PB][MAXJ];
 #pragma unroll
-      for (int j = 0; j < MAXJ; ++j) {
-        const int c = threadIdx.x + j * 256;
-        if (c < n4) d[j] = load4(delta + p * plane_stride + src + 4 * c);
+      for (int q = 0; q < PB; ++q) {
+        const int p = p0 + q < planes ? p0 + q : planes - 1;
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+          const int c = threadIdx.x + j * 256;
+          if (c < n4) d[q][j] = load4(delta + p * plane_stride + src + 4 * c);
+        }
       }
 #pragma unroll
-      for (int j = 0; j < MAXJ; ++j) {
-        const int c = threadIdx.x + j * 256;
-        if (c < n4)
+      for (int q = 0; q < PB; ++q) {
+        if (p0 + q < planes) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) v[j].v[i] += d[j].v[i];
+          for (int j = 0; j < MAXJ; ++j) {
+            const int c = threadIdx.x + j * 256;
+            if (c < n4)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) v[j].v[i] += d[q][j].v[i];
+          }
+        }
       }
     }
   }
@@ -261,23 +273,34 @@ static int add_rmsnorm_out(float* resid, const TD* delta, const TW* w, void* out
   dim3 grid(n_rows), block(256);
   const bool vec = width % 4 == 0 && width <= 4096 && ((uintptr_t)resid & 15) == 0 && ((uintptr_t)delta & 15) == 0 &&
                    ((uintptr_t)w & 15) == 0 && ((uintptr_t)out & 15) == 0 && plane_stride % 4 == 0;
+#define ATOMA_NORM_VEC(TO_)                                                                                         \
+  do {                                                                                                             \
+    if (width <= 1024)                                                                                             \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TO_, 1>), grid, block, 0, stream, resid, delta, w,        \
+                         (TO_*)out, rows, width, eps, planes, plane_stride);                                       \
+    else if (width <= 2048)                                                                                        \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TO_, 2>), grid, block, 0, stream, resid, delta, w,        \
+                         (TO_*)out, rows, width, eps, planes, plane_stride);                                       \
+    else                                                                                                           \
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TO_, 4>), grid, block, 0, stream, resid, delta, w,        \
+                         (TO_*)out, rows, width, eps, planes, plane_stride);                                       \
+  } while (0)
   if (out_dtype == kF32) {
     if (vec)
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, float>), grid, block, 0, stream, resid, delta, w,
-                         (float*)out, rows, width, eps, planes, plane_stride);
+      ATOMA_NORM_VEC(float);
     else
       hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, float>), grid, block, 0, stream, resid, delta, w, (float*)out,
                          rows, width, eps, planes, plane_stride);
   } else if (out_dtype == kBF16) {
     if (vec)
-      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, bf16_t>), grid, block, 0, stream, resid, delta, w,
-                         (bf16_t*)out, rows, width, eps, planes, plane_stride);
+      ATOMA_NORM_VEC(bf16_t);
     else
       hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, bf16_t>), grid, block, 0, stream, resid, delta, w,
                          (bf16_t*)out, rows, width, eps, planes, plane_stride);
   } else {
     return ATOMA_ERR_DTYPE;
   }
+#undef ATOMA_NORM_VEC
   ATOMA_LAUNCH_CHECK();
   return 0;
 }

@@ -633,6 +633,7 @@ extern "C" int atoma_gemm_bf16_skinny_rope(const void* a, const void* w, void* c
 // The fused q, k, v projection of 17 to 64 rows as float32 planes of a K-split product (which about 256 workgroups
 // share, each fetching an eighth of the activations, where the product with the rotary epilogue has 192 that each
 // fetch all of them), summed here in the order of the planes, rotated and stored: a thread takes four outputs of a row.
+constexpr int kMaxPlanes = 8;
 __global__ void __launch_bounds__(256)
 rope_from_planes_kernel(const float* __restrict__ planes, int slices, size_t plane, int M, int N, uint16_t* __restrict__ q_out,
                         int ldq, RopeArgs ra) {
@@ -640,11 +641,14 @@ rope_from_planes_kernel(const float* __restrict__ planes, int slices, size_t pla
   const int n0 = (blockIdx.y * 256 + threadIdx.x) * 4;
   if (n0 + 3 >= N) return;
   const float* p = planes + (size_t)row * N + n0;
-  f32x4 sum = *reinterpret_cast<const f32x4*>(p);
-  for (int s = 1; s < slices; ++s) {
-    const f32x4 v = *reinterpret_cast<const f32x4*>(p + (size_t)s * plane);
-    sum[0] += v[0], sum[1] += v[1], sum[2] += v[2], sum[3] += v[3];
-  }
+  // (all planes are asked for at once: each load is a trip to memory)
+  f32x4 v[kMaxPlanes];
+#pragma unroll
+  for (int s = 0; s < kMaxPlanes; ++s) v[s] = *reinterpret_cast<const f32x4*>(p + (size_t)(s < slices ? s : 0) * plane);
+  f32x4 sum = v[0];
+#pragma unroll
+  for (int s = 1; s < kMaxPlanes; ++s)
+    if (s < slices) sum[0] += v[s][0], sum[1] += v[s][1], sum[2] += v[s][2], sum[3] += v[s][3];
   rope_store4(sum[0], sum[1], sum[2], sum[3], row, n0, ra, q_out, ldq);
 }
 
@@ -656,7 +660,7 @@ extern "C" int atoma_rope_from_planes(const float* planes, int slices, int M, vo
                                       hipStream_t stream) {
   if (M <= 0) return 0;
   const int N = (nh + 2 * nkv) * hd;
-  if (slices <= 0 || M > 65535 || ldq < nh * hd || (ldq & 1) || ((uintptr_t)planes & 15) || ((uintptr_t)q_out & 3) ||
+  if (slices <= 0 || slices > kMaxPlanes || M > 65535 || ldq < nh * hd || (ldq & 1) || ((uintptr_t)planes & 15) || ((uintptr_t)q_out & 3) ||
       (hd & 3) || nh <= 0 || nkv <= 0 || page_size <= 0 || !positions || !cos_t || !sin_t || !kcache || !vcache ||
       !slot_mapping || ((uintptr_t)kcache & 3))
     return ATOMA_ERR_SHAPE;

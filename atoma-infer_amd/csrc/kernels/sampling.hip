@@ -86,13 +86,26 @@ template <typename F> __device__ __forceinline__ void sweep(const float* __restr
   if ((((uintptr_t)x) & 15) == 0) {
     const float4* x4 = reinterpret_cast<const float4*>(x);
     const int n4 = n >> 2;
-#pragma unroll 4
-    for (int i = tid; i < n4; i += kSampThreads) {
-      const float4 v = x4[i];
-      f(v.x, 4 * i);
-      f(v.y, 4 * i + 1);
-      f(v.z, 4 * i + 2);
-      f(v.w, 4 * i + 3);
+    // eight loads a thread are issued together: every batch is a trip to memory, and a row of a large vocabulary
+    // should take few of them
+    constexpr int U = 8;
+    for (int i0 = tid; i0 < n4; i0 += U * kSampThreads) {
+      float4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + u * kSampThreads;
+        v[u] = x4[i < n4 ? i : n4 - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + u * kSampThreads;
+        if (i < n4) {
+          f(v[u].x, 4 * i);
+          f(v[u].y, 4 * i + 1);
+          f(v[u].z, 4 * i + 2);
+          f(v[u].w, 4 * i + 3);
+        }
+      }
     }
     for (int i = (n4 << 2) + tid; i < n; i += kSampThreads) f(x[i], i);
   } else {
