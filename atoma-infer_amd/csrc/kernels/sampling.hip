@@ -1,5 +1,5 @@
-// Sampling from float32 logits, one block of 1024 threads per row (two walks over the row without a cut, five or
-// six with top-k or top-p):
+// Sampling from float32 logits, one block of 1024 threads per row that draws (two walks over the row without a cut,
+// five or six with top-k or top-p), up to eight per greedy row:
 //   greedy (temperature <= 0): argmax, lowest index on ties;
 //   else weights w_i = exp((l_i - max) / T), optionally cut to the k largest and then to the smallest set of
 //   largest weights whose mass reaches top_p of the whole, ties towards the lower index; the token is the first
@@ -139,6 +139,22 @@ __device__ void select_bin(const T* hist, T target, int& sel, T& rest, T* wave_s
   __syncthreads();
 }
 
+// What the blocks of a greedy row leave for the one that finishes last (see the kernel): a row's bests and how many
+// have arrived.  Arrays of the code object, zero when it is loaded and left at zero by every launch; all launches on
+// a device share them, so two that overlap in time (two streams, two threads) race, as they would on one workspace.
+constexpr int kMaxSplits = 8;
+constexpr int kSplitRows = 1024;        // launches of more rows give every row one block
+static __device__ float split_val[kSplitRows * kMaxSplits];
+static __device__ int split_idx[kSplitRows * kMaxSplits];
+static __device__ int split_count[kSplitRows];
+
+// blocks a row: enough that a few rows of a large vocabulary keep many CUs reading
+static int sample_splits(int n_rows, int vocab) {
+  if (n_rows > kSplitRows || vocab < 16384) return 1;
+  int s = 256 / n_rows;
+  return s < 1 ? 1 : s > kMaxSplits ? kMaxSplits : s;
+}
+
 __global__ void __launch_bounds__(kSampThreads)
 sample_kernel(const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ temperature,
               const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
@@ -158,12 +174,50 @@ sample_kernel(const float* __restrict__ logits, int ld, int vocab, const float* 
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* lr = logits + (size_t)row * ld;
   float* w = weights + (size_t)row * vocab;
+  const float temp = temperature[row];
+
+  // A greedy row is shared by the gridDim.y blocks of its row: one block reads a large vocabulary no faster than one
+  // CU can load (a row of 128k logits: 10 us).  Each takes a stretch of the row and leaves its best; the block that
+  // finishes last picks among them (stores and loads that go through to memory, a device-wide counter that it leaves
+  // at zero: no fence that would flush a cache).  Rows that draw keep one block: its walks share what they find.
+  const int parts = gridDim.y, part = blockIdx.y;
+  if (parts > 1) {
+    if (temp > 0.f) {
+      if (part > 0) return;
+    } else {
+      const int len = ((vocab + parts * 4 - 1) / (parts * 4)) * 4;
+      const int lo = part * len, hi = lo + len < vocab ? lo + len : vocab;
+      ArgMax a = {-INFINITY, 0x7fffffff};
+      if (lo < hi) sweep(lr + lo, hi - lo, [&](float v, int i) { a = better(a, ArgMax{v, i + lo}); });
+      a = block_argmax(a, am);
+      if (tid == 0) {
+        __hip_atomic_store(&split_val[row * kMaxSplits + part], a.v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&split_idx[row * kMaxSplits + part], a.i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+        const int before = __hip_atomic_fetch_add(&split_count[row], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (before + 1 == parts) {
+          __hip_atomic_store(&split_count[row], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          ArgMax r = {-INFINITY, 0x7fffffff};
+          for (int p = 0; p < parts; ++p) {
+            ArgMax b;
+            b.v = __hip_atomic_load(&split_val[row * kMaxSplits + p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            b.i = __hip_atomic_load(&split_idx[row * kMaxSplits + p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            r = better(r, b);
+          }
+          if ((unsigned)r.i >= (unsigned)vocab) r.i = 0;   // a row of NaN has no largest value: still name a token
+          out_token[row] = r.i;
+          out_logit[row] = lr[r.i];
+        }
+      }
+      return;
+    }
+  }
 
   ArgMax a = {-INFINITY, 0x7fffffff};
   sweep(lr, vocab, [&](float v, int i) { a = better(a, ArgMax{v, i}); });
   a = block_argmax(a, am);
   if ((unsigned)a.i >= (unsigned)vocab) a.i = 0;       // a row of NaN has no largest value: still name a token
-  const float temp = temperature[row];
   if (tid == 0) {          // the answer of a greedy row, and of a row whose weights are no numbers
     out_token[row] = a.i;
     out_logit[row] = lr[a.i];
@@ -483,8 +537,8 @@ extern "C" int atoma_sample(const float* logits, int ld, int n_rows, int vocab, 
                             int32_t* out_token, float* out_logit, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (vocab <= 0 || ld < vocab) return ATOMA_ERR_SHAPE;
-  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(kSampThreads), 0, stream, logits, ld, vocab, temperature, top_k,
-                     top_p, uniform, weights, out_token, out_logit);
+  hipLaunchKernelGGL(sample_kernel, dim3(n_rows, sample_splits(n_rows, vocab)), dim3(kSampThreads), 0, stream, logits, ld,
+                     vocab, temperature, top_k, top_p, uniform, weights, out_token, out_logit);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
@@ -569,8 +623,8 @@ extern "C" int atoma_sample_static(const float* logits, int ld, int n_rows, int 
   int rc;
   float* weights = scratch_address(rc);
   if (weights == nullptr) return rc;
-  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(kSampThreads), 0, stream, logits, ld, vocab, temperature, top_k,
-                     top_p, uniform, weights, out_token, out_logit);
+  hipLaunchKernelGGL(sample_kernel, dim3(n_rows, sample_splits(n_rows, vocab)), dim3(kSampThreads), 0, stream, logits, ld,
+                     vocab, temperature, top_k, top_p, uniform, weights, out_token, out_logit);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
