@@ -1,5 +1,8 @@
 // What this GPU delivers, measured: a read stream and a copy over device memory, and a loop of bfloat16 MFMAs.
 // bench.py prints these beside the published peaks (8 TB/s, 2.5 PFLOP/s), which stay the yardstick of its fractions.
+// And what a chain of dependent kernels costs beyond its bytes: the read stream launched over and over inside a
+// graph (with no bytes: an empty kernel behind another), and, for comparison, a barrier over the whole grid inside
+// one kernel, the thing a single persistent kernel would put in a launch's place.
 #include "common.h"
 
 using namespace atoma;
@@ -90,6 +93,47 @@ extern "C" int atoma_probe_copy(const void* src, void* dst, size_t bytes, int gr
 extern "C" int atoma_probe_mfma(int iters, int grid, void* sink, hipStream_t stream) {
   if (grid <= 0 || iters <= 0) return ATOMA_ERR_SHAPE;
   hipLaunchKernelGGL(probe_mfma_kernel, dim3(grid), dim3(256), 0, stream, iters, (float*)sink);
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// A barrier over the whole grid, nb times in one kernel: every workgroup counts itself in at a device-wide counter and
+// polls it until all have (relaxed atomics that go through to memory; no fence that would write back or invalidate a
+// cache).  Every wait is bounded: past kSpinLimit polls a workgroup writes an error word and no wait spins again.
+constexpr unsigned kSpinLimit = 1u << 18;
+
+__global__ void __launch_bounds__(512)
+probe_barrier_kernel(unsigned* __restrict__ counter, unsigned* __restrict__ err, int nb) {
+  for (int b = 0; b < nb; ++b) {
+    __syncthreads();
+    if (threadIdx.x == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
+      const unsigned target = (unsigned)(b + 1) * gridDim.x;
+      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      unsigned spins = 0;
+      while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        __builtin_amdgcn_s_sleep(1);
+        if (++spins > kSpinLimit) {
+          __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ctrl: 128 zeroed 32-bit words (word 0: the counter, word 64: set if a wait ran out).  grid workgroups of 512 threads,
+// which must all be resident at once: refused if the device cannot hold them.
+extern "C" int atoma_probe_barrier(void* ctrl, int grid, int nb, hipStream_t stream) {
+  if (grid <= 0 || nb <= 0 || ((uintptr_t)ctrl & 3)) return ATOMA_ERR_SHAPE;
+  int dev = 0, cus = 0, per_cu = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e == hipSuccess) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, probe_barrier_kernel, 512, 0);
+  if (e != hipSuccess) return (int)e;
+  if ((long long)grid > (long long)cus * per_cu) return ATOMA_ERR_SHAPE;
+  unsigned* c = (unsigned*)ctrl;
+  hipLaunchKernelGGL(probe_barrier_kernel, dim3(grid), dim3(512), 0, stream, c, c + 64, nb);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }

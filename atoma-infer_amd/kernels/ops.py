@@ -366,3 +366,60 @@ def measure_device_peaks(device: Optional[torch.device] = None, size_bytes: int 
     out["hbm_copy_gbs"] = round(2 * size_bytes / copy / 1e9, 1)
     out["mfma_bf16_tflops"] = round(grid * 4 * iters * 4 * 2 * 32 * 32 * 16 / mfma / 1e12, 1)
     return out
+
+
+def measure_chain_floors(device: Optional[torch.device] = None) -> dict:
+    """What a chain of dependent kernels costs on this GPU beyond its bytes, in microseconds a kernel (the probes of
+    ``microbench.hip``, each launched 32 times in a row inside one graph, every launch over other memory, so that
+    nothing comes from a cache): an empty kernel behind another; a read stream of 8, 16, 32 and 64 MB (the sizes of a
+    decode step's weight matrices); and a barrier over a grid of one workgroup a CU inside one kernel, which is what
+    a persistent kernel would pay where the chain pays a launch."""
+    lib = load_hip_module("microbench")
+    dev = device or torch.device("cuda:0")
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    n = 32
+    out = {}
+    with torch.cuda.device(dev):
+        src = torch.empty(n * (64 << 20), dtype=torch.uint8, device=dev).random_(0, 255)
+        sink = torch.zeros(4, dtype=torch.float32, device=dev)
+        base = src.data_ptr()
+
+        def chain(nbytes: int) -> float:
+            def launches():
+                for i in range(n):
+                    _check(lib.atoma_probe_read(ctypes.c_void_p(base + i * (64 << 20)), ctypes.c_size_t(nbytes), cus * 2,
+                                                4, _p(sink), _stream()), "probe_read")
+            launches()
+            torch.cuda.synchronize(dev)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                launches()
+            graph.replay()
+            torch.cuda.synchronize(dev)
+            best = float("inf")
+            for _ in range(4):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                graph.replay()
+                b.record()
+                torch.cuda.synchronize(dev)
+                best = min(best, a.elapsed_time(b) * 1e3 / n)
+            return round(best, 2)
+
+        out["empty_kernel_us"] = chain(0)
+        for mb in (8, 16, 32, 64):
+            out[f"read_{mb}mb_us"] = chain(mb << 20)
+        nb = 2000
+        best = float("inf")
+        for _ in range(3):
+            ctrl = torch.zeros(128, dtype=torch.int32, device=dev)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            _check(lib.atoma_probe_barrier(_p(ctrl), cus, nb, _stream()), "probe_barrier")
+            b.record()
+            torch.cuda.synchronize(dev)
+            if int(ctrl[64]) != 0:
+                raise KernelError("probe_barrier: a wait ran out (the grid was not resident at once)")
+            best = min(best, a.elapsed_time(b) * 1e3 / nb)
+        out["grid_barrier_us"] = round(best, 2)
+    return out

@@ -226,6 +226,9 @@ def main() -> int:
                     help="decode: the default run; serve3b, long8b: the other two workloads, one line of their own")
     ap.add_argument("--requests", type=int, default=0, help="requests of a --workload run (default: the workload's)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the probes of what the GPU delivers")
+    ap.add_argument("--chain-floors", action="store_true",
+                    help="only measure what a chain of dependent kernels costs beyond its bytes (an empty kernel, read "
+                         "streams of 8 to 64 MB, a grid-wide barrier), print one JSON line and stop")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
@@ -233,6 +236,11 @@ def main() -> int:
     if int(os.environ.get("WORLD_SIZE", "1")) > 1:
         print("bench.py: started with WORLD_SIZE > 1; this engine runs on one GPU", flush=True)
         return 2
+    if args.chain_floors:
+        import atoma_infer_amd  # noqa: F401
+        from atoma_infer_amd.kernels.ops import measure_chain_floors
+        print(json.dumps({"chain_floors": measure_chain_floors(), "unit": "us a kernel"}), flush=True)
+        return 0
     if args.workload != "decode":
         return workload_main(args)
     if args.prompt_len + args.steps + args.warmup + 2 * args.batch * (-(-args.prompt_len // 2048)) + 8 > args.context:

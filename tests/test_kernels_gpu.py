@@ -859,3 +859,18 @@ def test_decode_plans_behind_a_window(window, plan, monkeypatch):
         want = plain_attention(q, ks[e], vs[e], s0, scale, window, nh // nkv).reshape(1, nh * hd)
         err = (out[e:e + 1].double().cpu() - want).abs().max() / want.abs().max()
         assert err < 2e-2, f"request {e} at {s0}: {err:.3e}"
+
+
+def test_the_probes_of_what_the_gpu_delivers():
+    """The yardsticks that the bench prints beside its own figures: a read stream faster than any kernel here reads, a
+    copy, a loop of MFMAs near the published peak; and the costs of a chain of kernels (an empty kernel, read streams,
+    a grid-wide barrier whose waits are bounded and report if they run out)."""
+    from atoma_infer_amd.kernels import ops
+    peaks = ops.measure_device_peaks(size_bytes=1 << 28)
+    assert 3000 < peaks["hbm_read_gbs"] < 8000 and peaks["hbm_read_how"]
+    assert 2000 < peaks["hbm_copy_gbs"] < 8000
+    assert 1500 < peaks["mfma_bf16_tflops"] < 2600
+    floors = ops.measure_chain_floors()
+    assert 0.5 < floors["empty_kernel_us"] < 10
+    assert floors["empty_kernel_us"] < floors["read_8mb_us"] < floors["read_32mb_us"] < floors["read_64mb_us"] < 40
+    assert 0.5 < floors["grid_barrier_us"] < 50
