@@ -192,9 +192,10 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16
   const int kvh = blockIdx.x % nkv;
   const int ti = (blockIdx.x / nkv) * TASKS + slot;
   // with KSPLIT > 1 every wave must reach the barrier below: a wave without work runs an empty range
-  const bool has_task = ti < n_tasks && tasks[ti < n_tasks ? ti : 0].entry >= 0;
+  // (one load of the record: an empty one has an empty key range of its own)
+  const Task task = tasks[ti < n_tasks ? ti : 0];
+  const bool has_task = ti < n_tasks && task.entry >= 0;
   if (KSPLIT == 1 && !has_task) return;
-  const Task task = tasks[has_task ? ti : 0];
   const int g = nh / nkv;
   const int c = lane & 31, hg = lane >> 5;
   // the same in every lane; saying so keeps loop control and page arithmetic in scalar registers
