@@ -628,8 +628,10 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
 // a workgroup may have the 160 KB of a CU
 constexpr size_t kLdsBytes = 160 * 1024;
 constexpr size_t kMerge2Bytes = (DTILES * 16 + 2) * 64 * 4 * sizeof(float);
+constexpr size_t kMerge4Bytes = (DTILES * 16 + 2) * 64 * 6 * sizeof(float);      // two tasks, three waves each
 constexpr size_t kMerge8Bytes = (DTILES * 16 + 2) * 64 * 7 * sizeof(float);
 constexpr bool kSplit2Fits = kMerge2Bytes <= kLdsBytes;
+constexpr bool kSplit4Fits = kMerge4Bytes <= kLdsBytes;
 constexpr bool kSplit8Fits = kMerge8Bytes <= kLdsBytes;
 // two pieces of rows a wave: where the accumulators of both fit the registers of eight waves a workgroup, and the
 // merge of two waves a task (twice as large) lets two workgroups share a CU
@@ -687,6 +689,7 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
   if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
   else if (ksplit == 2 && row_tiles == 2) ATOMA_ATTN(4, 2, 2 * kMerge2Bytes, (kTwoPieces ? 2 : 1));
   else if (ksplit == 2 && kSplit2Fits) ATOMA_ATTN(4, (kSplit2Fits ? 2 : 1), kMerge2Bytes);
+  else if (ksplit == 4 && kSplit4Fits) ATOMA_ATTN(2, (kSplit4Fits ? 4 : 1), kMerge4Bytes);
   else if (ksplit == 8 && kSplit8Fits) ATOMA_ATTN(1, (kSplit8Fits ? 8 : 1), kMerge8Bytes);
   else return ATOMA_ERR_SHAPE;
 #undef ATOMA_ATTN

@@ -27,6 +27,7 @@ MAX_SPLIT_TASKS = 1024
 SPLIT_MAX_TOKENS = 16  # entries with at most this many tokens may be split along the keys
 SPLIT_MIN_KEYS = 2 * CHUNK
 SPLIT_WAVES_MIN_KEYS = 128   # a task of at least this many keys is walked by two waves, every other block each
+FOUR_WAVES_MIN_KEYS = 256    # ... by four, where the launch leaves half of the GPU idle (see build_tasks)
 _libs: Dict[Tuple[int, int], ctypes.CDLL] = {}
 
 
@@ -321,6 +322,14 @@ def build_tasks(starts: np.ndarray, counts: np.ndarray, group: int, window: int,
     arr = np.concatenate([head, rest])
     if len(head) and int((head[:, 5] - head[:, 4]).max()) >= SPLIT_WAVES_MIN_KEYS:
         waves = 2
+        # Four waves a task where the workgroups of two waves a task would fill at most half of the GPU (each then
+        # becomes two): a launch lasts as long as its longest wave, and halving the walks pays while there is room
+        # (prompts of 512 and 1,024 tokens at head size 64: 10.7 -> 8.8 and 17.2 -> 14.6 us; at 2,048 tokens, where
+        # the GPU is full, two waves a task share their keys among more rows and win, 31 against 36 us).
+        room = compute_units * (2 if head_size <= 64 else 1)
+        if (max_waves >= 4 and (len(head) // 4) * kv_heads * 2 <= room
+                and int((head[:, 5] - head[:, 4]).max()) >= FOUR_WAVES_MIN_KEYS):
+            waves = 4
     if row_tiles > 1 and len(head):
         waves = 2                     # tasks of two pieces run in the launch of two waves a task only
     return arr, (len(head) + len(split), len(combine), n_part, waves, row_tiles if len(head) else 1, merge)

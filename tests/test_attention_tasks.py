@@ -8,7 +8,7 @@ from atoma_infer_amd.kernels import attention_bf16 as A
 
 def coverage(arr, meta, starts, counts, group, window):
     n_main, n_comb, n_part, waves, tiles, merge = meta
-    assert waves in (1, 2, 8) and tiles in (1, 2) and (tiles == 1 or waves == 2)
+    assert waves in (1, 2, 4, 8) and tiles in (1, 2) and (tiles == 1 or waves == 2)
     main, comb = arr[:n_main], arr[n_main:]
     assert len(comb) == n_comb and (n_main % 4 == 0 or waves == 8)    # (eight waves: one task a workgroup)
     seen = {}          # (entry, token, head) -> list of key ranges, direct
@@ -202,3 +202,17 @@ def test_long_and_short_groups_meet_on_a_cu():
     sums = spans[:32] + spans[32:]
     assert sums.max() - sums.min() <= 32
     coverage(arr, meta, np.asarray([0]), np.asarray([2048]), 4, 0)
+
+
+def test_four_waves_a_task_where_two_would_leave_half_of_the_gpu_idle():
+    """A prompt whose tiles, at two waves a task, make no more workgroups than half of what the GPU holds is walked
+    by four waves a task (each workgroup becomes two); a prompt that fills the GPU keeps two, and so does a head size
+    whose merge of four waves' results does not fit."""
+    one = lambda n, **kw: A.build_tasks(np.asarray([0], dtype=np.int32), np.asarray([n], dtype=np.int32), 4, 0,
+                                        kv_heads=8, **kw)[1]
+    assert one(1024, max_waves=8)[3] == 4 and one(512, max_waves=8)[3] == 4
+    assert one(2048, max_waves=8)[3] == 2                       # 512 workgroups: the GPU is full
+    assert one(1024, max_waves=2)[3] == 2                       # the head size allows two at most
+    assert one(1024, max_waves=8, head_size=128)[3] == 2        # one workgroup a CU: 256 are a full round
+    assert one(512, max_waves=8, head_size=128)[3] == 4
+    assert one(100, max_waves=8)[3] == 1                        # short walks: a wave a task
