@@ -263,13 +263,6 @@ def main() -> int:
     log(f"model ready in {time.time() - t0:.1f} s; weights read per step: {model.weight_bytes() / 1e6:.1f} MB")
     kv_bytes_per_token = plan_cache(model.spec).bytes_per_token(2)
 
-    peaks = {}
-    if not args.no_peaks:
-        from atoma_infer_amd.kernels.ops import measure_device_peaks
-        log("probing what the GPU delivers (read stream, copy, MFMA loop) ...")
-        peaks = measure_device_peaks(model.device)
-        log(f"  {peaks}")
-
     log(f"prefill of {args.prefill_tokens} tokens ...")
     pre_s = prefill_run(model, args.prefill_tokens, 3, args.context)
     c = model.config
@@ -293,14 +286,6 @@ def main() -> int:
     achieved = step_bytes / (dt / args.steps) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4)}
-    if peaks:
-        # what the probes reached on this GPU, beside the published peaks that the fractions above are of
-        roofline["measured_peak"] = peaks["hbm_read_gbs"]
-        roofline["measured_how"] = peaks.get("hbm_read_how", "")
-        roofline["measured_copy"] = peaks["hbm_copy_gbs"]
-        roofline["frac_of_measured"] = round(achieved / peaks["hbm_read_gbs"], 4)
-        prefill["measured_peak_tflops"] = peaks["mfma_bf16_tflops"]
-        prefill["frac_of_measured"] = round(pre_flops / pre_s / (peaks["mfma_bf16_tflops"] * 1e12), 4)
 
     points = {}
     if not args.no_points:
@@ -311,6 +296,23 @@ def main() -> int:
             # the same roofline fraction as the headline's, with this batch's own mean context
             bytes_b = model.weight_bytes() + kv_bytes_per_token * ctx_b * b
             points[f"decode_b{b}_frac"] = round(bytes_b / (d / st) / 1e9 / HBM_PEAK_GBS, 4)
+
+    # the probes of what the GPU delivers run last: minutes of full load before the timed steps would only warm the
+    # chip against them
+    peaks = {}
+    if not args.no_peaks:
+        from atoma_infer_amd.kernels.ops import measure_device_peaks
+        log("probing what the GPU delivers (read stream, copy, MFMA loop) ...")
+        peaks = measure_device_peaks(model.device)
+        log(f"  {peaks}")
+    if peaks:
+        # what the probes reached on this GPU, beside the published peaks that the fractions above are of
+        roofline["measured_peak"] = peaks["hbm_read_gbs"]
+        roofline["measured_how"] = peaks.get("hbm_read_how", "")
+        roofline["measured_copy"] = peaks["hbm_copy_gbs"]
+        roofline["frac_of_measured"] = round(achieved / peaks["hbm_read_gbs"], 4)
+        prefill["measured_peak_tflops"] = peaks["mfma_bf16_tflops"]
+        prefill["frac_of_measured"] = round(pre_flops / pre_s / (peaks["mfma_bf16_tflops"] * 1e12), 4)
 
     line = {
         "metric": f"decode tok/s at batch {args.batch} ({name} sizes, {args.prompt_len}-token prompts); "
