@@ -11,41 +11,16 @@
 from __future__ import annotations
 
 import ctypes
-import dataclasses
 from typing import Optional
 
 import torch
 
+from ..parts.base import Begun        # (a norm begun by the product before it: the parts' type, finished here)
 from .library import load_hip_module
 from .ops import BF16, F32, _check, _p, _stream
 
 SKINNY_MAX_M = 64
 BEGUN_MAX_M = 16              # rows of a step whose norms are begun and finished by the products around them
-
-
-@dataclasses.dataclass
-class Begun:
-    """Activations whose norm is begun: ``data`` [T <= 16, W] bfloat16 is residual times norm weight, ``shares``
-    [parts, 16] float32 the rows' sums of squares in parts; the finished row is
-    ``data[t] / sqrt(shares[:, t].sum() / width + eps)``.  Products of this module finish it in their epilogue
-    (they are linear in their rows); ``tensor()`` finishes it into a tensor for any other reader."""
-    data: torch.Tensor
-    shares: torch.Tensor
-    eps: float
-    width: int
-    norm: object = None      # the part whose norm this is, so that no other takes it for its own
-
-    @property
-    def shape(self):
-        return self.data.shape
-
-    @property
-    def dtype(self):
-        return self.data.dtype
-
-    def tensor(self) -> torch.Tensor:
-        from . import ops
-        return ops.finish_norm(self.data, self.shares, self.eps, self.width)
 
 
 def _begun_args(x):

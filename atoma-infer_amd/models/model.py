@@ -13,7 +13,7 @@ import torch
 
 from ..config.base import ModelConfig
 from ..config.registry import Architecture, load_model_config
-from ..kernels.gemm_bf16 import Begun
+from ..parts.base import Begun
 from ..parts.linear import Normed
 from ..weights.loader import load_into, load_random_into
 from .spec import ModelSpec

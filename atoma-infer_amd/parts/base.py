@@ -101,6 +101,32 @@ class Part:
         return False
 
 
+@dataclasses.dataclass
+class Begun:
+    """Activations whose norm is begun (a norm's optional short cut, see ``Norm.add_product``): ``data`` [T <= 16, W]
+    bfloat16 is the residual rows times the norm's weight, ``shares`` [parts, 16] float32 the rows' sums of squares in
+    parts; the finished row is ``data[t] / sqrt(shares[:, t].sum() / width + eps)``.  A product that is linear in its
+    rows may finish it in its epilogue (those of ``kernels.gemm_bf16`` do); ``tensor()`` finishes it into a tensor
+    for any other reader."""
+    data: torch.Tensor
+    shares: torch.Tensor
+    eps: float
+    width: int
+    norm: object = None      # the part whose norm this is, so that no other takes it for its own
+
+    @property
+    def shape(self):
+        return self.data.shape
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    def tensor(self) -> torch.Tensor:
+        from ..kernels import ops
+        return ops.finish_norm(self.data, self.shares, self.eps, self.width)
+
+
 class Norm(Part):
     def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
                  ) -> torch.Tensor:
@@ -112,10 +138,10 @@ class Norm(Part):
         raise NotImplementedError
 
     # Optional: a norm may be *begun* by the kernel that makes its input rows and finished by the product that reads
-    # them (``kernels.gemm_bf16.Begun``), which saves the norm's own launch where launches are what a step costs.
+    # them (``Begun``), which saves the norm's own launch where launches are what a step costs.
     # A norm that cannot says None, and the caller runs ``add_norm``.
     def add_product(self, resid: torch.Tensor, x, w: torch.Tensor):
-        """``resid += x @ w^T`` in place with this norm of the new rows begun (``kernels.gemm_bf16.Begun``) or
+        """``resid += x @ w^T`` in place with this norm of the new rows begun (``Begun``) or
         finished (``parts.linear.Normed``); or None, nothing done."""
         return None
 

@@ -8,8 +8,7 @@ from __future__ import annotations
 
 from typing import Dict
 
-from ..kernels.gemm_bf16 import Begun
-from .base import Block, FeedForward, Mixer, Norm, WeightSpec, register_block
+from .base import Begun, Block, FeedForward, Mixer, Norm, WeightSpec, register_block
 from .linear import Normed, ResidualSink
 
 

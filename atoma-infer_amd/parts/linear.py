@@ -16,7 +16,7 @@ from typing import Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.gemm_bf16 import Begun
+from .base import Begun
 
 
 @dataclasses.dataclass

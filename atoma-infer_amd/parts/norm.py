@@ -10,7 +10,7 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import Norm, WeightSpec, register_norm
+from .base import Begun, Norm, WeightSpec, register_norm
 
 
 class RMSNorm(Norm):
@@ -53,7 +53,6 @@ class RMSNorm(Norm):
     def embed(self, table, tokens):
         if self.act_dtype is not torch.bfloat16 or tokens.numel() > 16 or table.shape[1] != self.width:
             return None
-        from ..kernels.gemm_bf16 import Begun
         resid, u, ss = ops.embed_begin_norm(tokens, table, self.weight)
         return resid, Begun(u, ss, self.eps, self.width, self)
 
