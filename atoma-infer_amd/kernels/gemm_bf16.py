@@ -11,6 +11,7 @@
 from __future__ import annotations
 
 import ctypes
+import dataclasses
 from typing import Optional
 
 import torch
@@ -95,6 +96,73 @@ def _slices_for(tiles: int, tiles_per_group: int, most: int) -> int:
     return slices
 
 
+@dataclasses.dataclass
+class TiledWeight:
+    """A weight [n, k] laid out in the order in which the streaming kernel's waves read it, for steps of at most 16
+    rows (``csrc/kernels/gemm_bf16.hip``, TILED): tiles of 16 rows x 32 values of K in the lanes' order, ordered by
+    batch of ``u`` steps, workgroup, wave, step, tile, for waves of ``rt`` tiles and ``wk`` waves a workgroup.  The
+    loads of a whole launch then sweep memory front to back as a plain read stream does (the gate-up matrix of Llama
+    1B: 11.5 us for the loads alone against 13.3 row-major).  A second copy of the weight: the row-major one serves
+    the products of more rows."""
+    data: torch.Tensor
+    n: int
+    k: int
+    rt: int
+    wk: int
+    u: int
+
+
+TILED_MAX_M = 16
+TILED_FOUR_TILES_MIN_M = 32
+TILED_SWIGLU_MAX_M = 64          # the fused SiLU-multiply reads the tiled copy with more rows too, in the copy's tiles
+TILED_MIN_ELEMENTS = 1 << 24      # smaller weights stream at the same pace row-major (measured: 8 and 34 MB)
+
+
+def tile_weight(w: torch.Tensor, rt: int, wk: int) -> Optional[TiledWeight]:
+    """The tiled copy of ``w`` [n, k] (bfloat16, row-major) for waves of ``rt`` tiles and ``wk`` waves a workgroup, or
+    None where the shape does not divide into whole batches of tiles."""
+    n, k = w.shape
+    u = int(lib().atoma_gemm_bf16_batch_depth(1, rt, wk))
+    if (w.dtype is not torch.bfloat16 or n % (16 * rt) or k % (32 * wk * u)
+            or not w.is_contiguous()):
+        return None
+    groups, batches = n // (16 * rt), k // (32 * wk * u)
+    t = w.view(groups, rt, 16, wk, batches, u, 4, 8)             # group, tile, row, wave, batch, step, piece, value
+    t = t.permute(4, 0, 3, 5, 1, 6, 2, 7).contiguous()            # batch, group, wave, step, tile, piece, row, value
+    return TiledWeight(t.view(-1), n, k, rt, wk, u)
+
+
+def tiled_plan(n: int, k: int, swiglu: bool):
+    """(rt, wk) of the tiled layout for a weight [n, k]: what ``_plan`` gives steps of at most 8 rows (the fused
+    SiLU-multiply's own choice for the gate-up matrix), so that the tiled kernel is the planned one; None for
+    weights that gain nothing."""
+    if n * k < TILED_MIN_ELEMENTS:
+        return None
+    rt, wk, _ = _plan(8, n, k, False)
+    if swiglu:
+        if rt % 2:
+            rt = 2
+        if wk == 4 and -(-n // 16) >= 1536:
+            rt = 4
+        if wk != 4 or rt not in (2, 4):
+            return None
+    elif (rt, wk) not in ((2, 8), (4, 4), (2, 4)):
+        return None
+    return rt, wk
+
+
+def skinny_tiled(x, tw: TiledWeight, out: torch.Tensor) -> None:
+    """out [M <= 16, n] = x @ w^T over the tiled copy of w; x may be a ``Begun`` norm."""
+    begun = _begun_args(x)
+    if isinstance(x, Begun):
+        x = x.data
+    m, k = x.shape
+    code = {torch.float32: F32, torch.bfloat16: BF16}[out.dtype]
+    _check(lib().atoma_gemm_bf16_skinny_tiled(_p(x), _p(tw.data), _p(out), code, m, tw.n, k, x.stride(0) if m > 1 else k,
+                                              out.stride(-2) if m > 1 else tw.n, tw.rt, tw.wk, *begun, _stream()),
+           "gemm_bf16_skinny_tiled")
+
+
 def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return (x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16 and x.dim() == 2 and w.dim() == 2
             and x.shape[1] == w.shape[1] and x.shape[1] % 32 == 0 and _aligned(x) and _aligned(w))
@@ -141,9 +209,21 @@ _MM_OUT_DTYPE = _probe_mm_out_dtype()
 
 
 def try_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None,
-               library_only: bool = False) -> Optional[torch.Tensor]:
+               library_only: bool = False, tiled: Optional[TiledWeight] = None) -> Optional[torch.Tensor]:
     """x [M, K] @ w [N, K]^T if a fast kernel takes the shape, else None (the caller falls back to float32 FMAs).
-    ``library_only``: None also where the library would not be the choice."""
+    ``library_only``: None also where the library would not be the choice.  ``tiled``: the tiled copy of ``w``, read
+    in its place by steps of at most 16 rows, in the copy's own plan (the head of Llama 1B, 525 MB, tiled for two
+    tiles and eight waves: 88, 90 and 99 us at 1, 8 and 16 rows against 88, 95 and 103 for the best row-major plan of
+    each)."""
+    if tiled is not None and not library_only and x.shape[0] <= TILED_MAX_M and x.shape[1] == tiled.k:
+        xd = x.data if isinstance(x, Begun) else x
+        dtype = out_dtype if out is None else out.dtype
+        if (xd.dtype is torch.bfloat16 and _aligned(xd)
+                and (dtype is torch.float32 or (dtype is torch.bfloat16 and (tiled.rt, tiled.wk) != (4, 4)))):
+            if out is None:
+                out = torch.empty((xd.shape[0], tiled.n), dtype=out_dtype, device=xd.device)
+            skinny_tiled(x, tiled, out)
+            return out
     if isinstance(x, Begun):
         if not skinny_ok(x.data, w):
             return None
@@ -209,7 +289,7 @@ def linear_planes(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
     return out
 
 
-def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
+def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor, tiled: Optional[TiledWeight] = None) -> Optional[torch.Tensor]:
     """silu(gate) * up of x @ w^T in one kernel, for few rows of x; w [2 I, K] is interleaved in blocks of 16.
 
     None when the shape is not taken (the caller then runs the product and the activation separately).
@@ -232,6 +312,16 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
     if (rt, wk) not in ((2, 1), (4, 1), (2, 4), (2, 8), (4, 4)):
         return None
     out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    if tiled is not None and (tiled.n, tiled.k) == (n, k) and tiled.wk == wk and m <= TILED_SWIGLU_MAX_M:
+        # waves of four tiles read a copy made for two as well, and gain on it from 32 rows on (measured over the
+        # 16 layers of Llama 1B: 1,346 against 1,362 us a step at 32 rows, 1,929 against 1,970 at 64; 1,235 against
+        # 1,231 at 24)
+        rt = 4 if tiled.rt == 4 or (m >= TILED_FOUR_TILES_MIN_M and n % 64 == 0) else 2
+        _check(lib().atoma_gemm_bf16_skinny_swiglu_tiled(_p(x), _p(tiled.data), _p(out), m, n, k,
+                                                         x.stride(0) if m > 1 else k, n // 2, rt, tiled.rt, wk, *begun,
+                                                         _stream()),
+               "gemm_bf16_skinny_swiglu_tiled")
+        return out
     _check(lib().atoma_gemm_bf16_skinny_swiglu(_p(x), _p(w), _p(out), m, n, k, x.stride(0) if m > 1 else k,
                                                w.stride(0), n // 2, rt, wk, *begun, _stream()),
            "gemm_bf16_skinny_swiglu")

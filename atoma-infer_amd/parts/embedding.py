@@ -45,6 +45,7 @@ class OutputHead(Part):
     def __init__(self, width: int, vocab_size: int, tied_to: Optional[TokenEmbedding] = None):
         self.width, self.vocab_size, self.tied_to = int(width), int(vocab_size), tied_to
         self.weight: Optional[torch.Tensor] = None
+        self.tiled = None
 
     def graph_safe(self) -> bool:
         return True
@@ -54,9 +55,17 @@ class OutputHead(Part):
 
     def load(self, get, device, act_dtype) -> None:
         self.weight = self.tied_to.weight if self.tied_to is not None else get("weight").to(device).contiguous()
+        # a second copy in the order the streaming kernel's waves read it, for steps of few rows (the row-major one
+        # serves the embedding's gather and the products of many rows)
+        self.tiled = None
+        if act_dtype is torch.bfloat16 and self.weight.dtype is torch.bfloat16 and self.weight.is_cuda:
+            from ..kernels import gemm_bf16
+            plan = gemm_bf16.tiled_plan(self.vocab_size, self.width, swiglu=False)
+            if plan is not None:
+                self.tiled = gemm_bf16.tile_weight(self.weight, *plan)
 
     def device_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
 
     def forward(self, x) -> torch.Tensor:
-        return linear(x, self.weight, torch.float32)
+        return linear(x, self.weight, torch.float32, tiled=self.tiled)

@@ -40,13 +40,14 @@ def as_tensor(x) -> torch.Tensor:
 
 
 def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+           out: Optional[torch.Tensor] = None, tiled=None) -> torch.Tensor:
     """x [M, K] (row stride free) times w [N, K] transposed -> [M, N] in ``out_dtype`` (default: x's dtype).
-    x may be a ``Begun`` norm."""
+    x may be a ``Begun`` norm.  ``tiled``: a copy of ``w`` in the order the streaming kernel reads it
+    (``kernels.gemm_bf16.tile_weight``), which steps of few rows read in its place."""
     out_dtype = out_dtype or x.dtype
     if x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16:
         from ..kernels import gemm_bf16
-        y = gemm_bf16.try_linear(x, w, out_dtype, out)
+        y = gemm_bf16.try_linear(x, w, out_dtype, out, tiled=tiled)
         if y is not None:
             return y
     return ops.gemm_generic(as_tensor(x), w, out_dtype, out)

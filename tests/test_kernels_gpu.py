@@ -1,4 +1,5 @@
 """Each kernel alone against a plain float32 formula in PyTorch, at sizes other than the engine's."""
+import ctypes
 import math
 
 import pytest
@@ -874,3 +875,62 @@ def test_the_probes_of_what_the_gpu_delivers():
     assert 0.5 < floors["empty_kernel_us"] < 10
     assert floors["empty_kernel_us"] < floors["read_8mb_us"] < floors["read_32mb_us"] < floors["read_64mb_us"] < 40
     assert 0.5 < floors["grid_barrier_us"] < 50
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 13, 16])
+@pytest.mark.parametrize("n,k,rt,wk", [(128, 512, 2, 8), (4032, 1024, 2, 8), (256, 256, 4, 4), (1000 * 64, 256, 4, 4),
+                                       (96, 256, 2, 4), (2048, 2048, 2, 4)])
+def test_gemm_over_a_tiled_weight_equals_the_row_major_one(m, n, k, rt, wk):
+    """The copy of a weight laid out in the order the streaming kernel's waves read it (batch of steps, workgroup,
+    wave, step, tile, lane) gives the very bits of the row-major weight read by the same plan, also with the rows a
+    begun norm; and the offsets the library states are where the Python tiling puts every element."""
+    from atoma_infer_amd.kernels import gemm_bf16, ops
+    x = rnd(m, k, dtype=torch.bfloat16, seed=m)
+    w = rnd(n, k, dtype=torch.bfloat16, seed=n + k, scale=0.1)
+    tw = gemm_bf16.tile_weight(w, rt, wk)
+    assert tw is not None and (tw.n, tw.k, tw.rt, tw.wk) == (n, k, rt, wk) and tw.data.numel() == n * k
+    g = torch.Generator().manual_seed(3)
+    off = gemm_bf16.lib().atoma_gemm_bf16_tiled_offset
+    off.restype = ctypes.c_longlong
+    for _ in range(50):
+        i, j = int(torch.randint(0, n, (1,), generator=g)), int(torch.randint(0, k, (1,), generator=g))
+        at = off(ctypes.c_longlong(i), ctypes.c_longlong(j), ctypes.c_longlong(n), ctypes.c_longlong(k), rt, wk, tw.u)
+        assert tw.data[at] == w[i, j], (i, j, at)
+    for dtype in (torch.float32, torch.bfloat16):
+        if dtype is torch.bfloat16 and (rt, wk) == (4, 4):
+            continue                                            # no such instance: the head's plan, float32 out
+        want = torch.empty(m, n, dtype=dtype, device=DEV)
+        gemm_bf16.skinny(x, w, want, 1, rt, wk)
+        got = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+        gemm_bf16.skinny_tiled(x, tw, got)
+        assert torch.equal(got, want)
+    ref = x.double().cpu() @ w.double().cpu().T
+    assert (got.double().cpu() - ref).abs().max() <= 2e-2 * ref.abs().max()
+    # a begun norm as the rows
+    ss = torch.rand(7, 16, device=DEV) + 0.5
+    b = gemm_bf16.Begun(x, ss, 1e-5, k)
+    want = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    gemm_bf16.skinny(b, w, want, 1, rt, wk)
+    got = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    gemm_bf16.skinny_tiled(b, tw, got)
+    assert torch.equal(got, want)
+    assert gemm_bf16.tile_weight(rnd(n + 16, k + 32, dtype=torch.bfloat16), rt, wk) is None      # no whole batches
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 23, 48, 64])
+@pytest.mark.parametrize("inter,k,rt", [(64, 256, 2), (8192, 2048, 2), (1024, 512, 4)])
+def test_swiglu_gemm_over_a_tiled_weight_equals_the_row_major_one(m, inter, k, rt, monkeypatch):
+    from atoma_infer_amd.kernels import gemm_bf16
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    wg, wu = rnd(inter, k, dtype=torch.bfloat16, seed=2, scale=0.1), rnd(inter, k, dtype=torch.bfloat16, seed=3, scale=0.1)
+    w = interleave16(wg, wu)
+    # the plan that the fused product would choose must be the tiled copy's: force it for the small shapes
+    monkeypatch.setattr(gemm_bf16, "_plan", lambda *a, **kw: (rt, 4, 1))
+    tw = gemm_bf16.tile_weight(w, rt, 4)
+    assert tw is not None
+    want = gemm_bf16.try_linear_swiglu(x, w)
+    got = gemm_bf16.try_linear_swiglu(x, w, tw)
+    assert want is not None and got is not None and torch.equal(got, want)
+    g, u = x.double().cpu() @ wg.double().cpu().T, x.double().cpu() @ wu.double().cpu().T
+    ref = torch.nn.functional.silu(g) * u
+    assert (got.double().cpu() - ref).abs().max() <= 1e-2 * ref.abs().max()
