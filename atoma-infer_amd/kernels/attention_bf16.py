@@ -93,6 +93,7 @@ LONG_KEYS = 16384
 # 1,024 keys and equal at 2,048 for the pair alone, and 10 to 27 us quicker over the 16 layers of a decode step of 8
 # requests or of 1; from 4,096 keys on one wave's walk over the parts costs more than the second launch.
 MERGE_MAX_KEYS = 2304
+MERGE_WHOLE_MAX_KEYS = 512    # with the merge in the kernel: whole ranges for few pairs only up to this many keys
 MERGE_IN_KERNEL = True        # False: always the merging kernel (tests run both)
 
 
@@ -117,13 +118,31 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False
     heads; ``max_keys`` is rounded up to 256.
     """
     pairs = n_split * kv_heads
+    tasks = n_split * -(-max_keys // CHUNK) * kv_heads
+    if whole_ok and merges_in_kernel(max_keys):
+        # With the chunks merged by the attention kernel itself, chunks cost no second launch, and four waves that
+        # share a chunk (64 or 128 keys each, merged in LDS) shorten a wave's chain of dependent loads without more
+        # partial results.  Measured over the 16 layers of a Llama 1B decode step (head size 64, 8 KV heads; 700,
+        # 1,000, 1,500 and 2,049 keys; 1 to 16 requests): 256-key chunks up to 512 tasks (one request of 2,049 keys
+        # 773 against 788 us a step with 128-key chunks of a wave each, four 816 against 851, eight of 1,000 keys 838
+        # against 860 for whole ranges), 512-key chunks beyond (eight requests of 2,049 keys 901 against 909 us with
+        # 256-key chunks of two waves, twelve of 1,500 keys 943 against 968 for whole ranges); whole ranges from 128
+        # pairs on (sixteen requests of 2,049 keys 1,084 against 1,125 us) and, for the pair alone, up to 512 keys.
+        # Wide heads with few tasks keep a wave a chunk (head size 128, one request of 1,024 keys: 12.2 against
+        # 12.8 us a layer).
+        if max_keys <= MERGE_WHOLE_MAX_KEYS or pairs >= WHOLE_MIN_PAIRS:
+            return 0, 8
+        if tasks > 544:
+            return 2 * CHUNK, 4
+        if head_size > 64 and tasks <= 300:
+            return 128, 1
+        return CHUNK, 4
     if whole_ok:
         walk = max_keys * head_size
         if pairs >= WHOLE_MIN_PAIRS or any(pairs >= p and walk <= w for p, w in WHOLE_SHORT_WALKS):
             return 0, 8
-    tasks = n_split * -(-max_keys // CHUNK) * kv_heads
     if merges_in_kernel(max_keys):
-        # (with the chunks merged by the attention kernel itself; measured at 1,024 and 2,048 keys, 1 to 16 requests)
+        # (heads so wide that fewer than four waves may share a task; and the split entries of a prompt step)
         return (128, 1) if tasks <= 300 else (CHUNK, 2)
     if tasks <= 160:
         return 128, 1

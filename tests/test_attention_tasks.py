@@ -137,11 +137,22 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     assert A.build_tasks(far, counts[:8], group, 0, 3072, kv_heads=8, max_waves=8)[1][1] > 0
     assert A.build_tasks(far, counts[:8], group, 0, 3072, kv_heads=8, max_waves=8, head_size=128)[1][1] > 0
     # few pairs with few keys to walk: whole ranges again (the second kernel would cost more than the walk)
-    near = np.full(8, 999, dtype=np.int32)
-    arr2, meta2 = A.build_tasks(near, counts[:8], group, 0, 1024, kv_heads=8, max_waves=8)
+    near = np.full(8, 500, dtype=np.int32)
+    arr2, meta2 = A.build_tasks(near, counts[:8], group, 0, 512, kv_heads=8, max_waves=8)
     assert meta2 == (8 * -(-group // 32), 0, 0, 8, 1, False)
     coverage(arr2, meta2, near, counts[:8], group, 0)
-    assert A.build_tasks(near, counts[:8], group, 0, 1024, kv_heads=8, max_waves=8, head_size=128)[1][1] > 0
+    assert A.build_tasks(near + 500, counts[:8], group, 0, 1024, kv_heads=8, max_waves=8)[1][1] > 0
+    # contexts whose chunks the attention kernel merges itself: four waves share a chunk of 256 keys, of 512 where
+    # there are many; whole ranges for short contexts and from sixteen requests of 8 KV heads on; a wave a chunk for
+    # wide heads with few tasks, and where fewer than four waves may share a task
+    assert A.chunk_for(1, 2048, 8, whole_ok=True, head_size=64) == (256, 4)
+    assert A.chunk_for(8, 2048, 8, whole_ok=True, head_size=64) == (256, 4)
+    assert A.chunk_for(8, 2304, 8, whole_ok=True, head_size=64) == (512, 4)
+    assert A.chunk_for(12, 2048, 8, whole_ok=True, head_size=128) == (512, 4)
+    assert A.chunk_for(16, 2048, 8, whole_ok=True, head_size=64) == (0, 8)
+    assert A.chunk_for(4, 512, 8, whole_ok=True, head_size=64) == (0, 8)
+    assert A.chunk_for(1, 2048, 8, whole_ok=True, head_size=128) == (128, 1)
+    assert A.chunk_for(1, 2048, 8, whole_ok=False, head_size=64) == (128, 1)
     # twelve requests of 8 KV heads: whole ranges up to 8,192 keys of head size 64, 4,096 of head size 128
     assert A.chunk_for(12, 8192, 8, whole_ok=True, head_size=64) == (0, 8)
     assert A.chunk_for(12, 8192, 8, whole_ok=True, head_size=128)[0] > 0

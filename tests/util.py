@@ -130,5 +130,6 @@ def force_chunked_decode(monkeypatch, second_kernel: bool = False):
     from atoma_infer_amd.kernels import attention_bf16
     monkeypatch.setattr(attention_bf16, "WHOLE_MIN_PAIRS", 10 ** 9)
     monkeypatch.setattr(attention_bf16, "WHOLE_SHORT_WALKS", ())
+    monkeypatch.setattr(attention_bf16, "MERGE_WHOLE_MAX_KEYS", 0)
     if second_kernel:
         monkeypatch.setattr(attention_bf16, "MERGE_IN_KERNEL", False)
