@@ -124,7 +124,8 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   const int r16 = lane & 15, kg = lane >> 4;
   static_assert(!HALF || (RT == 1 && MT == 1 && !SWIGLU && !ROPE), "half tiles: one tile, residual epilogue");
   static_assert(!PACK || HALF, "packed activations go with half tiles");
-  static_assert(!TILED || (WN == 1 && !HALF && !ROPE), "the tiled layout: whole tiles, K split over a workgroup's waves");
+  static_assert(!TILED || (WN == 1 && (!HALF || TILED == 1)),
+                "the tiled layout: K split over a workgroup's waves");
   const int n_base = (blockIdx.x * WN + wn) * (HALF ? 8 : RT * 16);
   constexpr int KSTEP = HALF ? 64 : 32;               // values of K that a wave's step covers
   const int k_slices = gridDim.y * WK;
@@ -594,11 +595,33 @@ extern "C" int atoma_gemm_bf16_resid_parts(int N, int rt, int wk, int half) {
   return ((N + cols - 1) / cols) * wn;
 }
 
-extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M, int N, int K, int lda, int ldw,
-                                            int rt, int wk, int depth, int half, const float* ss_in, int parts_in, float eps_in,
-                                            int width_in, float* resid, const void* gamma, int gamma_dtype,
-                                            void* u_out, float* ss_out, hipStream_t stream) {
+template <int R, int WN, int WK, int U, bool H>
+static void resid_kernels(bool tiled, const void* a, const void* w, int M, int N, int K, int lda, int ldw, float* resid,
+                          const FuseArgs& fa, hipStream_t stream) {
+  const int cols = H ? WN * 8 : WN * R * 16;
+  dim3 grid((N + cols - 1) / cols, 1), block(64 * WN * WK);
+#define ATOMA_RESID_KERNEL(PACK_, TILED_)                                                                             \
+  hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN, WK, float, false, false, U, H, PACK_, TILED_>), grid, block, 0,    \
+                     stream, (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0,         \
+                     RopeArgs{}, fa)
+  if constexpr (H && WN == 1 && WK == 8 && U == 4) {
+    if (tiled) {
+      if (M <= 8) ATOMA_RESID_KERNEL(true, 1);
+      else ATOMA_RESID_KERNEL(false, 1);
+      return;
+    }
+  }
+  if (H && M <= 8) ATOMA_RESID_KERNEL(H, 0);        // (activations packed as the half tiles are)
+  else ATOMA_RESID_KERNEL(false, 0);
+#undef ATOMA_RESID_KERNEL
+}
+
+static int launch_resid(const void* a, const void* w, bool tiled, int M, int N, int K, int lda, int ldw, int rt, int wk,
+                        int depth, int half, const float* ss_in, int parts_in, float eps_in, int width_in, float* resid,
+                        const void* gamma, int gamma_dtype, void* u_out, float* ss_out, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
+  // the tiled layout (half tiles only: 8 rows x 64 values of K in the lanes' order, see atoma_gemm_bf16_tiled_offset_half)
+  if (tiled && (!half || wk != 8 || depth != 4 || (N & 7) || K % (64 * wk * depth))) return ATOMA_ERR_SHAPE;
   if (M > 16 || K <= 0 || K % ((half ? 64 : 32) * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K || (N & 3) ||
       ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || !resid || !gamma || !u_out || !ss_out ||
       ((uintptr_t)resid & 15) || ((uintptr_t)gamma & 15) || ((uintptr_t)u_out & 7) ||
@@ -613,16 +636,7 @@ extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M,
   // (the float32 instance; nothing is stored through c)
 #define ATOMA_RESID(R, WN_, WK_, U_, H_)                                                                           \
   if (rt == R && wk == WK_ && depth == U_ && (half != 0) == H_) {                                                  \
-    const int cols = H_ ? WN_ * 8 : WN_ * R * 16;                                                                  \
-    dim3 grid((N + cols - 1) / cols, 1), block(64 * WN_ * WK_);                                                    \
-    if (H_ && M <= 8)                                                                                              \
-      hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN_, WK_, float, false, false, U_, H_, H_>), grid, block, 0,    \
-                         stream, (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0,   \
-                         RopeArgs{}, fa);                                                                          \
-    else                                                                                                           \
-      hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN_, WK_, float, false, false, U_, H_>), grid, block, 0,        \
-                         stream, (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0,   \
-                         RopeArgs{}, fa);                                                                          \
+    resid_kernels<R, WN_, WK_, U_, H_>(tiled, a, w, M, N, K, lda, ldw, resid, fa, stream);                         \
     ATOMA_LAUNCH_CHECK();                                                                                          \
     return 0;                                                                                                      \
   }
@@ -639,6 +653,34 @@ extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M,
   ATOMA_RESID(1, 4, 1, 4, true)
 #undef ATOMA_RESID
   return ATOMA_ERR_SHAPE;
+}
+
+extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M, int N, int K, int lda, int ldw,
+                                            int rt, int wk, int depth, int half, const float* ss_in, int parts_in, float eps_in,
+                                            int width_in, float* resid, const void* gamma, int gamma_dtype,
+                                            void* u_out, float* ss_out, hipStream_t stream) {
+  return launch_resid(a, w, false, M, N, K, lda, ldw, rt, wk, depth, half, ss_in, parts_in, eps_in, width_in, resid,
+                      gamma, gamma_dtype, u_out, ss_out, stream);
+}
+
+// The same over a weight in the tiled layout of half tiles (eight waves a workgroup, batches of four steps).
+extern "C" int atoma_gemm_bf16_skinny_resid_tiled(const void* a, const void* w_tiled, int M, int N, int K, int lda,
+                                                  const float* ss_in, int parts_in, float eps_in, int width_in,
+                                                  float* resid, const void* gamma, int gamma_dtype, void* u_out,
+                                                  float* ss_out, hipStream_t stream) {
+  return launch_resid(a, w_tiled, true, M, N, K, lda, K, 1, 8, 4, 1, ss_in, parts_in, eps_in, width_in, resid, gamma,
+                      gamma_dtype, u_out, ss_out, stream);
+}
+
+// Where element (row n, column k) of a weight [N, K] lies in the tiled layout of half tiles: tiles of 8 rows x 64
+// values of K (lane l holds row l % 8 and the 8 values from 8 (l / 16) + 32 (l / 8 % 2) on), ordered by batch of u
+// steps, workgroup (8 rows), wave (K / wk values each), step.  N % 8 == 0 and K % (64 wk u) == 0.
+extern "C" long long atoma_gemm_bf16_tiled_offset_half(long long n, long long k, long long N, long long K, int wk,
+                                                       int u) {
+  const long long k_len = K / wk, wg = n / 8, row = n % 8;
+  const long long slice = k / k_len, kk = k % k_len, batch = kk / (64 * u), step = (kk / 64) % u, p = kk % 64;
+  const long long lane = ((p % 32) / 8) * 16 + (p / 32) * 8 + row;
+  return (((batch * (N / 8) + wg) * wk + slice) * u + step) * 512 + lane * 8 + k % 8;
 }
 
 template <int MT, int RT, int WN, int WK>
@@ -683,11 +725,11 @@ extern "C" int atoma_gemm_bf16_skinny_swiglu(const void* a, const void* w, void*
   }
 }
 
-template <int MT, int RT, int WN, int WK>
+template <int MT, int RT, int WN, int WK, int TILED = 0>
 static int launch_rope(const void* a, const void* w, void* c, int M, int N, int K, int lda, int ldw, int ldc,
                        const RopeArgs& ra, const FuseArgs& fa, hipStream_t stream) {
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, false, true>), grid, block, 0, stream,
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, false, true, 0, false, false, TILED>), grid, block, 0, stream,
                      (const uint16_t*)a, (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, ra, fa);
   ATOMA_LAUNCH_CHECK();
   return 0;
@@ -734,6 +776,28 @@ extern "C" int atoma_gemm_bf16_skinny_rope(const void* a, const void* w, void* c
     case 3: return launch_rope_mt<3>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, fa, stream);
     default: return launch_rope_mt<4>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, ra, fa, stream);
   }
+}
+
+// The same for at most 16 rows over a weight in the tiled layout made for waves of rt tiles (1 or 2) and 4 waves a
+// workgroup.
+extern "C" int atoma_gemm_bf16_skinny_rope_tiled(const void* a, const void* w_tiled, void* c, int M, int K, int lda,
+                                                 int ldc, int rt, int wk, const int32_t* positions, const float* cos_t,
+                                                 const float* sin_t, void* kcache, void* vcache,
+                                                 const int32_t* slot_mapping, int page_size, int nh, int nkv, int hd,
+                                                 const float* ss_in, int parts_in, float eps_in, int width_in,
+                                                 hipStream_t stream) {
+  if (M <= 0) return 0;
+  const int N = (nh + 2 * nkv) * hd;
+  if (!fuse_in_ok(ss_in, parts_in, eps_in, width_in, M)) return ATOMA_ERR_SHAPE;
+  const FuseArgs fa = fuse_in(ss_in, parts_in, eps_in, width_in);
+  if (M > 16 || K <= 0 || wk != 4 || (rt != 1 && rt != 2) || N % (16 * rt) || K % (32 * wk * batch_depth(1, rt, wk)) ||
+      (lda & 7) || lda < K || ldc < nh * hd || (ldc & 1) || ((uintptr_t)a & 15) || ((uintptr_t)w_tiled & 15) ||
+      ((uintptr_t)c & 3) || (hd & 3) || nh <= 0 || nkv <= 0 || page_size <= 0 || !positions || !cos_t || !sin_t ||
+      !kcache || !vcache || !slot_mapping || ((uintptr_t)kcache & 3))
+    return ATOMA_ERR_SHAPE;
+  const RopeArgs ra{positions, cos_t, sin_t, (uint16_t*)kcache, (uint16_t*)vcache, slot_mapping, page_size, nh, nkv, hd};
+  if (rt == 1) return launch_rope<1, 1, 1, 4, 1>(a, w_tiled, c, M, N, K, lda, K, ldc, ra, fa, stream);
+  return launch_rope<1, 2, 1, 4, 2>(a, w_tiled, c, M, N, K, lda, K, ldc, ra, fa, stream);
 }
 
 // The fused q, k, v projection of 17 to 64 rows as float32 planes of a K-split product (which about 256 workgroups

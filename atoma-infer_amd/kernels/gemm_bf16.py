@@ -132,6 +132,30 @@ def tile_weight(w: torch.Tensor, rt: int, wk: int) -> Optional[TiledWeight]:
     return TiledWeight(t.view(-1), n, k, rt, wk, u)
 
 
+def tile_weight_half(w: torch.Tensor) -> Optional[TiledWeight]:
+    """The tiled copy of ``w`` [n, k] for the product that adds into the residual stream with half tiles (8 rows of
+    the weight a wave, eight waves a workgroup, batches of four steps of 64 values of K), or None where the shape
+    does not divide or ``resid_plan`` would not choose that plan."""
+    n, k = w.shape
+    wk, u = 8, 4
+    if (w.dtype is not torch.bfloat16 or not w.is_contiguous() or n % 8 or k % (64 * wk * u)
+            or resid_plan(1, n, k) != (1, wk, u, 1)):
+        return None
+    t = w.view(n // 8, 8, wk, k // (64 * wk * u), u, 2, 4, 8)     # group, row, wave, batch, step, half, piece, value
+    t = t.permute(3, 0, 2, 4, 6, 5, 1, 7).contiguous()            # batch, group, wave, step, piece, half, row, value
+    return TiledWeight(t.view(-1), n, k, 0, wk, u)
+
+
+def tile_weight_rope(w: torch.Tensor) -> Optional[TiledWeight]:
+    """The tiled copy of a fused q, k, v weight for the product with the rotary epilogue at up to 8 rows, or None
+    where that product's plan has no tiled kernel."""
+    n, k = w.shape
+    rt, wk, _ = _plan(8, n, k, False)
+    if wk != 4 or rt > 2:
+        return None
+    return tile_weight(w, rt, wk)
+
+
 def tiled_plan(n: int, k: int, swiglu: bool):
     """(rt, wk) of the tiled layout for a weight [n, k]: what ``_plan`` gives steps of at most 8 rows (the fused
     SiLU-multiply's own choice for the gate-up matrix), so that the tiled kernel is the planned one; None for
@@ -337,7 +361,8 @@ ROPE_PLANES_MIN_M = 40
 
 def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                     kcache: torch.Tensor, vcache: torch.Tensor, slot_mapping: torch.Tensor, page_size: int, nh: int,
-                    nkv: int, hd: int, always: bool = False) -> Optional[torch.Tensor]:
+                    nkv: int, hd: int, always: bool = False, tiled: Optional[TiledWeight] = None,
+                    ) -> Optional[torch.Tensor]:
     """The fused q, k, v projection with rotary encoding and the cache write in its epilogue, for few rows of x.
 
     ``w`` has the rows of its q and k heads in pair order (see ``parts/attention.py``).  Returns the rotated q
@@ -371,6 +396,12 @@ def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, c
         rt = 2
     if 8 < m <= 16 and rt == 1 and wk == 4 and n >= 5120:
         rt = 2          # (9 to 16 rows at Llama 3B's and 8B's sizes: 14.1 and 17.1 us against 15.3 and 18.9)
+    if tiled is not None and m <= TILED_MAX_M and (tiled.n, tiled.k, tiled.rt, tiled.wk) == (n, k, rt, wk):
+        _check(lib().atoma_gemm_bf16_skinny_rope_tiled(_p(x), _p(tiled.data), _p(out), m, k, x.stride(0) if m > 1 else k,
+                                                       nh * hd, rt, wk, _p(positions), _p(cos), _p(sin), _p(kcache),
+                                                       _p(vcache), _p(slot_mapping), int(page_size), nh, nkv, hd, *begun,
+                                                       _stream()), "gemm_bf16_skinny_rope_tiled")
+        return out
     _check(lib().atoma_gemm_bf16_skinny_rope(_p(x), _p(w), _p(out), m, k, x.stride(0) if m > 1 else k, w.stride(0),
                                              nh * hd, rt, wk, _p(positions), _p(cos), _p(sin), _p(kcache), _p(vcache),
                                              _p(slot_mapping), int(page_size), nh, nkv, hd, *begun, _stream()),
@@ -398,9 +429,11 @@ def resid_plan(m: int, n: int, k: int):
     return 1, wk, depth, half
 
 
-def try_linear_resid(x, w: torch.Tensor, resid: torch.Tensor, gamma: torch.Tensor, eps: float) -> Optional[Begun]:
+def try_linear_resid(x, w: torch.Tensor, resid: torch.Tensor, gamma: torch.Tensor, eps: float,
+                     tiled: Optional[TiledWeight] = None) -> Optional[Begun]:
     """resid [M <= 16, N] float32 += x @ w^T in place, with the norm (gamma, eps) of the new rows begun: returns
-    it as ``Begun``, or None (and nothing done) when the shape is not taken.  x may itself be ``Begun``."""
+    it as ``Begun``, or None (and nothing done) when the shape is not taken.  x may itself be ``Begun``.  ``tiled``:
+    the copy of ``w`` that ``tile_weight_half`` made, read in its place."""
     begun = _begun_args(x)
     xd = x.data if isinstance(x, Begun) else x
     m, k = xd.shape
@@ -414,6 +447,11 @@ def try_linear_resid(x, w: torch.Tensor, resid: torch.Tensor, gamma: torch.Tenso
     u = torch.empty((m, n), dtype=torch.bfloat16, device=w.device)
     shares = torch.empty((parts, 16), dtype=torch.float32, device=w.device)
     code = F32 if gamma.dtype is torch.float32 else BF16
+    if tiled is not None and (tiled.n, tiled.k, tiled.rt) == (n, k, 0) and (rt, wk, depth, half) == (1, 8, 4, 1):
+        _check(lib().atoma_gemm_bf16_skinny_resid_tiled(_p(xd), _p(tiled.data), m, n, k, xd.stride(0) if m > 1 else k,
+                                                        *begun, _p(resid), _p(gamma), code, _p(u), _p(shares),
+                                                        _stream()), "gemm_bf16_skinny_resid_tiled")
+        return Begun(u, shares, float(eps), n)
     _check(lib().atoma_gemm_bf16_skinny_resid(_p(xd), _p(w), m, n, k, xd.stride(0) if m > 1 else k, w.stride(0), rt, wk,
                                               depth, half, *begun, _p(resid), _p(gamma), code, _p(u), _p(shares), _stream()),
            "gemm_bf16_skinny_resid")

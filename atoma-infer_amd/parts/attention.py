@@ -44,6 +44,7 @@ class PagedAttention(Mixer):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
+        self.w_qkv_tiled = self.w_o_tiled = None
         self.act_dtype = torch.float32
         self.paired = False      # q and k columns in pair order (set at load time)
         self.slopes: Optional[torch.Tensor] = None      # per-head bias of the scores by distance, if the encoding has one
@@ -81,6 +82,13 @@ class PagedAttention(Mixer):
         self.w_qkv = torch.cat([w.to(device=device, dtype=dt) for w in ws], dim=0).contiguous()
         self.w_o = get("o_proj.weight").to(device).contiguous()
         self.act_dtype = act_dtype
+        # second copies in the order in which the kernels of steps of few rows read them
+        self.w_qkv_tiled = self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_qkv.dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            if self.paired:
+                self.w_qkv_tiled = gemm_bf16.tile_weight_rope(self.w_qkv)
+            self.w_o_tiled = gemm_bf16.tile_weight_half(self.w_o)
 
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
@@ -129,7 +137,8 @@ class PagedAttention(Mixer):
         if self.paired and writes and x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16:
             from ..kernels import gemm_bf16
             qkv = gemm_bf16.try_linear_rope(x, w, ctx.positions, tables[0], tables[1], k_cache, v_cache,
-                                            cache.slot_mapping, cache.page_size, nh, nkv, hd)
+                                            cache.slot_mapping, cache.page_size, nh, nkv, hd,
+                                            tiled=self.w_qkv_tiled)
         if qkv is None:
             x = as_tensor(x)
         if qkv is not None:
@@ -157,7 +166,7 @@ class PagedAttention(Mixer):
                 self.position.apply(q, q[:, :0], ctx.positions)
         out = torch.empty((t, nh * hd), dtype=qkv.dtype, device=qkv.device)
         self.attend(qkv, k_cache, v_cache, out, ctx, cache)
-        return linear_delta(out, self.w_o, sink)
+        return linear_delta(out, self.w_o, sink, self.w_o_tiled)
 
     def attend(self, q, k_cache, v_cache, out, ctx, cache) -> None:
         if self.slopes is None and q.dtype is torch.bfloat16 and k_cache.dtype is torch.bfloat16:

@@ -140,9 +140,10 @@ class Norm(Part):
     # Optional: a norm may be *begun* by the kernel that makes its input rows and finished by the product that reads
     # them (``Begun``), which saves the norm's own launch where launches are what a step costs.
     # A norm that cannot says None, and the caller runs ``add_norm``.
-    def add_product(self, resid: torch.Tensor, x, w: torch.Tensor):
+    def add_product(self, resid: torch.Tensor, x, w: torch.Tensor, tiled=None):
         """``resid += x @ w^T`` in place with this norm of the new rows begun (``Begun``) or
-        finished (``parts.linear.Normed``); or None, nothing done."""
+        finished (``parts.linear.Normed``); or None, nothing done.  ``tiled`` is passed only by a part that keeps
+        a second copy of ``w`` in the order a few-row kernel reads it (``kernels.gemm_bf16.tile_weight_half``)."""
         return None
 
     def embed(self, table: torch.Tensor, tokens: torch.Tensor):

@@ -21,7 +21,7 @@ class SwiGLU(FeedForward):
         self.width, self.inter = int(width), int(intermediate)
         self.block = 0
         self.w_gate_up: Optional[torch.Tensor] = None
-        self.w_gate_up_tiled = None
+        self.w_gate_up_tiled = self.w_down_tiled = None
         self.w_down: Optional[torch.Tensor] = None
 
     def graph_safe(self) -> bool:
@@ -43,13 +43,14 @@ class SwiGLU(FeedForward):
         else:
             self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = get("down_proj.weight").to(device).contiguous()
-        # a second copy of the gate-up matrix in the order the streaming kernel's waves read it, for steps of few rows
-        self.w_gate_up_tiled = None
-        if self.block and act_dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16:
+        # second copies of the matrices in the order the streaming kernels' waves read them, for steps of few rows
+        self.w_gate_up_tiled = self.w_down_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16 and self.w_down.dtype is torch.bfloat16:
             from ..kernels import gemm_bf16
-            plan = gemm_bf16.tiled_plan(2 * self.inter, self.width, swiglu=True)
+            plan = gemm_bf16.tiled_plan(2 * self.inter, self.width, swiglu=True) if self.block else None
             if plan is not None:
                 self.w_gate_up_tiled = gemm_bf16.tile_weight(self.w_gate_up, *plan)
+            self.w_down_tiled = gemm_bf16.tile_weight_half(self.w_down)
 
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))
@@ -64,7 +65,7 @@ class SwiGLU(FeedForward):
             h = gemm_bf16.try_linear_swiglu(x, self.w_gate_up, self.w_gate_up_tiled)
         if h is None:
             h = ops.swiglu(linear(x, self.w_gate_up), block=self.block)
-        return linear_delta(h, self.w_down, sink)
+        return linear_delta(h, self.w_down, sink, self.w_down_tiled)
 
 
 register_feed_forward("swiglu", SwiGLU)

@@ -53,17 +53,20 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     return ops.gemm_generic(as_tensor(x), w, out_dtype, out)
 
 
-def linear_delta(x, w: torch.Tensor, sink: Optional[ResidualSink] = None):
+def linear_delta(x, w: torch.Tensor, sink: Optional[ResidualSink] = None, tiled=None):
     """A product whose result is only ever added to the residual stream.
 
     With a ``sink`` whose norm can, the product adds itself to the residual rows and begins that norm (few rows) or
     the norm follows at once (many rows): the result is then a ``Begun`` norm or a ``Normed`` one, not a delta, and
     the caller hands it on as it is.  Otherwise the delta comes back for
     ``Norm.add_norm``: for few rows as float32 planes [slices, M, N] of a K-split product, which ``add_norm`` sums
-    (the split keeps the whole GPU busy on a small product and costs no extra kernel).
+    (the split keeps the whole GPU busy on a small product and costs no extra kernel).  ``tiled``: a copy of ``w``
+    in the order the sink's few-row kernel reads it (``kernels.gemm_bf16.tile_weight_half``), if the part keeps one.
     """
     if sink is not None:
-        y = sink.norm.add_product(sink.resid, x, w)
+        # (a copy of w in the order its kernel reads it goes along only where the part has made one)
+        y = sink.norm.add_product(sink.resid, x, w) if tiled is None else \
+            sink.norm.add_product(sink.resid, x, w, tiled=tiled)
         if y is not None:
             return y
     x = as_tensor(x)

@@ -37,12 +37,12 @@ class RMSNorm(Norm):
 
     # the norm begun by its neighbours (bfloat16 steps of at most 16 rows): see kernels/gemm_bf16.py; with many rows
     # the library adds its product to the residual rows itself, and the norm reads them once
-    def add_product(self, resid, x, w):
+    def add_product(self, resid, x, w, tiled=None):
         if self.act_dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16:
             return None
         from ..kernels import gemm_bf16
         from .linear import Normed, as_tensor
-        y = gemm_bf16.try_linear_resid(x, w, resid, self.weight, self.eps)
+        y = gemm_bf16.try_linear_resid(x, w, resid, self.weight, self.eps, tiled)
         if y is not None:
             y.norm = self
             return y

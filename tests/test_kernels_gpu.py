@@ -587,6 +587,17 @@ def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k, planes, monkeypatch):
     kc1, vc1 = caches()
     q1 = gemm_bf16.try_linear_rope(x, w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv, hd, always=True)
     assert q1 is not None and tuple(q1.shape) == (m, nh * hd)
+    # over the copy of the weight in the order the kernel's waves read it: the same bits
+    tw = gemm_bf16.tile_weight_rope(w)
+    assert (tw is not None) == (k % 512 == 0 and n % 16 == 0)
+    if tw is not None and (m <= 8 or (m <= 16 and n < 5120)):
+        kc3, vc3 = caches()
+        with monkeypatch.context() as mp:
+            def row_major(*a):
+                raise AssertionError("the row-major kernel ran")
+            mp.setattr(gemm_bf16.lib(), "atoma_gemm_bf16_skinny_rope", row_major)
+            q3 = gemm_bf16.try_linear_rope(x, w, pos, cos, sin, kc3, vc3, slots, page, nh, nkv, hd, always=True, tiled=tw)
+        assert torch.equal(q3, q1) and torch.equal(kc3, kc1) and torch.equal(vc3, vc1)
     # apart, with float32 in between (the fused kernel rotates the float32 sums)
     kc2, vc2 = caches()
     qkv = ops.gemm_generic(x, w, torch.float32)
@@ -934,3 +945,35 @@ def test_swiglu_gemm_over_a_tiled_weight_equals_the_row_major_one(m, inter, k, r
     g, u = x.double().cpu() @ wg.double().cpu().T, x.double().cpu() @ wu.double().cpu().T
     ref = torch.nn.functional.silu(g) * u
     assert (got.double().cpu() - ref).abs().max() <= 1e-2 * ref.abs().max()
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 9, 16])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (72, 4096), (1000, 2048)])
+def test_residual_product_over_a_tiled_weight_equals_the_row_major_one(m, n, k):
+    """The product that adds into the residual rows and begins the next norm, over the copy of its weight laid out in
+    the order its waves read it (half tiles): the very bits of the row-major product, and the library's offsets are
+    where the Python tiling puts every element."""
+    from atoma_infer_amd.kernels import gemm_bf16
+    x = rnd(m, k, dtype=torch.bfloat16, seed=m)
+    w = rnd(n, k, dtype=torch.bfloat16, seed=n + k, scale=0.05)
+    gamma = (1 + 0.1 * rnd(n, dtype=torch.float32, seed=2)).bfloat16()
+    tw = gemm_bf16.tile_weight_half(w)
+    assert tw is not None and tw.data.numel() == n * k
+    off = gemm_bf16.lib().atoma_gemm_bf16_tiled_offset_half
+    off.restype = ctypes.c_longlong
+    g = torch.Generator().manual_seed(4)
+    for _ in range(50):
+        i, j = int(torch.randint(0, n, (1,), generator=g)), int(torch.randint(0, k, (1,), generator=g))
+        at = off(ctypes.c_longlong(i), ctypes.c_longlong(j), ctypes.c_longlong(n), ctypes.c_longlong(k), tw.wk, tw.u)
+        assert tw.data[at] == w[i, j], (i, j, at)
+    r0 = rnd(m, n, dtype=torch.float32, seed=9)
+    want_r, got_r = r0.clone(), r0.clone()
+    want = gemm_bf16.try_linear_resid(x, w, want_r, gamma, 1e-5)
+    got = gemm_bf16.try_linear_resid(x, w, got_r, gamma, 1e-5, tw)
+    assert want is not None and got is not None
+    assert torch.equal(got_r, want_r) and torch.equal(got.data, want.data) and torch.equal(got.shares, want.shares)
+    ref = r0.double().cpu() + x.double().cpu() @ w.double().cpu().T
+    assert (got_r.double().cpu() - ref).abs().max() <= 1e-2 * ref.abs().max()
+    # shapes that the half-tile plan does not take have no such copy
+    assert gemm_bf16.tile_weight_half(rnd(4096, 2048, dtype=torch.bfloat16)) is None
+    assert gemm_bf16.tile_weight_half(rnd(2048, 1024 + 512, dtype=torch.bfloat16)) is None
