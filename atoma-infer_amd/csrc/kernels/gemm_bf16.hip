@@ -604,9 +604,9 @@ static void resid_kernels(bool tiled, const void* a, const void* w, int M, int N
   hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN, WK, float, false, false, U, H, PACK_, TILED_>), grid, block, 0,    \
                      stream, (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0,         \
                      RopeArgs{}, fa)
-  if constexpr (H && WN == 1 && WK == 8 && U == 4) {
+  if constexpr (WN == 1 && WK == 8 && (U == 4 || U == 8)) {
     if (tiled) {
-      if (M <= 8) ATOMA_RESID_KERNEL(true, 1);
+      if (H && M <= 8) ATOMA_RESID_KERNEL(H, 1);
       else ATOMA_RESID_KERNEL(false, 1);
       return;
     }
@@ -620,8 +620,11 @@ static int launch_resid(const void* a, const void* w, bool tiled, int M, int N, 
                         int depth, int half, const float* ss_in, int parts_in, float eps_in, int width_in, float* resid,
                         const void* gamma, int gamma_dtype, void* u_out, float* ss_out, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  // the tiled layout (half tiles only: 8 rows x 64 values of K in the lanes' order, see atoma_gemm_bf16_tiled_offset_half)
-  if (tiled && (!half || wk != 8 || depth != 4 || (N & 7) || K % (64 * wk * depth))) return ATOMA_ERR_SHAPE;
+  // the tiled layout: eight waves a workgroup, batches of 4 or 8 steps; whole tiles (atoma_gemm_bf16_tiled_offset with
+  // one tile a wave) or half tiles (8 rows x 64 values of K in the lanes' order, atoma_gemm_bf16_tiled_offset_half)
+  if (tiled && (wk != 8 || (depth != 4 && depth != 8) || rt != 1 || N % (half ? 8 : 16) ||
+                K % ((half ? 64 : 32) * wk * depth)))
+    return ATOMA_ERR_SHAPE;
   if (M > 16 || K <= 0 || K % ((half ? 64 : 32) * wk) || (lda & 7) || (ldw & 7) || lda < K || ldw < K || (N & 3) ||
       ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || !resid || !gamma || !u_out || !ss_out ||
       ((uintptr_t)resid & 15) || ((uintptr_t)gamma & 15) || ((uintptr_t)u_out & 7) ||
@@ -663,13 +666,14 @@ extern "C" int atoma_gemm_bf16_skinny_resid(const void* a, const void* w, int M,
                       gamma, gamma_dtype, u_out, ss_out, stream);
 }
 
-// The same over a weight in the tiled layout of half tiles (eight waves a workgroup, batches of four steps).
+// The same over a weight in the tiled layout: eight waves a workgroup, one tile or half tile a wave, batches of
+// ``depth`` steps (4 or 8).
 extern "C" int atoma_gemm_bf16_skinny_resid_tiled(const void* a, const void* w_tiled, int M, int N, int K, int lda,
-                                                  const float* ss_in, int parts_in, float eps_in, int width_in,
-                                                  float* resid, const void* gamma, int gamma_dtype, void* u_out,
-                                                  float* ss_out, hipStream_t stream) {
-  return launch_resid(a, w_tiled, true, M, N, K, lda, K, 1, 8, 4, 1, ss_in, parts_in, eps_in, width_in, resid, gamma,
-                      gamma_dtype, u_out, ss_out, stream);
+                                                  int depth, int half, const float* ss_in, int parts_in, float eps_in,
+                                                  int width_in, float* resid, const void* gamma, int gamma_dtype,
+                                                  void* u_out, float* ss_out, hipStream_t stream) {
+  return launch_resid(a, w_tiled, true, M, N, K, lda, K, 1, 8, depth, half, ss_in, parts_in, eps_in, width_in, resid,
+                      gamma, gamma_dtype, u_out, ss_out, stream);
 }
 
 // Where element (row n, column k) of a weight [N, K] lies in the tiled layout of half tiles: tiles of 8 rows x 64

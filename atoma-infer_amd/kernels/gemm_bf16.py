@@ -118,11 +118,12 @@ TILED_SWIGLU_MAX_M = 64          # the fused SiLU-multiply reads the tiled copy 
 TILED_MIN_ELEMENTS = 1 << 24      # smaller weights stream at the same pace row-major (measured: 8 and 34 MB)
 
 
-def tile_weight(w: torch.Tensor, rt: int, wk: int) -> Optional[TiledWeight]:
+def tile_weight(w: torch.Tensor, rt: int, wk: int, u: int = 0) -> Optional[TiledWeight]:
     """The tiled copy of ``w`` [n, k] (bfloat16, row-major) for waves of ``rt`` tiles and ``wk`` waves a workgroup, or
-    None where the shape does not divide into whole batches of tiles."""
+    None where the shape does not divide into whole batches of tiles.  ``u``: steps a batch, for a kernel that does
+    not take the depth that goes with (rt, wk)."""
     n, k = w.shape
-    u = int(lib().atoma_gemm_bf16_batch_depth(1, rt, wk))
+    u = u or int(lib().atoma_gemm_bf16_batch_depth(1, rt, wk))
     if (w.dtype is not torch.bfloat16 or n % (16 * rt) or k % (32 * wk * u)
             or not w.is_contiguous()):
         return None
@@ -132,14 +133,18 @@ def tile_weight(w: torch.Tensor, rt: int, wk: int) -> Optional[TiledWeight]:
     return TiledWeight(t.view(-1), n, k, rt, wk, u)
 
 
-def tile_weight_half(w: torch.Tensor) -> Optional[TiledWeight]:
-    """The tiled copy of ``w`` [n, k] for the product that adds into the residual stream with half tiles (8 rows of
-    the weight a wave, eight waves a workgroup, batches of four steps of 64 values of K), or None where the shape
-    does not divide or ``resid_plan`` would not choose that plan."""
+def tile_weight_resid(w: torch.Tensor) -> Optional[TiledWeight]:
+    """The tiled copy of ``w`` [n, k] for the product that adds into the residual stream, in the plan that
+    ``resid_plan`` gives it: eight waves a workgroup and batches of 4 or 8 steps, of whole tiles or (``rt`` 0 in the
+    result) of half tiles, 8 rows of the weight and 64 values of K a wave and step.  None where the plan is another
+    or the shape does not divide."""
     n, k = w.shape
-    wk, u = 8, 4
-    if (w.dtype is not torch.bfloat16 or not w.is_contiguous() or n % 8 or k % (64 * wk * u)
-            or resid_plan(1, n, k) != (1, wk, u, 1)):
+    rt, wk, u, half = resid_plan(1, n, k)
+    if w.dtype is not torch.bfloat16 or not w.is_contiguous() or (rt, wk) != (1, 8) or u not in (4, 8):
+        return None
+    if not half:
+        return tile_weight(w, 1, wk, u)
+    if n % 8 or k % (64 * wk * u):
         return None
     t = w.view(n // 8, 8, wk, k // (64 * wk * u), u, 2, 4, 8)     # group, row, wave, batch, step, half, piece, value
     t = t.permute(3, 0, 2, 4, 6, 5, 1, 7).contiguous()            # batch, group, wave, step, piece, half, row, value
@@ -433,7 +438,7 @@ def try_linear_resid(x, w: torch.Tensor, resid: torch.Tensor, gamma: torch.Tenso
                      tiled: Optional[TiledWeight] = None) -> Optional[Begun]:
     """resid [M <= 16, N] float32 += x @ w^T in place, with the norm (gamma, eps) of the new rows begun: returns
     it as ``Begun``, or None (and nothing done) when the shape is not taken.  x may itself be ``Begun``.  ``tiled``:
-    the copy of ``w`` that ``tile_weight_half`` made, read in its place."""
+    the copy of ``w`` that ``tile_weight_resid`` made, read in its place."""
     begun = _begun_args(x)
     xd = x.data if isinstance(x, Begun) else x
     m, k = xd.shape
@@ -447,10 +452,10 @@ def try_linear_resid(x, w: torch.Tensor, resid: torch.Tensor, gamma: torch.Tenso
     u = torch.empty((m, n), dtype=torch.bfloat16, device=w.device)
     shares = torch.empty((parts, 16), dtype=torch.float32, device=w.device)
     code = F32 if gamma.dtype is torch.float32 else BF16
-    if tiled is not None and (tiled.n, tiled.k, tiled.rt) == (n, k, 0) and (rt, wk, depth, half) == (1, 8, 4, 1):
+    if tiled is not None and (tiled.n, tiled.k, tiled.rt, tiled.wk, tiled.u) == (n, k, 0 if half else rt, wk, depth):
         _check(lib().atoma_gemm_bf16_skinny_resid_tiled(_p(xd), _p(tiled.data), m, n, k, xd.stride(0) if m > 1 else k,
-                                                        *begun, _p(resid), _p(gamma), code, _p(u), _p(shares),
-                                                        _stream()), "gemm_bf16_skinny_resid_tiled")
+                                                        depth, half, *begun, _p(resid), _p(gamma), code, _p(u),
+                                                        _p(shares), _stream()), "gemm_bf16_skinny_resid_tiled")
         return Begun(u, shares, float(eps), n)
     _check(lib().atoma_gemm_bf16_skinny_resid(_p(xd), _p(w), m, n, k, xd.stride(0) if m > 1 else k, w.stride(0), rt, wk,
                                               depth, half, *begun, _p(resid), _p(gamma), code, _p(u), _p(shares), _stream()),

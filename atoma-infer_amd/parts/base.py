@@ -143,7 +143,7 @@ class Norm(Part):
     def add_product(self, resid: torch.Tensor, x, w: torch.Tensor, tiled=None):
         """``resid += x @ w^T`` in place with this norm of the new rows begun (``Begun``) or
         finished (``parts.linear.Normed``); or None, nothing done.  ``tiled`` is passed only by a part that keeps
-        a second copy of ``w`` in the order a few-row kernel reads it (``kernels.gemm_bf16.tile_weight_half``)."""
+        a second copy of ``w`` in the order a few-row kernel reads it (``kernels.gemm_bf16.tile_weight_resid``)."""
         return None
 
     def embed(self, table: torch.Tensor, tokens: torch.Tensor):

@@ -61,7 +61,7 @@ def linear_delta(x, w: torch.Tensor, sink: Optional[ResidualSink] = None, tiled=
     the caller hands it on as it is.  Otherwise the delta comes back for
     ``Norm.add_norm``: for few rows as float32 planes [slices, M, N] of a K-split product, which ``add_norm`` sums
     (the split keeps the whole GPU busy on a small product and costs no extra kernel).  ``tiled``: a copy of ``w``
-    in the order the sink's few-row kernel reads it (``kernels.gemm_bf16.tile_weight_half``), if the part keeps one.
+    in the order the sink's few-row kernel reads it (``kernels.gemm_bf16.tile_weight_resid``), if the part keeps one.
     """
     if sink is not None:
         # (a copy of w in the order its kernel reads it goes along only where the part has made one)

@@ -948,7 +948,8 @@ def test_swiglu_gemm_over_a_tiled_weight_equals_the_row_major_one(m, inter, k, r
 
 
 @pytest.mark.parametrize("m", [1, 5, 8, 9, 16])
-@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (72, 4096), (1000, 2048)])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (72, 4096), (1000, 2048), (4096, 2048), (3072, 8192),
+                                 (3072, 3072), (4096, 14336)])
 def test_residual_product_over_a_tiled_weight_equals_the_row_major_one(m, n, k):
     """The product that adds into the residual rows and begins the next norm, over the copy of its weight laid out in
     the order its waves read it (half tiles): the very bits of the row-major product, and the library's offsets are
@@ -957,14 +958,17 @@ def test_residual_product_over_a_tiled_weight_equals_the_row_major_one(m, n, k):
     x = rnd(m, k, dtype=torch.bfloat16, seed=m)
     w = rnd(n, k, dtype=torch.bfloat16, seed=n + k, scale=0.05)
     gamma = (1 + 0.1 * rnd(n, dtype=torch.float32, seed=2)).bfloat16()
-    tw = gemm_bf16.tile_weight_half(w)
+    tw = gemm_bf16.tile_weight_resid(w)
     assert tw is not None and tw.data.numel() == n * k
-    off = gemm_bf16.lib().atoma_gemm_bf16_tiled_offset_half
+    half = gemm_bf16.resid_plan(m, n, k)[3]
+    assert (tw.rt == 0) == bool(half) == (n <= 2048)
+    off = gemm_bf16.lib().atoma_gemm_bf16_tiled_offset_half if half else gemm_bf16.lib().atoma_gemm_bf16_tiled_offset
     off.restype = ctypes.c_longlong
     g = torch.Generator().manual_seed(4)
+    ll = ctypes.c_longlong
     for _ in range(50):
         i, j = int(torch.randint(0, n, (1,), generator=g)), int(torch.randint(0, k, (1,), generator=g))
-        at = off(ctypes.c_longlong(i), ctypes.c_longlong(j), ctypes.c_longlong(n), ctypes.c_longlong(k), tw.wk, tw.u)
+        at = off(ll(i), ll(j), ll(n), ll(k), tw.wk, tw.u) if half else off(ll(i), ll(j), ll(n), ll(k), 1, tw.wk, tw.u)
         assert tw.data[at] == w[i, j], (i, j, at)
     r0 = rnd(m, n, dtype=torch.float32, seed=9)
     want_r, got_r = r0.clone(), r0.clone()
@@ -974,6 +978,6 @@ def test_residual_product_over_a_tiled_weight_equals_the_row_major_one(m, n, k):
     assert torch.equal(got_r, want_r) and torch.equal(got.data, want.data) and torch.equal(got.shares, want.shares)
     ref = r0.double().cpu() + x.double().cpu() @ w.double().cpu().T
     assert (got_r.double().cpu() - ref).abs().max() <= 1e-2 * ref.abs().max()
-    # shapes that the half-tile plan does not take have no such copy
-    assert gemm_bf16.tile_weight_half(rnd(4096, 2048, dtype=torch.bfloat16)) is None
-    assert gemm_bf16.tile_weight_half(rnd(2048, 1024 + 512, dtype=torch.bfloat16)) is None
+    # shapes that do not divide into whole batches of the plan's tiles have no such copy
+    assert gemm_bf16.tile_weight_resid(rnd(2048, 1024 + 512, dtype=torch.bfloat16)) is None
+    assert gemm_bf16.tile_weight_resid(rnd(4096 + 8, 2048, dtype=torch.bfloat16)) is None
