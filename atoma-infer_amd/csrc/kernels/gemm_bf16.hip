@@ -153,8 +153,11 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   // reads those of RT / TILED neighbouring groups of the layout)
   constexpr int LRT = TILED ? TILED : 1;
   static_assert(RT % LRT == 0, "a wave covers whole groups of the layout");
-  const uint16_t* const wt = w + ((size_t)(blockIdx.x * (RT / LRT) * WK + wk) * U * LRT) * 512 + lane * 8;
-  const size_t wt_batch = (size_t)gridDim.x * WK * U * RT * 512;
+  // (with K split over the grid too, every slice of K counts as a wave of the layout: k_slices of them a group)
+  const uint16_t* const wt =
+      w + ((size_t)(blockIdx.x * (RT / LRT) * k_slices + blockIdx.y * WK + wk) * U * LRT) * 512 + lane * 8;
+  const size_t wt_batch = (size_t)gridDim.x * k_slices * U * RT * 512;
+  const size_t wt_group = (size_t)k_slices * U * LRT * 512;      // between the layout's groups that a wave covers
 
   f32x4 acc[RT][MT];
 #pragma unroll
@@ -198,7 +201,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
       for (int r = 0; r < RT; ++r) {
         if constexpr (TILED)
           wf[buf][u][r] = *reinterpret_cast<const bf16x8*>(wt + (size_t)(k0 / (KSTEP * U)) * wt_batch +
-                                                           ((r / LRT) * WK * U * LRT + u * LRT + r % LRT) * 512);
+                                                           (r / LRT) * wt_group + (u * LRT + r % LRT) * 512);
         else
           wf[buf][u][r] = *reinterpret_cast<const bf16x8*>(wp[r] + k0 + u * KSTEP);
       }
@@ -557,6 +560,37 @@ static int launch_swiglu_tiled(const void* a, const void* w_tiled, void* c, int 
 #undef ATOMA_SWIGLU_TILED
   ATOMA_LAUNCH_CHECK();
   return 0;
+}
+
+template <int MT, int RT>
+static int launch_tiled_planes(const void* a, const void* w_tiled, float* c, int M, int N, int K, int lda, int ldc,
+                               int slices, hipStream_t stream) {
+  dim3 grid(N / (16 * RT), slices);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, 1, 4, float, false, false, 0, false, false, RT>), grid, dim3(256), 0,
+                     stream, (const uint16_t*)a, (const uint16_t*)w_tiled, c, M, N, K, lda, K, ldc, (size_t)M * ldc,
+                     RopeArgs{}, FuseArgs{});
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// Float32 planes c [slices][M, N] of a product of 17 to 64 rows, K split over four waves a workgroup and ``slices``
+// ways over the grid, over a weight in the tiled layout made for waves of rt tiles (2 or 4) and 4 * slices slices of K.
+extern "C" int atoma_gemm_bf16_skinny_tiled_planes(const void* a, const void* w_tiled, float* c, int M, int N, int K,
+                                                   int lda, int ldc, int rt, int slices, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  static_assert(batch_depth(2, 2, 4) == 2 && batch_depth(4, 4, 4) == 2 && batch_depth(2, 4, 4) == 2 &&
+                batch_depth(4, 2, 4) == 2, "one layout for 17 to 64 rows");
+  if (M <= 16 || M > 64 || K <= 0 || (rt != 2 && rt != 4) || slices <= 0 || slices > 65535 || N % (16 * rt) ||
+      K % (32 * 4 * slices * 2) || (lda & 7) || lda < K || ldc < N || ((uintptr_t)a & 15) || ((uintptr_t)w_tiled & 15))
+    return ATOMA_ERR_SHAPE;
+  const int mt = (M + 15) / 16;
+#define ATOMA_PLANES(MT_)                                                                                             \
+  return rt == 2 ? launch_tiled_planes<MT_, 2>(a, w_tiled, c, M, N, K, lda, ldc, slices, stream)                     \
+                 : launch_tiled_planes<MT_, 4>(a, w_tiled, c, M, N, K, lda, ldc, slices, stream)
+  if (mt == 2) ATOMA_PLANES(2);
+  if (mt == 3) ATOMA_PLANES(3);
+  ATOMA_PLANES(4);
+#undef ATOMA_PLANES
 }
 
 // The gate-up product with SiLU(gate) * up in its epilogue over a weight in the tiled layout (gate and up rows

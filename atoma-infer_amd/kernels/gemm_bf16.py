@@ -112,6 +112,13 @@ class TiledWeight:
     u: int
 
 
+@dataclasses.dataclass
+class TiledCopies:
+    """The tiled copies of one weight: for steps of at most 16 rows, and for the K-split product of 17 to 64."""
+    few: Optional[TiledWeight] = None
+    many: Optional[TiledWeight] = None
+
+
 TILED_MAX_M = 16
 TILED_FOUR_TILES_MIN_M = 32
 TILED_SWIGLU_MAX_M = 64          # the fused SiLU-multiply reads the tiled copy with more rows too, in the copy's tiles
@@ -159,6 +166,18 @@ def tile_weight_rope(w: torch.Tensor) -> Optional[TiledWeight]:
     if wk != 4 or rt > 2:
         return None
     return tile_weight(w, rt, wk)
+
+
+def tile_copies_resid(w: torch.Tensor) -> Optional[TiledCopies]:
+    """The tiled copies of a weight whose product is added to the residual stream; None if there is none."""
+    c = TiledCopies(tile_weight_resid(w), tile_weight_planes(w))
+    return c if c.few is not None or c.many is not None else None
+
+
+def tile_copies_rope(w: torch.Tensor) -> Optional[TiledCopies]:
+    """The tiled copies of a fused q, k, v weight; None if there is none."""
+    c = TiledCopies(tile_weight_rope(w), tile_weight_planes(w))
+    return c if c.few is not None or c.many is not None else None
 
 
 def tiled_plan(n: int, k: int, swiglu: bool):
@@ -306,14 +325,30 @@ def try_addmm_resid(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor) -> bo
     return True
 
 
-def linear_planes(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
-    """For M <= 64: float32 planes [slices, M, N] whose sum is x @ w^T (K split over the grid), else None."""
+def tile_weight_planes(w: torch.Tensor) -> Optional[TiledWeight]:
+    """The tiled copy of ``w`` [n, k] for the K-split product of 17 to 64 rows (``linear_planes``; the plan is the same
+    for all of them): ``wk`` in the result counts the slices of K over workgroup and grid.  None where that plan has
+    no tiled kernel or the shape does not divide."""
+    n, k = w.shape
+    rt, wk, slices = _plan(SKINNY_MAX_M, n, k, True)
+    if wk != 4 or rt not in (2, 4) or slices < 2:
+        return None
+    return tile_weight(w, rt, wk * slices, 2)
+
+
+def linear_planes(x: torch.Tensor, w: torch.Tensor, tiled: Optional[TiledWeight] = None) -> Optional[torch.Tensor]:
+    """For M <= 64: float32 planes [slices, M, N] whose sum is x @ w^T (K split over the grid), else None.
+    ``tiled``: the copy of ``w`` that ``tile_weight_planes`` made, read in its place by 17 rows and more."""
     m, k = x.shape
     n = w.shape[0]
     if m > SKINNY_MAX_M or not skinny_ok(x, w):
         return None
     rt, wk, slices = _plan(m, n, k, True)
     out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+    if tiled is not None and m > 16 and (tiled.n, tiled.k, tiled.rt, tiled.wk, tiled.u) == (n, k, rt, wk * slices, 2):
+        _check(lib().atoma_gemm_bf16_skinny_tiled_planes(_p(x), _p(tiled.data), _p(out), m, n, k, x.stride(0), n, rt,
+                                                         slices, _stream()), "gemm_bf16_skinny_tiled_planes")
+        return out
     skinny(x, w, out, slices, rt, wk)
     return out
 
@@ -366,7 +401,7 @@ ROPE_PLANES_MIN_M = 40
 
 def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                     kcache: torch.Tensor, vcache: torch.Tensor, slot_mapping: torch.Tensor, page_size: int, nh: int,
-                    nkv: int, hd: int, always: bool = False, tiled: Optional[TiledWeight] = None,
+                    nkv: int, hd: int, always: bool = False, tiled: Optional[TiledCopies] = None,
                     ) -> Optional[torch.Tensor]:
     """The fused q, k, v projection with rotary encoding and the cache write in its epilogue, for few rows of x.
 
@@ -390,8 +425,7 @@ def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, c
         # the activations, not all of them), summed, rotated and stored by a second kernel
         rt, wk, slices = _plan(m, n, k, True)
         if slices > 1:
-            planes = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
-            skinny(x, w, planes, slices, rt, wk)
+            planes = linear_planes(x, w, tiled.many if tiled is not None else None)
             _check(lib().atoma_rope_from_planes(_p(planes), slices, m, _p(out), nh * hd, _p(positions), _p(cos), _p(sin),
                                                 _p(kcache), _p(vcache), _p(slot_mapping), int(page_size), nh, nkv, hd,
                                                 _stream()), "rope_from_planes")
@@ -401,8 +435,9 @@ def try_linear_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, c
         rt = 2
     if 8 < m <= 16 and rt == 1 and wk == 4 and n >= 5120:
         rt = 2          # (9 to 16 rows at Llama 3B's and 8B's sizes: 14.1 and 17.1 us against 15.3 and 18.9)
-    if tiled is not None and m <= TILED_MAX_M and (tiled.n, tiled.k, tiled.rt, tiled.wk) == (n, k, rt, wk):
-        _check(lib().atoma_gemm_bf16_skinny_rope_tiled(_p(x), _p(tiled.data), _p(out), m, k, x.stride(0) if m > 1 else k,
+    few = tiled.few if tiled is not None else None
+    if few is not None and m <= TILED_MAX_M and (few.n, few.k, few.rt, few.wk) == (n, k, rt, wk):
+        _check(lib().atoma_gemm_bf16_skinny_rope_tiled(_p(x), _p(few.data), _p(out), m, k, x.stride(0) if m > 1 else k,
                                                        nh * hd, rt, wk, _p(positions), _p(cos), _p(sin), _p(kcache),
                                                        _p(vcache), _p(slot_mapping), int(page_size), nh, nkv, hd, *begun,
                                                        _stream()), "gemm_bf16_skinny_rope_tiled")

@@ -87,8 +87,8 @@ class PagedAttention(Mixer):
         if act_dtype is torch.bfloat16 and self.w_qkv.dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
             from ..kernels import gemm_bf16
             if self.paired:
-                self.w_qkv_tiled = gemm_bf16.tile_weight_rope(self.w_qkv)
-            self.w_o_tiled = gemm_bf16.tile_weight_resid(self.w_o)
+                self.w_qkv_tiled = gemm_bf16.tile_copies_rope(self.w_qkv)
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
 
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))

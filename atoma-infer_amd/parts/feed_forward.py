@@ -50,7 +50,7 @@ class SwiGLU(FeedForward):
             plan = gemm_bf16.tiled_plan(2 * self.inter, self.width, swiglu=True) if self.block else None
             if plan is not None:
                 self.w_gate_up_tiled = gemm_bf16.tile_weight(self.w_gate_up, *plan)
-            self.w_down_tiled = gemm_bf16.tile_weight_resid(self.w_down)
+            self.w_down_tiled = gemm_bf16.tile_copies_resid(self.w_down)
 
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))

@@ -60,19 +60,19 @@ def linear_delta(x, w: torch.Tensor, sink: Optional[ResidualSink] = None, tiled=
     the norm follows at once (many rows): the result is then a ``Begun`` norm or a ``Normed`` one, not a delta, and
     the caller hands it on as it is.  Otherwise the delta comes back for
     ``Norm.add_norm``: for few rows as float32 planes [slices, M, N] of a K-split product, which ``add_norm`` sums
-    (the split keeps the whole GPU busy on a small product and costs no extra kernel).  ``tiled``: a copy of ``w``
-    in the order the sink's few-row kernel reads it (``kernels.gemm_bf16.tile_weight_resid``), if the part keeps one.
+    (the split keeps the whole GPU busy on a small product and costs no extra kernel).  ``tiled``: the copies of
+    ``w`` in the order the few-row kernels read it (``kernels.gemm_bf16.tile_copies_resid``), if the part keeps any.
     """
     if sink is not None:
         # (a copy of w in the order its kernel reads it goes along only where the part has made one)
-        y = sink.norm.add_product(sink.resid, x, w) if tiled is None else \
-            sink.norm.add_product(sink.resid, x, w, tiled=tiled)
+        y = sink.norm.add_product(sink.resid, x, w) if tiled is None or tiled.few is None else \
+            sink.norm.add_product(sink.resid, x, w, tiled=tiled.few)
         if y is not None:
             return y
     x = as_tensor(x)
     if x.dtype is torch.bfloat16 and w.dtype is torch.bfloat16:
         from ..kernels import gemm_bf16
-        y = gemm_bf16.linear_planes(x, w)
+        y = gemm_bf16.linear_planes(x, w, tiled.many if tiled is not None else None)
         if y is not None:
             return y
         # many rows: the library's product, its float32 sums handed to the residual stream unrounded, as the

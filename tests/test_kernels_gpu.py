@@ -588,14 +588,17 @@ def test_gemm_with_rotary_epilogue(m, nh, nkv, hd, k, planes, monkeypatch):
     q1 = gemm_bf16.try_linear_rope(x, w, pos, cos, sin, kc1, vc1, slots, page, nh, nkv, hd, always=True)
     assert q1 is not None and tuple(q1.shape) == (m, nh * hd)
     # over the copy of the weight in the order the kernel's waves read it: the same bits
-    tw = gemm_bf16.tile_weight_rope(w)
-    assert (tw is not None) == (k % 512 == 0 and n % 16 == 0)
-    if tw is not None and (m <= 8 or (m <= 16 and n < 5120)):
+    tw = gemm_bf16.tile_copies_rope(w)
+    assert (tw is not None and tw.few is not None) == (k % 512 == 0 and n % 16 == 0)
+    tiled_runs = tw is not None and ((tw.few is not None and (m <= 8 or (m <= 16 and n < 5120)))
+                                     or (tw.many is not None and planes))
+    if tiled_runs:
         kc3, vc3 = caches()
         with monkeypatch.context() as mp:
             def row_major(*a):
                 raise AssertionError("the row-major kernel ran")
             mp.setattr(gemm_bf16.lib(), "atoma_gemm_bf16_skinny_rope", row_major)
+            mp.setattr(gemm_bf16.lib(), "atoma_gemm_bf16_skinny", row_major)
             q3 = gemm_bf16.try_linear_rope(x, w, pos, cos, sin, kc3, vc3, slots, page, nh, nkv, hd, always=True, tiled=tw)
         assert torch.equal(q3, q1) and torch.equal(kc3, kc1) and torch.equal(vc3, vc1)
     # apart, with float32 in between (the fused kernel rotates the float32 sums)
@@ -981,3 +984,23 @@ def test_residual_product_over_a_tiled_weight_equals_the_row_major_one(m, n, k):
     # shapes that do not divide into whole batches of the plan's tiles have no such copy
     assert gemm_bf16.tile_weight_resid(rnd(2048, 1024 + 512, dtype=torch.bfloat16)) is None
     assert gemm_bf16.tile_weight_resid(rnd(4096 + 8, 2048, dtype=torch.bfloat16)) is None
+
+
+@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 8192), (3072, 2048), (4096, 4096), (4096, 14336), (96, 1024)])
+def test_planes_of_a_split_product_over_a_tiled_weight_equal_the_row_major_ones(n, k):
+    """17 to 64 rows: the float32 planes of the K-split product over the copy of the weight in the order its waves read
+    it (every slice of K, over workgroup and grid, a wave of the layout) are the very bits of the row-major planes."""
+    from atoma_infer_amd.kernels import gemm_bf16
+    w = rnd(n, k, dtype=torch.bfloat16, seed=n + k, scale=0.05)
+    tw = gemm_bf16.tile_weight_planes(w)
+    rt, wk, slices = gemm_bf16._plan(64, n, k, True)
+    assert tw is not None and (tw.rt, tw.wk, tw.u) == (rt, wk * slices, 2) and slices > 1
+    for m in (17, 32, 33, 48, 64):
+        x = rnd(m, k, dtype=torch.bfloat16, seed=m)
+        want = gemm_bf16.linear_planes(x, w)
+        got = gemm_bf16.linear_planes(x, w, tw)
+        assert want.shape == (slices, m, n) and torch.equal(got, want)
+        ref = x.double().cpu() @ w.double().cpu().T
+        assert (got.double().sum(0).cpu() - ref).abs().max() <= 1e-2 * ref.abs().max()
+    x = rnd(16, k, dtype=torch.bfloat16)
+    assert torch.equal(gemm_bf16.linear_planes(x, w, tw), gemm_bf16.linear_planes(x, w))     # (few rows: row-major)
