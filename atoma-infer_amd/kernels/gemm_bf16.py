@@ -119,6 +119,7 @@ class TiledCopies:
     many: Optional[TiledWeight] = None
 
 
+TILED_COPIES = True               # False: no part gets a tiled copy of a weight (half the memory, slower decode steps)
 TILED_MAX_M = 16
 TILED_FOUR_TILES_MIN_M = 32
 TILED_SWIGLU_MAX_M = 64          # the fused SiLU-multiply reads the tiled copy with more rows too, in the copy's tiles
@@ -131,7 +132,7 @@ def tile_weight(w: torch.Tensor, rt: int, wk: int, u: int = 0) -> Optional[Tiled
     not take the depth that goes with (rt, wk)."""
     n, k = w.shape
     u = u or int(lib().atoma_gemm_bf16_batch_depth(1, rt, wk))
-    if (w.dtype is not torch.bfloat16 or n % (16 * rt) or k % (32 * wk * u)
+    if (not TILED_COPIES or w.dtype is not torch.bfloat16 or n % (16 * rt) or k % (32 * wk * u)
             or not w.is_contiguous()):
         return None
     groups, batches = n // (16 * rt), k // (32 * wk * u)
@@ -151,7 +152,7 @@ def tile_weight_resid(w: torch.Tensor) -> Optional[TiledWeight]:
         return None
     if not half:
         return tile_weight(w, 1, wk, u)
-    if n % 8 or k % (64 * wk * u):
+    if not TILED_COPIES or n % 8 or k % (64 * wk * u):
         return None
     t = w.view(n // 8, 8, wk, k // (64 * wk * u), u, 2, 4, 8)     # group, row, wave, batch, step, half, piece, value
     t = t.permute(3, 0, 2, 4, 6, 5, 1, 7).contiguous()            # batch, group, wave, step, piece, half, row, value
