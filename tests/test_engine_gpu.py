@@ -372,7 +372,7 @@ LLAMA_8B_LAYER = dict(LLAMA_1B_LAYERS, hidden_size=4096, intermediate_size=14336
 
 
 @pytest.mark.parametrize("cfg", [LLAMA_1B_LAYERS, LLAMA_8B_LAYER], ids=["1b", "8b"])
-def test_layers_of_serving_size_in_mixed_steps(tmp_path, cfg):
+def test_layers_of_serving_size_in_mixed_steps(tmp_path, cfg, monkeypatch):
     """Layers with the sizes of Llama 3.2 1B (and its whole vocabulary) and of Llama 3.1 8B: at these widths the
     products take other plans (wider waves, K split over the grid, the library from 65 rows on) than any tiny
     configuration reaches."""
@@ -382,12 +382,32 @@ def test_layers_of_serving_size_in_mixed_steps(tmp_path, cfg):
     steps = [([("a", 200)], []), ([("a", 37), ("b", 50)], []), ([("a", 2), ("b", 1), ("c", 30)], [])]
     steps += [([("a", 1), ("b", 1), ("c", 1)], [])] * 3
     steps += [([("a", 58), ("b", 36)], ["a", "b", "c"])]
+    from atoma_infer_amd.kernels import gemm_bf16
     for dtype in DTYPES:
         runner = make_runner(model_dir, dtype, 16, 40)
         got = run_schedule(runner, requests, steps)
         assert len(got) == 300 + 90 + 33
         check_against_plain(model_dir, requests, got, dtype)
         assert runner.manager.num_free_pages() == 40
+        if dtype == "bfloat16":
+            # steps of few rows read copies of the weights in the order their kernels read them; without the copies
+            # the same steps give the same bits
+            block = runner.model.spec.layers[0][1]
+            copies = [block.mixer.w_qkv_tiled, block.mixer.w_o_tiled, block.feed_forward.w_gate_up_tiled,
+                      block.feed_forward.w_down_tiled]
+            if vocab % 32 == 0:             # (a vocabulary that does not divide into the kernel's tiles has no copy)
+                copies.append(runner.model.spec.head[1].tiled)
+            assert all(c is not None for c in copies), copies
+            del runner, block, copies
+            torch.cuda.empty_cache()
+            monkeypatch.setattr(gemm_bf16, "TILED_COPIES", False)
+            runner = make_runner(model_dir, dtype, 16, 40)
+            block = runner.model.spec.layers[0][1]
+            assert block.mixer.w_o_tiled is None and block.feed_forward.w_gate_up_tiled is None
+            plain_layout = run_schedule(runner, requests, steps)
+            monkeypatch.undo()
+            assert got.keys() == plain_layout.keys() and all(torch.equal(got[k], plain_layout[k]) for k in got)
+            del block
         del runner
         torch.cuda.empty_cache()
     _plain_cache.clear()
