@@ -73,6 +73,7 @@ class LlmEngine:
             pages = [min(p, cap) for p in pages]
         pool = CachePool(plan, page, pages, self.scheduler_config.max_num_sequences, cache_dtype, self.model.device)
         self.runner = ModelRunner(self.model, pool)
+        self.runner.external_fence = True       # the event behind a step's sampled tokens serves its staging buffer too
         self.scheduler = Scheduler(self.scheduler_config, RunnerCache(self.runner),
                                    chunk_alignment=spec.chunk_alignment)
         self.sampler = Sampler(self.model.device)
@@ -203,10 +204,15 @@ class LlmEngine:
         self.stats["steps"] += 1
         self.stats["tokens"] += plan.num_tokens
         flight = _InFlight(sampled, None, {r.uid: i for i, r in enumerate(sampled)}, False)
+        if not sampled:
+            fence = torch.cuda.Event()
+            fence.record()
+            self.runner.fence(fence)
         if sampled:
             flight.pending = self.sampler.launch(
                 logits, [r.plan for r in sampled], [r.num_sampled for r in sampled],
                 [r.all_ids() if r.plan.repetition_penalty != 1.0 else () for r in sampled])
+            self.runner.fence(flight.pending.event)       # (the step's staging buffer is free when the tokens are here)
             self.stats["sampled"] += len(sampled)
             limit = self.scheduler_config.max_model_len
             for r in sampled:

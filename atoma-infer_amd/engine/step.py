@@ -87,32 +87,61 @@ class StepContext:
 
 
 class _Staging:
-    """A pinned host buffer and its device twin, grown on demand."""
+    """Two pinned host buffers, taken in turn, and their one device twin, grown on demand.
+
+    A buffer may be written again when the copy out of it has been read, which an event behind that copy says.  The
+    event is the staging's own, or (``upload(record=False)``) one that the caller records later on the same stream
+    and names with ``mark``: with two buffers a caller that waits for a step's results before it builds the step
+    after the next never waits here, and a step needs no event beside the one its results have anyway.
+    """
 
     def __init__(self, device: torch.device):
         self.device = device
-        self.host: Optional[torch.Tensor] = None
+        self.hosts: List[Optional[torch.Tensor]] = [None, None]
+        self.events: List[Optional[torch.cuda.Event]] = [None, None]
+        self.unmarked = [False, False]        # a copy out of the buffer is on its way and no event marks its end
+        self.turn = 0
         self.dev: Optional[torch.Tensor] = None
-        self.pending: Optional[torch.cuda.Event] = None
 
-    def ensure(self, n: int) -> np.ndarray:
-        if self.host is None or self.host.numel() < n:
-            self.wait()
-            cap = max(1024, 1 << (n - 1).bit_length())
-            self.host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
-            self.dev = torch.empty(cap, dtype=torch.int32, device=self.device)
-        return self.host.numpy()
+    def _wait(self, i: int) -> None:
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+            self.events[i] = None
+        elif self.unmarked[i]:
+            torch.cuda.current_stream(self.device).synchronize()
+        self.unmarked[i] = False
+
+    def begin(self, n: int) -> np.ndarray:
+        """The next host buffer, at least ``n`` words long and free to be written."""
+        self.turn ^= 1
+        i = self.turn
+        self._wait(i)
+        if self.hosts[i] is None or self.hosts[i].numel() < n:
+            self.hosts[i] = torch.empty(max(1024, 1 << (n - 1).bit_length()), dtype=torch.int32, pin_memory=True)
+        if self.dev is None or self.dev.numel() < n:
+            self.dev = torch.empty(max(1024, 1 << (n - 1).bit_length()), dtype=torch.int32, device=self.device)
+        return self.hosts[i].numpy()
 
     def wait(self) -> None:
-        """The pinned buffer is reused by every step: wait until the last copy out of it has been read."""
-        if self.pending is not None:
-            self.pending.synchronize()
-            self.pending = None
+        """Wait until every copy out of the host buffers has been read."""
+        self._wait(0)
+        self._wait(1)
 
-    def upload(self, n: int) -> None:
-        self.dev[:n].copy_(self.host[:n], non_blocking=True)
-        self.pending = torch.cuda.Event()
-        self.pending.record()
+    def upload(self, n: int, record: bool = True) -> None:
+        """Copy the first ``n`` words of the buffer that ``begin`` gave to the device.  ``record``: mark the copy's end
+        with an event of its own; else the caller names one with ``mark`` (an event is a packet of its own in the
+        GPU's queue, 4 us on the path of every step, and a step that samples records one anyway)."""
+        i = self.turn
+        self.dev[:n].copy_(self.hosts[i][:n], non_blocking=True)
+        self.events[i], self.unmarked[i] = None, not record
+        if record:
+            self.events[i] = torch.cuda.Event()
+            self.events[i].record()
+
+    def mark(self, event: torch.cuda.Event) -> None:
+        """``event`` was recorded on the copies' stream behind the last ``upload(record=False)``."""
+        if self.unmarked[self.turn]:
+            self.events[self.turn] = event
 
 
 @dataclasses.dataclass
@@ -152,6 +181,10 @@ class ModelRunner:
         # decode steps are recorded into graphs only if every part of the model can be replayed
         self.use_graphs = use_graphs and model.spec.graph_safe()
         self._stage = _Staging(model.device)
+        self._last_stage: Optional[_Staging] = None
+        #: True: the caller records an event behind every step's work and hands it to ``fence``; the steps then record
+        #: none of their own (a step whose event never comes waits for the whole stream before its buffer is reused)
+        self.external_fence = False
         self._computed: Dict[int, int] = {}       # request -> tokens in the cache
         self._graphs: "OrderedDict[Tuple[int, int], _Graph]" = OrderedDict()
         # planners of the mixers, one per distinct key
@@ -269,8 +302,7 @@ class ModelRunner:
             total += (-total) % 4                  # every extra starts on a 16-byte boundary
             ex_off.append(total)
             total += arr.size
-        stage.wait()
-        buf = stage.ensure(total)
+        buf = stage.begin(total)
         # the arrays that depend on the entries alone are written by the host library in one call
         if t == s:
             tokens = np.fromiter((e.tokens[0] for e in entries), dtype=np.int32, count=s)
@@ -284,7 +316,8 @@ class ModelRunner:
         slots = buf[o_slot: o_slot + s].copy()
         for off, (_, arr, _) in zip(ex_off, extras):
             buf[off: off + arr.size] = arr.reshape(-1)
-        stage.upload(total)
+        stage.upload(total, record=not self.external_fence)
+        self._last_stage = stage
         dev = stage.dev
         if n_feed:
             from ..kernels import ops
@@ -363,6 +396,11 @@ class ModelRunner:
             g.graph, g.logits, g.ctx = graph, out, ctx
         g.graph.replay()
         return g.logits
+
+    def fence(self, event: torch.cuda.Event) -> None:
+        """With ``external_fence``: ``event`` was recorded on the step's stream behind the last step's work."""
+        if self._last_stage is not None:
+            self._last_stage.mark(event)
 
     def wait_staging(self):
         self._stage.wait()

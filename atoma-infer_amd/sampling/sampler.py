@@ -8,7 +8,7 @@ samples: backends/vllm/src/model_executor.rs:231-235, llm_engine.rs:379).
 """
 from __future__ import annotations
 
-from typing import List, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -31,20 +31,33 @@ def uniform(seed: int, counter: int) -> float:
 class Pending:
     """A sampling launched on the device whose tokens the host has not read yet."""
 
-    def __init__(self, tokens: torch.Tensor, logits: torch.Tensor, host: torch.Tensor, event: torch.cuda.Event):
-        self.tokens, self.logits, self._host, self._event = tokens, logits, host, event
+    def __init__(self, tokens: torch.Tensor, logits: torch.Tensor, host: torch.Tensor, event: torch.cuda.Event,
+                 pool: Optional[list] = None):
+        self.tokens, self.logits, self._host, self.event, self._pool = tokens, logits, host, event, pool
 
     def result(self) -> Tuple[List[int], List[float]]:
         """Wait for the copy and return (tokens, logits of the chosen tokens)."""
-        self._event.synchronize()
+        self.event.synchronize()
         n = self.tokens.numel()
-        return self._host[0, :n].view(torch.int32).tolist(), self._host[1, :n].tolist()
+        got = self._host[0, :n].view(torch.int32).tolist(), self._host[1, :n].tolist()
+        if self._pool is not None:            # the pinned buffer serves a later step
+            self._pool.append(self._host)
+            self._pool = None
+        return got
 
 
 class Sampler:
     def __init__(self, device: torch.device):
         self.device = device
         self._greedy_meta = {}        # rows -> the device copy of the parameters of that many greedy rows
+        # rows -> pinned buffers [2, rows] that have been read (a pinned tensor made and dropped every step costs an
+        # event in the GPU's queue when torch takes it back: 4 us a step)
+        self._host_pool = {}
+
+    def _host_buffer(self, s: int):
+        pool = self._host_pool.setdefault(s, [])
+        host = pool.pop() if pool else torch.empty((2, s), dtype=torch.float32, pin_memory=True)
+        return host, pool
 
     def launch(self, logits: torch.Tensor, plans: Sequence[SamplingPlan], steps: Sequence[int],
                contexts: Sequence[Sequence[int]]) -> Pending:
@@ -67,11 +80,11 @@ class Sampler:
         if all_greedy and s in self._greedy_meta:
             m = self._greedy_meta[s]
             out = ops.sample_packed(logits, m[0], m[4].view(torch.int32), m[1], m[2])
-            host = torch.empty((2, s), dtype=torch.float32, pin_memory=True)
+            host, pool = self._host_buffer(s)
             host.copy_(out, non_blocking=True)
             ev = torch.cuda.Event()
             ev.record()
-            return Pending(out[0].view(torch.int32), out[1], host, ev)
+            return Pending(out[0].view(torch.int32), out[1], host, ev, pool)
         # one packed upload: temperature, top_p, uniform, penalty (float32) and top_k (int32 bits)
         meta = torch.empty((5, s), dtype=torch.float32, pin_memory=True)
         mn = meta.numpy()
@@ -91,11 +104,11 @@ class Sampler:
             ops.repeat_penalty(logits, pen[0], pen[1], m[3])
         out = ops.sample_packed(logits, m[0], m[4].view(torch.int32), m[1], m[2])
         tok, lg = out[0].view(torch.int32), out[1]
-        host = torch.empty((2, s), dtype=torch.float32, pin_memory=True)
+        host, pool = self._host_buffer(s)
         host.copy_(out, non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
-        pending = Pending(tok, lg, host, ev)
+        pending = Pending(tok, lg, host, ev, pool)
         pending._meta = meta          # pinned memory must outlive the copy that reads it
         return pending
 
