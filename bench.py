@@ -264,7 +264,7 @@ def main() -> int:
     kv_bytes_per_token = plan_cache(model.spec).bytes_per_token(2)
 
     log(f"prefill of {args.prefill_tokens} tokens ...")
-    pre_s = prefill_run(model, args.prefill_tokens, 3, args.context)
+    pre_s = prefill_run(model, args.prefill_tokens, 8, args.context)
     c = model.config
     hd = c.head_size
     layer_params = (c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * hd

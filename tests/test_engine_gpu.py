@@ -338,6 +338,55 @@ def test_decode_graphs_replay_like_eager_steps(model_dirs, name, dtype):
     check_against_plain(model_dirs[name], {k: v for k, v in toks.items() if k != "c"}, got, dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["E", "LLAMA_1B"])
+def test_prompt_graphs_replay_like_eager_steps(model_dirs, tmp_path, name, dtype):
+    """A prompt (or a portion of one) alone in its step is recorded as a graph the third time its first position and
+    length are seen.  Every replay, with other tokens each time, is compared with the same step run eagerly, with
+    eager work and synchronisations between the replays (the library's products are part of such a graph: what they
+    record must replay right every time)."""
+    from atoma_infer_amd.engine import StepEntry
+    if name == "LLAMA_1B":
+        if dtype != "bfloat16":
+            pytest.skip("the serving sizes run in bfloat16")
+        model_dir = make_model_dir(str(tmp_path / "m"), LLAMA_1B_LAYERS, seed=4, dtype="bfloat16", norm_jitter=0.1)
+        vocab, page, first, second = LLAMA_1B_LAYERS["vocab_size"], 16, 2048, 700
+    else:
+        model_dir, vocab, page, first, second = model_dirs[name], TINY[name]["vocab_size"], PAGE[name], 300, 270
+    pages = -(-(first + second) // page) + 2
+    graphed = make_runner(model_dir, dtype, page, pages)
+    eager = make_runner(model_dir, dtype, page, pages)
+    eager.use_graphs = False
+    for rep in range(7):
+        toks = random_tokens(first + second, vocab, 900 + rep)
+        outs = []
+        for rn in (graphed, eager):
+            rn.add_request(rep)
+            a = rn.step([StepEntry(rep, toks[:first], 0, [first - 1])]).cpu()
+            if rep == 4:
+                torch.cuda.synchronize()
+            b = rn.step([StepEntry(rep, toks[first:first + second], first, [])])          # a portion that wants nothing
+            assert b is None
+            outs.append(a)
+            rn.free_request(rep)
+        assert torch.equal(outs[0], outs[1]), f"prompt {rep}"
+    keys = [k for k in graphed._graphs if k[0] == "prompt"]
+    assert ("prompt", 0, first, 1) in keys and ("prompt", first, second, 0) in keys
+    assert all(graphed._graphs[k].graph is not None for k in keys) and not eager._graphs
+    # what the second portion left in the cache is what an eager step leaves: decode on top of both
+    toks = random_tokens(first + second + 1, vocab, 77)
+    outs = []
+    for rn in (graphed, eager):
+        rn.add_request(99)
+        rn.step([StepEntry(99, toks[:first], 0, [first - 1])])
+        rn.step([StepEntry(99, toks[first:first + second], first, [])])
+        outs.append(rn.step([StepEntry(99, toks[first + second:], first + second, [0])]).cpu())
+        rn.free_request(99)
+    assert torch.equal(outs[0], outs[1])
+    if name == "E":
+        check_against_plain(model_dir, {"r": toks}, {("r", first + second): outs[0][0]}, dtype)
+
+
 def test_decoding_with_whole_key_ranges(model_dirs, monkeypatch):
     """Many decoding requests make every (request, KV head) pair one attention task for eight waves.  Here the
     threshold is lowered so that three requests do it: decoded through graphs, against the plain model."""
