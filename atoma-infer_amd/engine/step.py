@@ -29,6 +29,7 @@ from ..cache.pool import CachePool, LayerCache
 
 DECODE_BUCKET = 256      # tokens; a decode graph serves contexts up to a multiple of this
 MAX_GRAPHS = 48
+MAX_SEEN = 1024          # shapes of steps whose sightings are counted before they are recorded
 # A step that is one prompt, or one portion of a prompt, of at least this many tokens is recorded as a graph too, the
 # third time its (first position, length) is seen: its 150 launches then cost the GPU about 0.2 ms less
 PROMPT_GRAPH_MIN_TOKENS = 256
@@ -154,7 +155,6 @@ class _Graph:
     graph: Optional[torch.cuda.CUDAGraph] = None
     logits: Optional[torch.Tensor] = None
     ctx: Optional[StepContext] = None
-    seen: int = 0
 
 
 class RunnerCache:
@@ -193,6 +193,7 @@ class ModelRunner:
         self.external_fence = False
         self._computed: Dict[int, int] = {}       # request -> tokens in the cache
         self._graphs: "OrderedDict[Tuple[int, int], _Graph]" = OrderedDict()
+        self._seen: "OrderedDict[tuple, int]" = OrderedDict()
         # planners of the mixers, one per distinct key
         self._planners: Dict[object, Callable] = {}
         for _, block in model.spec.layers:
@@ -395,13 +396,17 @@ class ModelRunner:
         key (the earlier ones run eagerly, which also loads every kernel the step needs), replayed from then on."""
         g = self._graphs.get(key)
         if g is None:
+            # (shapes that have not been seen often enough are counted apart: they must not push recorded graphs out)
+            seen = self._seen.pop(key, 0) + 1
+            if seen < sightings:
+                self._seen[key] = seen
+                while len(self._seen) > MAX_SEEN:
+                    self._seen.popitem(last=False)
+                return False, None
             g = self._graphs[key] = _Graph(_Staging(self.model.device))
             while len(self._graphs) > MAX_GRAPHS:
                 self._graphs.popitem(last=False)
         self._graphs.move_to_end(key)
-        g.seen += 1
-        if g.graph is None and g.seen < sightings:
-            return False, None
         ctx = self._build(entries, g.stage, bucket, feed_src, arrays)
         if g.graph is None:
             torch.cuda.synchronize()
