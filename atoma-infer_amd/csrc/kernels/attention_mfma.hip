@@ -176,11 +176,14 @@ __device__ __forceinline__ void merge_parts(const float* __restrict__ part_o, co
 // long, fill the GPU worse.  The host asks for two pieces from 16,384 keys on.
 template <int TASKS, int KSPLIT, int RT = 1>
 __global__ void __launch_bounds__(64 * TASKS * KSPLIT)
-attention_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ kcache,
-                      const uint16_t* __restrict__ vcache, uint16_t* __restrict__ out, int out_stride,
-                      float* __restrict__ part_o, float* __restrict__ part_lse, const Task* __restrict__ tasks,
-                      int n_tasks, const int32_t* __restrict__ block_tables, int max_blocks, float scale,
-                      int window, int nh, int nkv, int32_t* __restrict__ counters) {
+attention_mfma_kernel(const Task* __restrict__ tasks, int n_tasks, int nkv, const uint16_t* __restrict__ q,
+                      int q_stride, int nh, const int32_t* __restrict__ block_tables, int max_blocks, int window,
+                      const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
+                      uint16_t* __restrict__ out, int out_stride, float* __restrict__ part_o,
+                      float* __restrict__ part_lse, float scale, int32_t* __restrict__ counters) {
+  // (the arguments come in the order in which a wave needs them: the first fourteen words, up to kcache, are in
+  // scalar registers when the wave starts, the others are fetched from memory, a trip that the task record, the
+  // queries, the page numbers and the first keys need not wait for)
   // (a wave's number is the same in all its lanes; saying so keeps what follows from it in scalar registers)
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave % TASKS, part = wave / TASKS;   // which of the workgroup's tasks, which share of its keys
@@ -682,9 +685,9 @@ extern "C" int atoma_attention_mfma(const void* q, int q_stride, const void* kca
     if (rc_lds != 0) return rc_lds;                                                                                \
     hipLaunchKernelGGL((attention_mfma_kernel<T, KS, ##__VA_ARGS__>), dim3(((n_tasks + T - 1) / T) * nkv),        \
                        dim3(64 * T * KS), BYTES,                                                                   \
-                       stream, (const uint16_t*)q, q_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,     \
-                       (uint16_t*)out, out_stride, part_o, part_lse, t, n_tasks, block_tables, max_blocks, scale,  \
-                       window, nh, nkv, counters);                                                                 \
+                       stream, t, n_tasks, nkv, (const uint16_t*)q, q_stride, nh, block_tables, max_blocks,        \
+                       window, (const uint16_t*)kcache, (const uint16_t*)vcache, (uint16_t*)out, out_stride,       \
+                       part_o, part_lse, scale, counters);                                                         \
   } while (0)
   if (ksplit == 1) ATOMA_ATTN(4, 1, 0);
   else if (ksplit == 2 && row_tiles == 2) ATOMA_ATTN(4, 2, 2 * kMerge2Bytes, (kTwoPieces ? 2 : 1));

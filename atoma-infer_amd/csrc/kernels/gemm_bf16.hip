@@ -110,11 +110,50 @@ struct FuseArgs {
 // about the same pace, so at any moment the loads in flight cover one stretch of memory that moves from the front of
 // the matrix to its back, as a plain streaming read does, where row-major rows have every wave fetch 64-byte
 // pieces 2 * K bytes apart (loads alone, the gate-up matrix of Llama 1B: 11.5 against 13.3 us).
+// The arguments of gemm_skinny_kernel behind k_len as they lie in its argument segment (the layout of a C struct of
+// the parameters in their order): three pointers and eight ints lie before them.
+struct SkinnyLateArgs {
+  size_t plane;
+  RopeArgs ra;
+  FuseArgs fa;
+};
+constexpr int kSkinnyLateArgsOffset = 3 * 8 + 8 * 4;
+static_assert(kSkinnyLateArgsOffset % alignof(SkinnyLateArgs) == 0, "plane follows k_len without padding");
+
 template <int MT, int RT, int WN, int WK, typename TC, bool SWIGLU = false, bool ROPE = false, int UO = 0,
           bool HALF = false, bool PACK = false, int TILED = 0>
 __global__ void __launch_bounds__(64 * WN * WK)
 gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, TC* __restrict__ c, int M, int N,
-                   int K, int lda, int ldw, int ldc, size_t plane, RopeArgs ra, FuseArgs fa) {
+                   int K, int lda, int ldw, int ldc, int grid_slices, int k_len, size_t plane_arg, RopeArgs ra_arg,
+                   FuseArgs fa_arg) {
+  // (The first arguments, up to grid_slices, are what a wave needs for the addresses of its first loads: the module
+  // is compiled so that they are in scalar registers when the wave starts, where the others, and the grid's sizes,
+  // are fetched from memory, a trip of its own that the first loads must not wait for.  Hence grid_slices, which
+  // says what gridDim.y would, k_len = K / (grid_slices * WK), the values of K that a wave walks (a division less on
+  // the way to the first load), and no use of gridDim.  The later arguments are not taken from the parameters, which
+  // the compiler fetches at the kernel's entry (into scalar registers that it then wants for something else, so
+  // that it waits for them after all), but read from the argument segment by fetch_late_args() below, behind the
+  // first loads.)
+  size_t plane = 0;
+  RopeArgs ra;
+  FuseArgs fa;
+  auto fetch_late_args = [&]() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef const __attribute__((address_space(4))) char* seg_bytes;
+    typedef const __attribute__((address_space(4))) SkinnyLateArgs* seg_late;
+    const seg_late seg = (seg_late)((seg_bytes)__builtin_amdgcn_kernarg_segment_ptr() + kSkinnyLateArgsOffset);
+    plane = seg->plane;
+    ra.positions = seg->ra.positions, ra.cos_t = seg->ra.cos_t, ra.sin_t = seg->ra.sin_t;
+    ra.kcache = seg->ra.kcache, ra.vcache = seg->ra.vcache, ra.slot_mapping = seg->ra.slot_mapping;
+    ra.page_size = seg->ra.page_size, ra.nh = seg->ra.nh, ra.nkv = seg->ra.nkv, ra.hd = seg->ra.hd;
+    fa.ss_in = seg->fa.ss_in, fa.parts_in = seg->fa.parts_in, fa.eps_in = seg->fa.eps_in;
+    fa.inv_width_in = seg->fa.inv_width_in, fa.resid = seg->fa.resid, fa.gamma = seg->fa.gamma;
+    fa.gamma_is_bf16 = seg->fa.gamma_is_bf16, fa.u_out = seg->fa.u_out, fa.ss_out = seg->fa.ss_out;
+#else
+    plane = plane_arg, ra = ra_arg, fa = fa_arg;
+#endif
+  };
+  (void)plane_arg, (void)ra_arg, (void)fa_arg;
   // loads of U steps of K are issued together before their MFMAs, so that a wave keeps U * (RT + MT) 16-byte
   // loads per lane in flight: the product is bound by memory latency and bandwidth, not by arithmetic
   // (eight waves of many tiles have 256 registers each: one step)
@@ -128,8 +167,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
                 "the tiled layout: K split over a workgroup's waves");
   const int n_base = (blockIdx.x * WN + wn) * (HALF ? 8 : RT * 16);
   constexpr int KSTEP = HALF ? 64 : 32;               // values of K that a wave's step covers
-  const int k_slices = gridDim.y * WK;
-  const int k_len = K / k_slices;
+  const int k_slices = grid_slices * WK;
   const int k_begin = (blockIdx.y * WK + wk) * k_len;
 
   // row pointers; rows past the end are clamped to the last valid row and never stored
@@ -156,7 +194,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   // (with K split over the grid too, every slice of K counts as a wave of the layout: k_slices of them a group)
   const uint16_t* const wt =
       w + ((size_t)(blockIdx.x * (RT / LRT) * k_slices + blockIdx.y * WK + wk) * U * LRT) * 512 + lane * 8;
-  const size_t wt_batch = (size_t)gridDim.x * k_slices * U * RT * 512;
+  const size_t wt_batch = (size_t)(N / (HALF ? 8 : 16 * RT)) * k_slices * U * RT * 512;   // (groups of the layout)
   const size_t wt_group = (size_t)k_slices * U * LRT * 512;      // between the layout's groups that a wave covers
 
   f32x4 acc[RT][MT];
@@ -171,26 +209,29 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   // and meet in LDS (behind the barrier that the K-split needs anyway).  They are asked for after the first loads
   // of the weight (below) and added after the last MFMA, so that nothing waits for them.
   __shared__ float ss_red[WN * WK][16];
-  const bool scaled = MT == 1 && fa.ss_in != nullptr;
+  // (fa lives in the later arguments: nothing may ask for it before the first loads of the weight are on their way)
+  auto is_scaled = [&]() { return MT == 1 && fa.ss_in != nullptr; };
   constexpr int SS_STRIDE = 4 * WN * WK;
   float ss_v[16];
   auto load_shares = [&]() {
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const int p = wave * 4 + kg + j * SS_STRIDE;
-      ss_v[j] = (scaled && p < fa.parts_in) ? fa.ss_in[p * 16 + r16] : 0.f;
+      ss_v[j] = (is_scaled() && p < fa.parts_in) ? fa.ss_in[p * 16 + r16] : 0.f;
     }
   };
   f32x4 res_in[RT];
-  if (MT == 1 && fa.resid != nullptr && wk == 0) {
+  auto load_resid = [&]() {
+    if (MT == 1 && fa.resid != nullptr && wk == 0) {
 #pragma unroll
-    for (int r = 0; r < RT; ++r) {
-      const int n0 = n_base + r * 16 + kg * 4;
-      res_in[r] = (r16 < M && n0 + 3 < N && (!HALF || kg < 2))
-                      ? *reinterpret_cast<const f32x4*>(fa.resid + (size_t)r16 * N + n0)
-                      : f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int r = 0; r < RT; ++r) {
+        const int n0 = n_base + r * 16 + kg * 4;
+        res_in[r] = (r16 < M && n0 + 3 < N && (!HALF || kg < 2))
+                        ? *reinterpret_cast<const f32x4*>(fa.resid + (size_t)r16 * N + n0)
+                        : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
     }
-  }
+  };
 
   // two buffers of U steps each: while the MFMAs of one run, the loads of the other are in flight
   bf16x8 wf[2][U][RT], af[2][U][MT], af_hi[2][U];
@@ -227,6 +268,9 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   int k = 0;
   if (n_batches > 0) {
     load(0, 0);
+    __builtin_amdgcn_sched_barrier(0);      // (what follows needs the later arguments: behind the first loads)
+    fetch_late_args();
+    load_resid();
     if constexpr (MT == 1) load_shares();
     int b = 0;
     for (; b + 2 <= n_batches; b += 2) {
@@ -237,6 +281,10 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
     }
     if (b < n_batches) multiply(0);
     k = n_batches * STEP;
+  }
+  if (n_batches <= 0) {
+    fetch_late_args();
+    load_resid();
   }
   for (; k < k_len; k += KSTEP) {
     bf16x8 wt[RT], at[MT];
@@ -268,7 +316,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
     }
   }
 
-  if (scaled) {
+  if (is_scaled()) {
     if (n_batches <= 0) load_shares();
     float ss_mine = 0.f;
 #pragma unroll
@@ -308,7 +356,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   }
 
   if constexpr (MT == 1) {
-    if (scaled) {
+    if (is_scaled()) {
       float t = 0.f;
 #pragma unroll
       for (int i = 0; i < WN * WK; ++i) t += ss_red[i][r16];
@@ -435,10 +483,10 @@ static int launch(const void* a, const void* w, void* c, int c_dtype, int M, int
   const size_t plane = (size_t)M * ldc;
   if (c_dtype == kF32)
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, float>), grid, block, 0, stream, (const uint16_t*)a,
-                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, plane, RopeArgs{}, fa);
+                       (const uint16_t*)w, (float*)c, M, N, K, lda, ldw, ldc, slices, K / (slices * WK), plane, RopeArgs{}, fa);
   else if (c_dtype == kBF16)
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t>), grid, block, 0, stream, (const uint16_t*)a,
-                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, plane, RopeArgs{}, fa);
+                       (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, slices, K / (slices * WK), plane, RopeArgs{}, fa);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();
@@ -532,7 +580,7 @@ extern "C" int atoma_gemm_bf16_skinny_tiled(const void* a, const void* w_tiled, 
   do {                                                                                                               \
     hipLaunchKernelGGL((gemm_skinny_kernel<1, R, 1, WK_, TC_, false, false, 0, false, false, R>), grid,              \
                        dim3(64 * WK_), 0, stream, (const uint16_t*)a, (const uint16_t*)w_tiled, (TC_*)c, M, N, K,    \
-                       lda, K, ldc, (size_t)0, RopeArgs{}, fa);                                                      \
+                       lda, K, ldc, 1, K / WK_, (size_t)0, RopeArgs{}, fa);                                             \
     ATOMA_LAUNCH_CHECK();                                                                                            \
     return 0;                                                                                                        \
   } while (0)
@@ -552,7 +600,7 @@ static int launch_swiglu_tiled(const void* a, const void* w_tiled, void* c, int 
 #define ATOMA_SWIGLU_TILED(R, L)                                                                                      \
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, R, 1, 4, bf16_t, true, false, 0, false, false, L>), grid, dim3(256), 0,  \
                      stream, (const uint16_t*)a, (const uint16_t*)w_tiled, (bf16_t*)c, M, N, K, lda, K, ldc,         \
-                     (size_t)0, RopeArgs{}, fa)
+                     1, K / 4, (size_t)0, RopeArgs{}, fa)
   if (rt == 2 && layout_rt == 2) ATOMA_SWIGLU_TILED(2, 2);
   else if (rt == 4 && layout_rt == 2) ATOMA_SWIGLU_TILED(4, 2);
   else if (rt == 4 && layout_rt == 4) ATOMA_SWIGLU_TILED(4, 4);
@@ -567,7 +615,7 @@ static int launch_tiled_planes(const void* a, const void* w_tiled, float* c, int
                                int slices, hipStream_t stream) {
   dim3 grid(N / (16 * RT), slices);
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, 1, 4, float, false, false, 0, false, false, RT>), grid, dim3(256), 0,
-                     stream, (const uint16_t*)a, (const uint16_t*)w_tiled, c, M, N, K, lda, K, ldc, (size_t)M * ldc,
+                     stream, (const uint16_t*)a, (const uint16_t*)w_tiled, c, M, N, K, lda, K, ldc, slices, K / (slices * 4), (size_t)M * ldc,
                      RopeArgs{}, FuseArgs{});
   ATOMA_LAUNCH_CHECK();
   return 0;
@@ -636,8 +684,8 @@ static void resid_kernels(bool tiled, const void* a, const void* w, int M, int N
   dim3 grid((N + cols - 1) / cols, 1), block(64 * WN * WK);
 #define ATOMA_RESID_KERNEL(PACK_, TILED_)                                                                             \
   hipLaunchKernelGGL((gemm_skinny_kernel<1, R, WN, WK, float, false, false, U, H, PACK_, TILED_>), grid, block, 0,    \
-                     stream, (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, (size_t)0,         \
-                     RopeArgs{}, fa)
+                     stream, (const uint16_t*)a, (const uint16_t*)w, resid, M, N, K, lda, ldw, N, 1, K / WK,          \
+                     (size_t)0, RopeArgs{}, fa)
   if constexpr (WN == 1 && WK == 8 && (U == 4 || U == 8)) {
     if (tiled) {
       if (H && M <= 8) ATOMA_RESID_KERNEL(H, 1);
@@ -726,7 +774,7 @@ static int launch_swiglu(const void* a, const void* w, void* c, int M, int N, in
                          const FuseArgs& fa, hipStream_t stream) {
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, true>), grid, block, 0, stream, (const uint16_t*)a,
-                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, RopeArgs{}, fa);
+                     (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, 1, K / WK, (size_t)0, RopeArgs{}, fa);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
@@ -768,7 +816,7 @@ static int launch_rope(const void* a, const void* w, void* c, int M, int N, int 
                        const RopeArgs& ra, const FuseArgs& fa, hipStream_t stream) {
   dim3 grid((N + WN * RT * 16 - 1) / (WN * RT * 16), 1), block(64 * WN * WK);
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, WN, WK, bf16_t, false, true, 0, false, false, TILED>), grid, block, 0, stream,
-                     (const uint16_t*)a, (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, (size_t)0, ra, fa);
+                     (const uint16_t*)a, (const uint16_t*)w, (bf16_t*)c, M, N, K, lda, ldw, ldc, 1, K / WK, (size_t)0, ra, fa);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }

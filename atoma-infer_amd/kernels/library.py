@@ -31,8 +31,11 @@ _KERNELS = os.path.join(_CSRC, "kernels")
 _HOST = os.path.join(_CSRC, "host")
 
 GPU_ARCH = "gfx950"
+# (kernarg preload: the first 14 words of a kernel's arguments are in scalar registers when a wave starts, where the
+# others are fetched from memory; the kernels order their arguments for it)
 HIP_FLAGS = ["--offload-arch=" + GPU_ARCH, "-O3", "-std=c++17", "-fPIC",
-             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+             "-mllvm", "-amdgpu-kernarg-preload-count=14"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
 
 
