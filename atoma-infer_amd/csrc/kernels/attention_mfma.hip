@@ -198,6 +198,9 @@ attention_mfma_kernel(const Task* __restrict__ tasks, int n_tasks, int nkv, cons
   // (one load of the record: an empty one has an empty key range of its own)
   const Task task = tasks[ti < n_tasks ? ti : 0];
   const bool has_task = ti < n_tasks && task.entry >= 0;
+  // (the record of the row piece that a chunk belongs to, for the wave that will merge the piece's chunks: asked for
+  // now, it is a trip to memory less behind the last chunk)
+  const Task comb = tasks[(has_task && task.dest >= 0 && counters != nullptr) ? n_tasks + task.n_parts : 0];
   if (KSPLIT == 1 && !has_task) return;
   const int g = nh / nkv;
   const int c = lane & 31, hg = lane >> 5;
@@ -519,7 +522,6 @@ attention_mfma_kernel(const Task* __restrict__ tasks, int n_tasks, int nkv, cons
       // (stores and loads that pass the L2 of this wave's XCD, which other XCDs do not see), this wave's stores have
       // arrived before it counts itself in, and the counter is a device-wide atomic: no fence that would write back or
       // invalidate a whole cache is needed.  The parts are added in the order of their index, whoever comes last.
-      const Task comb = tasks[n_tasks + task.n_parts];
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __builtin_amdgcn_s_waitcnt(0);
       int32_t* counter = counters + (size_t)task.n_parts * nkv + kvh;
@@ -529,7 +531,7 @@ attention_mfma_kernel(const Task* __restrict__ tasks, int n_tasks, int nkv, cons
       if (before + 1 == comb.n_parts) {
         if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         // (a wave a task: the launches of decoded tokens alone, which have registers to spare)
-        merge_parts<(KSPLIT == 1 ? 16 : 8)>(part_o, part_lse, out, out_stride, comb, kvh, nh, nkv, lane);
+        merge_parts<(KSPLIT == 1 ? 16 : 12)>(part_o, part_lse, out, out_stride, comb, kvh, nh, nkv, lane);
       }
     }
   }
