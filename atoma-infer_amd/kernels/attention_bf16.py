@@ -88,17 +88,57 @@ WHOLE_SHORT_WALKS = ((96, 8192 * 64), (32, 1536 * 64), (1, 1024 * 64))
 LONG_KEYS = 16384
 
 
-# Contexts up to which the chunks of a row piece are merged by the attention kernel itself (the wave that finishes the
-# last chunk does it; at most 18 chunks then): measured on MI355X, 0.5 to 1 us quicker than the merging kernel at
-# 1,024 keys and equal at 2,048 for the pair alone, and 10 to 27 us quicker over the 16 layers of a decode step of 8
-# requests or of 1; from 4,096 keys on one wave's walk over the parts costs more than the second launch.
+# Contexts up to which the chunks of a row piece are merged by the attention kernel itself whatever the plan (the wave
+# that finishes the last chunk does it; at most 18 chunks then): measured on MI355X, 0.5 to 1 us quicker than the
+# merging kernel at 1,024 keys and equal at 2,048 for the pair alone, and 10 to 27 us quicker over the 16 layers of a
+# decode step of 8 requests or of 1.  Beyond, the kernel merges where four waves share a chunk (decode steps, see
+# ``chunk_for``: the chunks grow with the context, so the parts stay few); other plans leave the parts to the merging
+# kernel, since one wave's walk over many parts costs more than the second launch.
 MERGE_MAX_KEYS = 2304
 MERGE_WHOLE_MAX_KEYS = 512    # with the merge in the kernel: whole ranges for few pairs only up to this many keys
+MERGE_MAX_PARTS = 48          # of a row piece, where the chunks grow with the context
+# (pairs from, keys beyond) which whole ranges serve such contexts at head sizes up to 64
+LONG_WHOLE_PAIRS = ((512, 0), (192, 6144), (WHOLE_MIN_PAIRS, 24576))
 MERGE_IN_KERNEL = True        # False: always the merging kernel (tests run both)
 
 
-def merges_in_kernel(max_keys: int) -> bool:
-    return MERGE_IN_KERNEL and max_keys <= MERGE_MAX_KEYS
+def merges_in_kernel(max_keys: int, waves: int = 1) -> bool:
+    return MERGE_IN_KERNEL and (max_keys <= MERGE_MAX_KEYS or waves == 4)
+
+
+def _long_decode_plan(pairs: int, tasks: int, max_keys: int, head_size: int) -> Optional[Tuple[int, int]]:
+    """``chunk_for`` for decode steps beyond ``MERGE_MAX_KEYS`` keys whose chunks the attention kernel merges itself:
+    four waves a chunk, and chunks so long that the launch has about 256 tasks, one workgroup a CU.  Measured over the
+    layers of a decode step on MI355X (forward graph, 1 to 64 requests of 3,072 to 32,768 keys; 16 layers of Llama
+    1B, head size 64, and 8 layers of Llama 8B, head size 128; ``tasks`` counts 256-key chunks over all KV heads):
+    up to 384 tasks 256-key chunks, up to 768 512, up to 1,536 1,024, up to 2,560 2,048 (head size 64, against
+    chunks walked by two waves and the merging kernel: one request of 4,096 keys 744 against 796 us, eight 933 against
+    968, eight of 8,192 keys 1,135 against 1,226, one of 32,768 keys 925 against 997; head size 128: 1.5 to 6 %);
+    more tasks want 1,024-key chunks at head size 64 (eight requests of 16,384 keys 1,519 against 1,586 us) and at
+    wider heads the two-wave chunks with the merging kernel (None).  Whole ranges where the pairs fill the GPU: at
+    head size 64 from 512 pairs, from 192 beyond 6,144 keys and from 128 beyond 24,576 (sixteen requests of 8,192
+    keys: 1,661 us in chunks against 1,757 whole; twenty-four: 2,109 against 2,086)."""
+    if head_size > 64:
+        walk = max_keys * head_size
+        if pairs >= WHOLE_MIN_PAIRS or any(pairs >= p and walk <= w for p, w in WHOLE_SHORT_WALKS):
+            return 0, 8
+    elif any(pairs >= p and max_keys > k for p, k in LONG_WHOLE_PAIRS):
+        return 0, 8
+    if tasks <= 384:
+        chunk = CHUNK
+    elif tasks <= 768:
+        chunk = 2 * CHUNK
+    elif tasks <= 1536:
+        chunk = 4 * CHUNK
+    elif tasks <= 2560:
+        chunk = 8 * CHUNK
+    elif head_size <= 64:
+        chunk = 4 * CHUNK
+    else:
+        return None
+    while max_keys > MERGE_MAX_PARTS * chunk:
+        chunk *= 2
+    return chunk, 4
 
 
 def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False, head_size: int = 64,
@@ -119,6 +159,10 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False
     """
     pairs = n_split * kv_heads
     tasks = n_split * -(-max_keys // CHUNK) * kv_heads
+    if whole_ok and MERGE_IN_KERNEL and max_keys > MERGE_MAX_KEYS:
+        plan = _long_decode_plan(pairs, tasks, max_keys, head_size)
+        if plan is not None:
+            return plan
     if whole_ok and merges_in_kernel(max_keys):
         # With the chunks merged by the attention kernel itself, chunks cost no second launch, and four waves that
         # share a chunk (64 or 128 keys each, merged in LDS) shorten a wave's chain of dependent loads without more
@@ -414,7 +458,7 @@ def _build_decode_tasks(starts: np.ndarray, group: int, window: int, bucket: int
     comb[..., 9] = 1
     comb[..., 10] = starts[:, None]
     arr = np.concatenate([main, comb.reshape(-1, 12)])
-    return arr, (len(main), s * row_chunks, s * row_chunks * slots, waves, 1, merges_in_kernel(keys))
+    return arr, (len(main), s * row_chunks, s * row_chunks * slots, waves, 1, merges_in_kernel(keys, waves))
 
 
 def plan_key(group: int, window: int, kv_heads: int, hd: int):

@@ -101,8 +101,9 @@ def test_long_contexts(seed):
     starts = rng.integers(15000, 40000, size=s).astype(np.int32)
     counts = np.ones(s, dtype=np.int32)
     bucket = -(-int(starts.max() + 1) // 256) * 256
-    fast, mf = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
-    slow, ms = A.build_tasks(starts, counts, group, window, bucket, vectorized=False, kv_heads=8, max_waves=8)
+    # where at most two waves may share a task (wide heads): two-wave chunks, left to the merging kernel
+    fast, mf = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=2)
+    slow, ms = A.build_tasks(starts, counts, group, window, bucket, vectorized=False, kv_heads=8, max_waves=2)
     assert mf == ms
     live = fast[:, 0] >= 0
     assert np.array_equal(live, slow[:, 0] >= 0) and np.array_equal(fast[live], slow[live])
@@ -110,7 +111,13 @@ def test_long_contexts(seed):
     seen = min(bucket, window + 256) if window else bucket       # keys a token can see
     if seen >= A.LONG_KEYS and s * -(-seen // 256) * 8 > 800:
         spans = fast[live][:, 5] - fast[live][:, 4]
-        assert int(spans.max()) == 512 and mf[3] == 2
+        assert int(spans.max()) == 512 and mf[3] == 2 and not mf[5]
+    # where eight may: four waves a chunk, the chunks the longer the more tasks there are, merged by the kernel
+    wide, mw = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
+    coverage(wide, mw, starts, counts, group, window)
+    assert mw[3] == 4 and mw[5] is True
+    spans = wide[wide[:, 0] >= 0][: mw[0]][:, 5] - wide[wide[:, 0] >= 0][: mw[0]][:, 4]
+    assert int(spans.max()) in (256, 512, 1024, 2048) and -(-seen // int(spans.max())) <= A.MERGE_MAX_PARTS
     # a portion of a prompt beside them
     counts2 = counts.copy()
     counts2[0] = 40
@@ -125,7 +132,7 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     rng = np.random.default_rng(900 + seed)
     s = int(rng.integers(24, 100))
     group, window = int(rng.choice([1, 4, 8])), int(rng.choice([0, 0, 300]))
-    starts = rng.integers(0, 3000, size=s).astype(np.int32)
+    starts = rng.integers(0, 2300, size=s).astype(np.int32)
     counts = np.ones(s, dtype=np.int32)
     bucket = -(-int(starts.max() + 1) // 256) * 256
     arr, meta = A.build_tasks(starts, counts, group, window, bucket, kv_heads=8, max_waves=8)
@@ -153,11 +160,28 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     assert A.chunk_for(4, 512, 8, whole_ok=True, head_size=64) == (0, 8)
     assert A.chunk_for(1, 2048, 8, whole_ok=True, head_size=128) == (128, 1)
     assert A.chunk_for(1, 2048, 8, whole_ok=False, head_size=64) == (128, 1)
-    # twelve requests of 8 KV heads: whole ranges up to 8,192 keys of head size 64, 4,096 of head size 128
-    assert A.chunk_for(12, 8192, 8, whole_ok=True, head_size=64) == (0, 8)
-    assert A.chunk_for(12, 8192, 8, whole_ok=True, head_size=128)[0] > 0
+    # longer contexts: four waves a chunk and chunks so long that about 256 tasks are left, merged by the kernel
+    assert A.chunk_for(1, 4096, 8, whole_ok=True, head_size=64) == (256, 4)
+    assert A.chunk_for(4, 4096, 8, whole_ok=True, head_size=64) == (512, 4)
+    assert A.chunk_for(8, 4096, 8, whole_ok=True, head_size=128) == (1024, 4)
+    assert A.chunk_for(8, 8192, 8, whole_ok=True, head_size=64) == (2048, 4)
+    assert A.chunk_for(1, 32768, 8, whole_ok=True, head_size=64) == (1024, 4)
+    assert A.chunk_for(8, 16384, 8, whole_ok=True, head_size=64) == (1024, 4)
+    assert A.chunk_for(16, 8192, 8, whole_ok=True, head_size=64) == (1024, 4)
+    # (a row piece's parts stay few however long the context)
+    chunk, waves = A.chunk_for(1, 131072, 8, whole_ok=True, head_size=64)
+    assert waves == 4 and 131072 <= A.MERGE_MAX_PARTS * chunk
+    assert A.merges_in_kernel(131072, 4) and not A.merges_in_kernel(131072, 2) and A.merges_in_kernel(2048, 2)
+    # whole ranges where the pairs fill the GPU
+    assert A.chunk_for(64, 4096, 8, whole_ok=True, head_size=64) == (0, 8)
+    assert A.chunk_for(24, 8192, 8, whole_ok=True, head_size=64) == (0, 8)
+    assert A.chunk_for(24, 4096, 8, whole_ok=True, head_size=64) == (1024, 4)
+    assert A.chunk_for(16, 32768, 8, whole_ok=True, head_size=64) == (0, 8)
+    assert A.chunk_for(16, 8192, 8, whole_ok=True, head_size=128) == (0, 8)
     assert A.chunk_for(12, 4096, 8, whole_ok=True, head_size=128) == (0, 8)
-    assert A.chunk_for(12, 32768, 8, whole_ok=True, head_size=64)[0] > 0
+    # wide heads with many tasks: two waves a chunk and the merging kernel, as where fewer than four waves may share
+    assert A.chunk_for(8, 32768, 8, whole_ok=True, head_size=128) == (512, 2)
+    assert A.chunk_for(12, 32768, 8, whole_ok=False, head_size=64)[1] <= 2
     # the merge of the waves' shares must fit the 160 KB of LDS of a CU: eight waves up to heads of 160, two beyond
     assert A.max_waves_for(64) == 8 and A.max_waves_for(128) == 8 and A.max_waves_for(160) == 8
     assert A.max_waves_for(176) == 2 and A.max_waves_for(256) == 2

@@ -749,7 +749,7 @@ def test_attention_whole_ranges_with_eight_waves(window, more):
     from atoma_infer_amd.kernels import attention_bf16 as A
     nh, nkv, hd, page = 32, 8, 64, 16
     g = torch.Generator().manual_seed(7)
-    starts = [0, 1, 30, 31, 32, 255, 256, 257, 511, 1000] + torch.randint(0, 2500, (more,), generator=g).tolist()
+    starts = [0, 1, 30, 31, 32, 255, 256, 257, 511, 1000] + torch.randint(0, 2300, (more,), generator=g).tolist()
     counts = [1] * len(starts)
     lens = [s + 1 for s in starts]
     ks, vs, kc, vc, bt = paged_setup(lens, nkv, hd, page, torch.bfloat16, seed=3)
@@ -834,6 +834,54 @@ def test_decode_plans_with_large_groups(nh, nkv, hd, plan, monkeypatch):
         want = plain_attention(q, ks[e], vs[e], s, scale, 0, group).reshape(1, nh * hd)
         err = (out[e:e + 1].double().cpu() - want).abs().max() / want.abs().max()
         assert err < 2e-2, f"request {e} at {s}: {err:.3e}"
+
+
+@pytest.mark.parametrize("nh,nkv,hd,starts,chunk", [
+    (32, 8, 64, [20000], 512),                      # 40 parts for one wave to merge, in rounds
+    (32, 8, 64, [5000, 0, 4999, 2303, 17], 1024),
+    (8, 2, 128, [9000, 8000, 1], 256),
+    (16, 8, 64, [3000] * 7 + [8191], 2048),         # four parts, of which most requests fill two
+])
+def test_decode_chunks_that_grow_with_the_context(nh, nkv, hd, starts, chunk):
+    """Decode steps beyond the contexts of a few thousand keys: four waves a chunk, chunks the longer the more there
+    are, and the wave that finishes a row piece's last chunk merges all of its parts, however many.  One key far
+    from the decoded token is made to stand out in the first request, so that a part lost in the merge shows."""
+    import numpy as np
+    from atoma_infer_amd.kernels import attention_bf16
+    group, page = nh // nkv, 16
+    counts = [1] * len(starts)
+    far = min(37, starts[0])
+
+    def edit(ks, vs):
+        ks[0][far] *= 3.0
+    ks, vs, kc, vc, bt = paged_setup([s + 1 for s in starts], nkv, hd, page, torch.bfloat16, seed=hd + len(starts),
+                                     edit=edit)
+    t = len(starts)
+    g = torch.Generator().manual_seed(5)
+    qkv = (torch.randn(t, (nh + 2 * nkv) * hd, generator=g) * 1.5).bfloat16().to(DEV)
+    # the first request's queries look for the far key
+    qkv[0, : nh * hd] = (ks[0][far].float().repeat_interleave(group, dim=0).reshape(-1) * 0.5).bfloat16().to(DEV)
+    out = torch.full((t, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ctx = FakeCtx(starts, counts)
+    bucket = -(-(max(starts) + 1) // 256) * 256
+    arr, meta = attention_bf16.build_tasks(np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32),
+                                           group, 0, bucket, kv_heads=nkv, max_waves=attention_bf16.max_waves_for(hd),
+                                           head_size=hd)
+    assert meta[3] == 4 and meta[5] is True
+    live = arr[: meta[0]][arr[: meta[0], 0] >= 0]
+    assert int((live[:, 5] - live[:, 4]).max()) == chunk
+    ctx.plans = {attention_bf16.plan_key(group, 0, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
+    scale = 1.0 / math.sqrt(hd)
+    wide = torch.zeros((t, bucket // page), dtype=torch.int32, device=DEV)
+    wide[:, : bt.shape[1]] = bt
+    for _ in range(2):                                 # the second launch finds the counters as the first left them
+        out.fill_(float("nan"))
+        assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, FakeCache(wide, page), scale, 0, nh, nkv, hd)
+        for e, s in enumerate(starts):
+            q = qkv[e:e + 1, : nh * hd].cpu().view(1, nh, hd)
+            want = plain_attention(q, ks[e], vs[e], s, scale, 0, group).reshape(1, nh * hd)
+            err = (out[e:e + 1].double().cpu() - want).abs().max() / want.abs().max()
+            assert err < 2e-2, f"request {e} at {s}: {err:.3e}"
 
 
 @pytest.mark.parametrize("plan", PLANS)
