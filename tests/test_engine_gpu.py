@@ -404,6 +404,26 @@ def test_decoding_with_whole_key_ranges(model_dirs, monkeypatch):
     assert attention_bf16.chunk_for(3, 700, 2, whole_ok=True) == (0, 8)
 
 
+def test_decoding_at_contexts_of_thousands_of_tokens(tmp_path):
+    """Beyond a few thousand keys a decoded token's chunks grow with the step's tasks, four waves share each and the
+    attention kernel merges a row piece's parts itself, twenty of them here.  Three requests of 5,000, 2,290 and 40
+    tokens decode together through graphs; the second crosses the length at which the plans change."""
+    from atoma_infer_amd.kernels import attention_bf16
+    cfg = dict(TINY["D"], max_position_embeddings=8192)
+    path = make_model_dir(str(tmp_path / "long"), cfg, seed=21, dtype="bfloat16", norm_jitter=0.1)
+    vocab = cfg["vocab_size"]
+    requests = {"a": random_tokens(5000, vocab, 41), "b": random_tokens(2330, vocab, 42), "c": random_tokens(82, vocab, 43)}
+    runner = make_runner(path, "bfloat16", 16, 480)
+    steps = [([("a", 2048)], []), ([("a", 2048)], []), ([("a", 862), ("b", 1100)], []), ([("b", 1188), ("c", 40)], [])]
+    steps += [([("a", 1), ("b", 1), ("c", 1)], []) for _ in range(42)]
+    got = run_schedule(runner, requests, steps)
+    check_against_plain(path, requests, got, "bfloat16")
+    graphs = [k for k, g in runner._graphs.items() if g.graph is not None]
+    assert any(k[0] == 3 for k in graphs), "the decode steps were meant to replay as graphs"
+    assert attention_bf16.chunk_for(3, 5120, 2, whole_ok=True) == (256, 4)
+    assert attention_bf16.merges_in_kernel(5120, 4)
+
+
 LLAMA_1B_LAYERS = {
     "architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": 2048, "intermediate_size": 8192,
     "vocab_size": 128256, "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8,
