@@ -172,14 +172,16 @@ def chunk_for(n_split: int, max_keys: int, kv_heads: int, whole_ok: bool = False
         # against 860 for whole ranges), 512-key chunks beyond (eight requests of 2,049 keys 901 against 909 us with
         # 256-key chunks of two waves, twelve of 1,500 keys 943 against 968 for whole ranges); whole ranges from 128
         # pairs on (sixteen requests of 2,049 keys 1,084 against 1,125 us) and, for the pair alone, up to 512 keys.
-        # Wide heads with few tasks keep a wave a chunk (head size 128, one request of 1,024 keys: 12.2 against
-        # 12.8 us a layer).
         if max_keys <= MERGE_WHOLE_MAX_KEYS or pairs >= WHOLE_MIN_PAIRS:
             return 0, 8
         if tasks > 544:
             return 2 * CHUNK, 4
-        if head_size > 64 and tasks <= 300:
-            return 128, 1
+        # few requests of up to 1,536 keys: 128-key chunks, whose parts (twelve at most) the merging wave still takes
+        # in one round (one to four requests of 700 to 1,024 keys 1.5 to 2 % quicker steps at head size 64, one to
+        # six at head size 128 about 1 %; with more tasks or keys the 256-key chunks are as quick or quicker)
+        short_tasks = n_split * -(-max_keys // 128) * kv_heads
+        if max_keys <= 1536 and short_tasks <= (400 if head_size > 64 else 200):
+            return 128, 4
         return CHUNK, 4
     if whole_ok:
         walk = max_keys * head_size

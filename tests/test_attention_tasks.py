@@ -158,7 +158,11 @@ def test_whole_ranges_for_many_decoding_requests(seed):
     assert A.chunk_for(12, 2048, 8, whole_ok=True, head_size=128) == (512, 4)
     assert A.chunk_for(16, 2048, 8, whole_ok=True, head_size=64) == (0, 8)
     assert A.chunk_for(4, 512, 8, whole_ok=True, head_size=64) == (0, 8)
-    assert A.chunk_for(1, 2048, 8, whole_ok=True, head_size=128) == (128, 1)
+    assert A.chunk_for(1, 2048, 8, whole_ok=True, head_size=128) == (256, 4)
+    assert A.chunk_for(2, 1024, 8, whole_ok=True, head_size=64) == (128, 4)
+    assert A.chunk_for(4, 1024, 8, whole_ok=True, head_size=64) == (256, 4)
+    assert A.chunk_for(4, 1024, 8, whole_ok=True, head_size=128) == (128, 4)
+    assert A.chunk_for(1, 1792, 8, whole_ok=True, head_size=64) == (256, 4)
     assert A.chunk_for(1, 2048, 8, whole_ok=False, head_size=64) == (128, 1)
     # longer contexts: four waves a chunk and chunks so long that about 256 tasks are left, merged by the kernel
     assert A.chunk_for(1, 4096, 8, whole_ok=True, head_size=64) == (256, 4)
