@@ -267,12 +267,17 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, out: 
     return out
 
 
+SPLIT_MAX_VOCAB = 262144       # the largest vocabulary whose rows ``sample_packed(split=True)`` cuts into parts
+
+
 def sample_packed(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-                  uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None, split: bool = False) -> torch.Tensor:
     """Per row of float32 ``logits`` [S, V]: argmax where temperature <= 0, else a draw (see sampling.hip).
 
     Returns one float32 tensor [2, S]: row 0 holds the tokens (int32 bits), row 1 the logits of the chosen tokens,
-    so that one copy brings both to the host.
+    so that one copy brings both to the host.  ``split``: every row is shared by several blocks over six short
+    launches instead of one long one (the same tokens; quicker when rows draw from a large vocabulary: one block
+    walks a row with top-k and top-p in over 100 us); vocabularies beyond ``SPLIT_MAX_VOCAB`` keep the one launch.
     """
     _dev(logits, temperature, top_k, top_p, uniform)
     _need(logits.dim() == 2 and logits.dtype is torch.float32 and logits.stride(1) == 1, "logits must be float32 [S, V]")
@@ -285,15 +290,24 @@ def sample_packed(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.
     _need(workspace.dtype is torch.float32 and workspace.is_contiguous() and workspace.numel() >= s * v,
           "sample: workspace too small")
     out = torch.empty((2, s), dtype=torch.float32, device=logits.device)
-    _check(core().atoma_sample(_p(logits), logits.stride(0) if s > 1 else v, s, v, _p(temperature), _p(top_k),
+    ld = logits.stride(0) if s > 1 else v
+    if split and v <= SPLIT_MAX_VOCAB:
+        lib = core()
+        lib.atoma_sample_split_scratch_bytes.restype = ctypes.c_size_t
+        scratch = torch.empty((int(lib.atoma_sample_split_scratch_bytes(s)) + 3) // 4, dtype=torch.int32,
+                              device=logits.device)
+        _check(lib.atoma_sample_split(_p(logits), ld, s, v, _p(temperature), _p(top_k), _p(top_p), _p(uniform),
+                                      _p(workspace), _p(scratch), _p(out[0]), _p(out[1]), _stream()), "sample (split)")
+        return out
+    _check(core().atoma_sample(_p(logits), ld, s, v, _p(temperature), _p(top_k),
                                _p(top_p), _p(uniform), _p(workspace), _p(out[0]), _p(out[1]), _stream()), "sample")
     return out
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None):
+           uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None, split: bool = False):
     """``sample_packed`` as (tokens int32 [S], logits of the chosen tokens float32 [S])."""
-    out = sample_packed(logits, temperature, top_k, top_p, uniform, workspace)
+    out = sample_packed(logits, temperature, top_k, top_p, uniform, workspace, split)
     return out[0].view(torch.int32), out[1]
 
 

@@ -17,6 +17,8 @@ from ..kernels import ops
 from .params import SamplingPlan
 
 _MASK = (1 << 64) - 1
+# vocabularies from which on the rows of a step that draws are cut into parts (a block walks fewer values quickly enough)
+SPLIT_MIN_VOCAB = 32768
 
 
 def uniform(seed: int, counter: int) -> float:
@@ -102,7 +104,9 @@ class Sampler:
         if pen_rows:
             pen = torch.tensor([pen_rows, pen_toks], dtype=torch.int32).to(self.device)
             ops.repeat_penalty(logits, pen[0], pen[1], m[3])
-        out = ops.sample_packed(logits, m[0], m[4].view(torch.int32), m[1], m[2])
+        # (rows that draw are shared by several blocks each: a block walks a row of a large vocabulary too slowly)
+        out = ops.sample_packed(logits, m[0], m[4].view(torch.int32), m[1], m[2],
+                                split=not all_greedy and logits.shape[1] >= SPLIT_MIN_VOCAB)
         tok, lg = out[0].view(torch.int32), out[1]
         host, pool = self._host_buffer(s)
         host.copy_(out, non_blocking=True)

@@ -192,8 +192,12 @@ def test_eos_stops_and_too_long_is_ignored(model_dirs):
 # the sampling kernel against the plain sampling functions
 
 
+SPLIT = [False, True]       # a block a row in one launch, or every row shared by several blocks over six launches
+
+
+@pytest.mark.parametrize("split", SPLIT)
 @pytest.mark.parametrize("vocab", [331, 1000, 5000, 50001, 128256])
-def test_sample_kernel(vocab):
+def test_sample_kernel(vocab, split):
     """Rows of a batch against the plain distribution and draw; 50001 leaves all rows but the first unaligned, 128256
     is a real vocabulary (every wave of the kernel has several slices of several pieces)."""
     from atoma_infer_amd.kernels import ops
@@ -208,7 +212,7 @@ def test_sample_kernel(vocab):
     for u in (0.0, 0.013, 0.25, 0.5, 0.77, 0.999):
         tok, lg = ops.sample(logits.cuda(), dev([r[0] for r in rows], torch.float32),
                              dev([r[1] for r in rows], torch.int32), dev([r[2] for r in rows], torch.float32),
-                             dev([u] * len(rows), torch.float32))
+                             dev([u] * len(rows), torch.float32), split=split)
         tok, lg = tok.cpu().tolist(), lg.cpu()
         for i, (t, k, p) in enumerate(rows):
             if t == 0.0:
@@ -222,9 +226,11 @@ def test_sample_kernel(vocab):
             assert float(lg[i]) == float(logits[i, tok[i]])
 
 
-def test_sample_kernel_many_ties_in_a_large_vocabulary():
-    """Ties at the threshold that are only partly kept, spread over the stretches of several waves: the kept ones
-    are those of lowest index, and every kept token can be drawn."""
+@pytest.mark.parametrize("split", SPLIT)
+def test_sample_kernel_many_ties_in_a_large_vocabulary(split):
+    """Ties at the threshold that are only partly kept, spread over the stretches of several waves (and over the
+    parts of a row that several blocks share): the kept ones are those of lowest index, and every kept token can be
+    drawn."""
     from atoma_infer_amd.kernels import ops
     vocab = 40000
     logits = torch.full((2, vocab), -3.0)
@@ -238,14 +244,15 @@ def test_sample_kernel_many_ties_in_a_large_vocabulary():
     for i in range(n):
         u = (i + 0.5) / n
         tok, _ = ops.sample(logits.cuda(), dev([1.0, 1.0], torch.float32), dev([7, 12], torch.int32),
-                            dev([1.0, 1.0], torch.float32), dev([u, u], torch.float32))
+                            dev([1.0, 1.0], torch.float32), dev([u, u], torch.float32), split=split)
         for r, t in enumerate(tok.cpu().tolist()):
             seen[r].add(t)
     assert seen[0] == set(tied[:7])
     assert seen[1] == {123} | set(tied[:11])
 
 
-def test_sample_kernel_kept_sets_and_ties():
+@pytest.mark.parametrize("split", SPLIT)
+def test_sample_kernel_kept_sets_and_ties(split):
     from atoma_infer_amd.kernels import ops
     vocab = 700
     logits = torch.zeros(3, vocab)
@@ -257,10 +264,35 @@ def test_sample_kernel_kept_sets_and_ties():
         u = (i + 0.5) / 64
         dev = lambda x, dt: torch.tensor(x, dtype=dt, device="cuda:0")
         tok, _ = ops.sample(logits.cuda(), dev([1.0, 1.0, 1.0], torch.float32), dev([2, 0, 3], torch.int32),
-                            dev([1.0, 0.5, 1.0], torch.float32), dev([u] * 3, torch.float32))
+                            dev([1.0, 0.5, 1.0], torch.float32), dev([u] * 3, torch.float32), split=split)
         for r, t in enumerate(tok.cpu().tolist()):
             seen[r].add(t)
     assert seen[0] == {5, 100} and seen[1] == {7} and seen[2] == {vocab - 3, vocab - 2, vocab - 1}
+
+
+@pytest.mark.parametrize("rows,vocab", [(1, 128256), (8, 128256), (3, 200003), (70, 50001), (300, 40000), (2, 262144)])
+def test_rows_shared_by_several_blocks_draw_the_same_tokens(rows, vocab):
+    """The six launches that share every row among several blocks against the one launch of a block a row: the same
+    tokens and logits bit for bit, for rows of every mode (greedy ones among them), flat and peaked logits, NaN rows,
+    vocabularies that leave rows unaligned and parts of unequal length."""
+    from atoma_infer_amd.kernels import ops
+    g = torch.Generator().manual_seed(rows * 7 + vocab)
+    logits = torch.randn(rows, vocab, generator=g) * torch.where(torch.arange(rows) % 2 == 0, 0.3, 3.0)[:, None]
+    modes = [(0.0, 0, 1.0), (0.8, 0, 1.0), (0.8, 50, 1.0), (0.8, 0, 0.9), (0.8, 50, 0.9), (1.5, 3, 0.5), (0.3, 1000, 0.99)]
+    pick = [modes[i % len(modes)] for i in range(rows)]
+    if rows >= 8:
+        logits[5] = float("nan")
+        logits[6, 100:5000] = 1.25                       # thousands of ties, partly kept
+        pick[6] = (1.0, 700, 0.9)
+    dev = lambda x, dt: torch.tensor(x, dtype=dt, device="cuda:0")
+    lg = logits.cuda()
+    t, k, p = (dev([m[i] for m in pick], dt) for i, dt in ((0, torch.float32), (1, torch.int32), (2, torch.float32)))
+    for u in (0.0, 0.31, 0.5, 0.93, 0.999999):
+        uu = dev([(u + 0.37 * i) % 1.0 for i in range(rows)], torch.float32)
+        one = ops.sample_packed(lg, t, k, p, uu)
+        six = ops.sample_packed(lg, t, k, p, uu, split=True)
+        assert torch.equal(one[0].view(torch.int32), six[0].view(torch.int32)), (u, one[0].view(torch.int32), six[0].view(torch.int32))
+        assert torch.equal(one[1].isnan(), six[1].isnan()) and torch.equal(one[1].nan_to_num(), six[1].nan_to_num())
 
 
 def test_repeat_penalty_kernel_and_temperature_limit():
