@@ -701,7 +701,7 @@ __global__ void __launch_bounds__(kSampThreads)
 split_weights_kernel(const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ temperature,
                      const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
                      float* __restrict__ weights, SplitRow* __restrict__ rows, int32_t* __restrict__ out_token,
-                     float* __restrict__ out_logit) {
+                     float* __restrict__ out_logit, int cuts) {
   __shared__ uint32_t hist_k[kBins];
   __shared__ u64 hist_pm[kBins];
   __shared__ u64 wave_u64[kSampWaves];
@@ -722,7 +722,7 @@ split_weights_kernel(const float* __restrict__ logits, int ld, int vocab, const 
     out_logit[row] = lr[a.i];
   }
   if (!(temp > 0.f)) return;
-  const bool cut_k = k > 0 && k < vocab, cut_p = p < 1.0f, cut = cut_k || cut_p;
+  const bool cut_k = cuts && k > 0 && k < vocab, cut_p = cuts && p < 1.0f, cut = cut_k || cut_p;
   hist_k[tid] = 0;
   hist_pm[tid] = 0;
   __syncthreads();
@@ -936,7 +936,8 @@ __global__ void __launch_bounds__(kSampThreads)
 split_draw_kernel(const float* __restrict__ logits, int ld, int vocab, int parts, const float* __restrict__ temperature,
                   const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
                   const float* __restrict__ uniform, const float* __restrict__ weights,
-                  SplitRow* __restrict__ rows, int32_t* __restrict__ out_token, float* __restrict__ out_logit) {
+                  SplitRow* __restrict__ rows, int32_t* __restrict__ out_token, float* __restrict__ out_logit,
+                  int cuts) {
   __shared__ u64 wave_u64[kSampWaves];
   __shared__ uint32_t wave_u32[kSampWaves];
   __shared__ int pick_s;
@@ -944,7 +945,7 @@ split_draw_kernel(const float* __restrict__ logits, int ld, int vocab, int parts
   if (!(temperature[row] > 0.f)) return;
   const int k = top_k[row];
   const float p = top_p[row];
-  const bool cut_k = k > 0 && k < vocab, cut_p = p < 1.0f, cut = cut_k || cut_p;
+  const bool cut_k = cuts && k > 0 && k < vocab, cut_p = cuts && p < 1.0f, cut = cut_k || cut_p;
   SplitRow& r = rows[row];
   SplitCut c = {0, 0xffffffffu, ~0ull, true};
   if (cut) c = split_cut(r.search[2], cut_k, cut_p);    // (the search ended in the launch before this one)
@@ -1117,10 +1118,12 @@ extern "C" size_t atoma_sample_split_scratch_bytes(int n_rows) { return (size_t)
 
 // atoma_sample for steps in which rows draw: the same tokens from six short launches (see above).  scratch: at
 // least atoma_sample_split_scratch_bytes(n_rows) bytes, 16-byte aligned, whatever they hold.  Vocabularies too
-// large for sixteen parts (above 262,144) are refused: atoma_sample takes them.
+// large for sixteen parts (above 262,144) are refused: atoma_sample takes them.  cuts == 0: the caller knows that
+// no row has a top-k or top-p cut; the three launches of the search are left out, and top_k and top_p are not read
+// (a row that has a cut all the same is drawn from all of its weights).
 extern "C" int atoma_sample_split(const float* logits, int ld, int n_rows, int vocab, const float* temperature,
                                   const int32_t* top_k, const float* top_p, const float* uniform, float* weights,
-                                  void* scratch, int32_t* out_token, float* out_logit, hipStream_t stream) {
+                                  void* scratch, int cuts, int32_t* out_token, float* out_logit, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (vocab <= 0 || ld < vocab || scratch == nullptr || ((uintptr_t)scratch & 15) != 0) return ATOMA_ERR_SHAPE;
   const int parts = split_parts(n_rows, vocab);
@@ -1129,12 +1132,15 @@ extern "C" int atoma_sample_split(const float* logits, int ld, int n_rows, int v
   const dim3 grid(n_rows, parts), block(kSampThreads);
   hipLaunchKernelGGL(split_max_kernel, grid, block, 0, stream, logits, ld, vocab, rows);
   hipLaunchKernelGGL(split_weights_kernel, grid, block, 0, stream, logits, ld, vocab, temperature, top_k, top_p, weights,
-                     rows, out_token, out_logit);
-  for (int level = 1; level <= 2; ++level)
-    hipLaunchKernelGGL(split_level_kernel, grid, block, 0, stream, level, vocab, temperature, top_k, top_p, weights, rows);
-  hipLaunchKernelGGL(split_mass_kernel, grid, block, 0, stream, vocab, temperature, top_k, top_p, weights, rows);
+                     rows, out_token, out_logit, cuts);
+  if (cuts) {
+    for (int level = 1; level <= 2; ++level)
+      hipLaunchKernelGGL(split_level_kernel, grid, block, 0, stream, level, vocab, temperature, top_k, top_p, weights,
+                         rows);
+    hipLaunchKernelGGL(split_mass_kernel, grid, block, 0, stream, vocab, temperature, top_k, top_p, weights, rows);
+  }
   hipLaunchKernelGGL(split_draw_kernel, dim3(n_rows), block, 0, stream, logits, ld, vocab, parts, temperature, top_k,
-                     top_p, uniform, weights, rows, out_token, out_logit);
+                     top_p, uniform, weights, rows, out_token, out_logit, cuts);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }

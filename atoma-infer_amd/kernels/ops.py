@@ -271,13 +271,16 @@ SPLIT_MAX_VOCAB = 262144       # the largest vocabulary whose rows ``sample_pack
 
 
 def sample_packed(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-                  uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None, split: bool = False) -> torch.Tensor:
+                  uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None, split: bool = False,
+                  cuts: bool = True) -> torch.Tensor:
     """Per row of float32 ``logits`` [S, V]: argmax where temperature <= 0, else a draw (see sampling.hip).
 
     Returns one float32 tensor [2, S]: row 0 holds the tokens (int32 bits), row 1 the logits of the chosen tokens,
     so that one copy brings both to the host.  ``split``: every row is shared by several blocks over six short
     launches instead of one long one (the same tokens; quicker when rows draw from a large vocabulary: one block
     walks a row with top-k and top-p in over 100 us); vocabularies beyond ``SPLIT_MAX_VOCAB`` keep the one launch.
+    ``cuts=False`` (with ``split``): the caller knows that no row has a top-k or top-p cut, and the three launches
+    that search for them are left out (``top_k`` and ``top_p`` are then not read).
     """
     _dev(logits, temperature, top_k, top_p, uniform)
     _need(logits.dim() == 2 and logits.dtype is torch.float32 and logits.stride(1) == 1, "logits must be float32 [S, V]")
@@ -297,7 +300,8 @@ def sample_packed(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.
         scratch = torch.empty((int(lib.atoma_sample_split_scratch_bytes(s)) + 3) // 4, dtype=torch.int32,
                               device=logits.device)
         _check(lib.atoma_sample_split(_p(logits), ld, s, v, _p(temperature), _p(top_k), _p(top_p), _p(uniform),
-                                      _p(workspace), _p(scratch), _p(out[0]), _p(out[1]), _stream()), "sample (split)")
+                                      _p(workspace), _p(scratch), 1 if cuts else 0, _p(out[0]), _p(out[1]), _stream()),
+               "sample (split)")
         return out
     _check(core().atoma_sample(_p(logits), ld, s, v, _p(temperature), _p(top_k),
                                _p(top_p), _p(uniform), _p(workspace), _p(out[0]), _p(out[1]), _stream()), "sample")
@@ -305,9 +309,9 @@ def sample_packed(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None, split: bool = False):
+           uniform: torch.Tensor, workspace: Optional[torch.Tensor] = None, split: bool = False, cuts: bool = True):
     """``sample_packed`` as (tokens int32 [S], logits of the chosen tokens float32 [S])."""
-    out = sample_packed(logits, temperature, top_k, top_p, uniform, workspace, split)
+    out = sample_packed(logits, temperature, top_k, top_p, uniform, workspace, split, cuts)
     return out[0].view(torch.int32), out[1]
 
 

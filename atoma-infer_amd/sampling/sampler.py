@@ -105,8 +105,9 @@ class Sampler:
             pen = torch.tensor([pen_rows, pen_toks], dtype=torch.int32).to(self.device)
             ops.repeat_penalty(logits, pen[0], pen[1], m[3])
         # (rows that draw are shared by several blocks each: a block walks a row of a large vocabulary too slowly)
+        cuts = any(not pl.greedy and (pl.top_k > 0 or pl.top_p < 1.0) for pl in plans)
         out = ops.sample_packed(logits, m[0], m[4].view(torch.int32), m[1], m[2],
-                                split=not all_greedy and logits.shape[1] >= SPLIT_MIN_VOCAB)
+                                split=not all_greedy and logits.shape[1] >= SPLIT_MIN_VOCAB, cuts=cuts)
         tok, lg = out[0].view(torch.int32), out[1]
         host, pool = self._host_buffer(s)
         host.copy_(out, non_blocking=True)

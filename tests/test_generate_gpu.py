@@ -293,6 +293,12 @@ def test_rows_shared_by_several_blocks_draw_the_same_tokens(rows, vocab):
         six = ops.sample_packed(lg, t, k, p, uu, split=True)
         assert torch.equal(one[0].view(torch.int32), six[0].view(torch.int32)), (u, one[0].view(torch.int32), six[0].view(torch.int32))
         assert torch.equal(one[1].isnan(), six[1].isnan()) and torch.equal(one[1].nan_to_num(), six[1].nan_to_num())
+    # a caller that knows of no cut leaves the search out: the rows are then drawn from all of their weights
+    no_k, no_p = torch.zeros_like(k), torch.ones_like(p)
+    uu = dev([(0.77 + 0.37 * i) % 1.0 for i in range(rows)], torch.float32)
+    one = ops.sample_packed(lg, t, no_k, no_p, uu)
+    four = ops.sample_packed(lg, t, k, p, uu, split=True, cuts=False)
+    assert torch.equal(one[0].view(torch.int32), four[0].view(torch.int32))
 
 
 def test_repeat_penalty_kernel_and_temperature_limit():
