@@ -836,13 +836,15 @@ def test_decode_plans_with_large_groups(nh, nkv, hd, plan, monkeypatch):
         assert err < 2e-2, f"request {e} at {s}: {err:.3e}"
 
 
-@pytest.mark.parametrize("nh,nkv,hd,starts,chunk", [
-    (32, 8, 64, [20000], 512),                      # 40 parts for one wave to merge, in rounds
-    (32, 8, 64, [5000, 0, 4999, 2303, 17], 1024),
-    (8, 2, 128, [9000, 8000, 1], 256),
-    (16, 8, 64, [3000] * 7 + [8191], 2048),         # four parts, of which most requests fill two
+@pytest.mark.parametrize("nh,nkv,hd,starts,chunk,window", [
+    (32, 8, 64, [20000], 512, 0),                   # 40 parts for one wave to merge, in rounds
+    (32, 8, 64, [5000, 0, 4999, 2303, 17], 1024, 0),
+    (8, 2, 128, [9000, 8000, 1], 256, 0),
+    (16, 8, 64, [3000] * 7 + [8191], 2048, 0),      # four parts, of which most requests fill two
+    (32, 8, 64, [9000, 3100, 2999, 40], 512, 3000), # a window of 3,000 keys wherever it lies: its chunks' slots
+    (32, 8, 64, [30000] * 6 + [7], 1024, 5000),
 ])
-def test_decode_chunks_that_grow_with_the_context(nh, nkv, hd, starts, chunk):
+def test_decode_chunks_that_grow_with_the_context(nh, nkv, hd, starts, chunk, window):
     """Decode steps beyond the contexts of a few thousand keys: four waves a chunk, chunks the longer the more there
     are, and the wave that finishes a row piece's last chunk merges all of its parts, however many.  One key far
     from the decoded token is made to stand out in the first request, so that a part lost in the merge shows."""
@@ -850,7 +852,7 @@ def test_decode_chunks_that_grow_with_the_context(nh, nkv, hd, starts, chunk):
     from atoma_infer_amd.kernels import attention_bf16
     group, page = nh // nkv, 16
     counts = [1] * len(starts)
-    far = min(37, starts[0])
+    far = min(37, starts[0]) if not window else starts[0] - window + 2       # (the second key the window shows)
 
     def edit(ks, vs):
         ks[0][far] *= 3.0
@@ -865,21 +867,21 @@ def test_decode_chunks_that_grow_with_the_context(nh, nkv, hd, starts, chunk):
     ctx = FakeCtx(starts, counts)
     bucket = -(-(max(starts) + 1) // 256) * 256
     arr, meta = attention_bf16.build_tasks(np.asarray(starts, dtype=np.int32), np.asarray(counts, dtype=np.int32),
-                                           group, 0, bucket, kv_heads=nkv, max_waves=attention_bf16.max_waves_for(hd),
-                                           head_size=hd)
+                                           group, window, bucket, kv_heads=nkv,
+                                           max_waves=attention_bf16.max_waves_for(hd), head_size=hd)
     assert meta[3] == 4 and meta[5] is True
     live = arr[: meta[0]][arr[: meta[0], 0] >= 0]
     assert int((live[:, 5] - live[:, 4]).max()) == chunk
-    ctx.plans = {attention_bf16.plan_key(group, 0, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
+    ctx.plans = {attention_bf16.plan_key(group, window, nkv, hd): (torch.from_numpy(arr).to(DEV), meta)}
     scale = 1.0 / math.sqrt(hd)
     wide = torch.zeros((t, bucket // page), dtype=torch.int32, device=DEV)
     wide[:, : bt.shape[1]] = bt
     for _ in range(2):                                 # the second launch finds the counters as the first left them
         out.fill_(float("nan"))
-        assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, FakeCache(wide, page), scale, 0, nh, nkv, hd)
+        assert attention_bf16.try_attention(qkv, kc, vc, out, ctx, FakeCache(wide, page), scale, window, nh, nkv, hd)
         for e, s in enumerate(starts):
             q = qkv[e:e + 1, : nh * hd].cpu().view(1, nh, hd)
-            want = plain_attention(q, ks[e], vs[e], s, scale, 0, group).reshape(1, nh * hd)
+            want = plain_attention(q, ks[e], vs[e], s, scale, window, group).reshape(1, nh * hd)
             err = (out[e:e + 1].double().cpu() - want).abs().max() / want.abs().max()
             assert err < 2e-2, f"request {e} at {s}: {err:.3e}"
 
