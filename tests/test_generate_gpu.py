@@ -301,6 +301,48 @@ def test_rows_shared_by_several_blocks_draw_the_same_tokens(rows, vocab):
     assert torch.equal(one[0].view(torch.int32), four[0].view(torch.int32))
 
 
+def test_the_sampler_shares_the_rows_of_a_large_vocabulary():
+    """Through the engine's sampler: a step whose rows draw from 128k logits goes to the launches that share every
+    row among several blocks, with the search left out when no row has a cut; the tokens are those of a block a row
+    with the same uniform numbers, and those of the plain distribution."""
+    from atoma_infer_amd.kernels import ops
+    from atoma_infer_amd.sampling import Sampler, validate, GenerateParameters
+    from atoma_infer_amd.sampling.sampler import uniform
+    vocab = 128256
+    logits = (torch.randn(5, vocab, generator=torch.Generator().manual_seed(3)) * 2.5).cuda()
+    make = lambda **kw: validate(GenerateParameters(ignore_eos_token=True, **kw), 3, 100, 200)
+    with_cuts = [make(temperature=0.8, top_k=50, top_p=0.9, random_seed=5), make(do_sample=False),
+                 make(temperature=1.3, random_seed=6), make(temperature=0.6, top_p=0.5, random_seed=7),
+                 make(temperature=0.9, top_k=3, random_seed=8)]
+    without = [make(temperature=0.8, random_seed=5), make(do_sample=False), make(temperature=1.3, random_seed=6),
+               make(temperature=0.6, random_seed=7), make(temperature=2.0, random_seed=8)]
+    sampler = Sampler(torch.device("cuda:0"))
+    dev = lambda x, dt: torch.tensor(x, dtype=dt, device="cuda:0")
+    calls = []
+    real = ops.sample_packed
+    try:
+        # (the sampler names its options; the comparison below goes through ops.sample, which does not)
+        ops.sample_packed = lambda *a, **kw: (calls.append(kw) if kw else None, real(*a, **kw))[1]
+        for plans in (with_cuts, without):
+            for step in (0, 1, 17):
+                got, got_lg = sampler.sample(logits.clone(), plans, [step] * 5, [()] * 5)
+                uu = [0.0 if pl.greedy else uniform(pl.random_seed, step) for pl in plans]
+                t = [0.0 if pl.greedy else pl.temperature for pl in plans]
+                want, want_lg = ops.sample(logits, dev(t, torch.float32), dev([pl.top_k for pl in plans], torch.int32),
+                                           dev([pl.top_p for pl in plans], torch.float32), dev(uu, torch.float32))
+                assert got == want.cpu().tolist() and got_lg == want_lg.cpu().tolist()
+                for i, pl in enumerate(plans):
+                    if pl.greedy:
+                        assert got[i] == int(logits[i].argmax())
+                    else:
+                        d = plain_llama.sampling_distribution(logits[i].cpu(), pl.temperature, pl.top_k, pl.top_p)
+                        assert d[got[i]] > 0
+    finally:
+        ops.sample_packed = real
+    assert all(kw.get("split") for kw in calls)
+    assert [kw.get("cuts") for kw in calls] == [True] * 3 + [False] * 3
+
+
 def test_repeat_penalty_kernel_and_temperature_limit():
     from atoma_infer_amd.kernels import ops
     from atoma_infer_amd.sampling import Sampler, validate, GenerateParameters
