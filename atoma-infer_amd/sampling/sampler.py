@@ -36,6 +36,7 @@ class Pending:
     def __init__(self, tokens: torch.Tensor, logits: torch.Tensor, host: torch.Tensor, event: torch.cuda.Event,
                  pool: Optional[list] = None):
         self.tokens, self.logits, self._host, self.event, self._pool = tokens, logits, host, event, pool
+        self._meta, self._meta_pool = None, None
 
     def result(self) -> Tuple[List[int], List[float]]:
         """Wait for the copy and return (tokens, logits of the chosen tokens)."""
@@ -45,6 +46,9 @@ class Pending:
         if self._pool is not None:            # the pinned buffer serves a later step
             self._pool.append(self._host)
             self._pool = None
+        if self._meta_pool is not None:       # (so does the one that brought the parameters: its copy is over too)
+            self._meta_pool.append(self._meta)
+            self._meta_pool = None
         return got
 
 
@@ -55,6 +59,7 @@ class Sampler:
         # rows -> pinned buffers [2, rows] that have been read (a pinned tensor made and dropped every step costs an
         # event in the GPU's queue when torch takes it back: 4 us a step)
         self._host_pool = {}
+        self._meta_pool = {}          # rows -> pinned buffers [5, rows] for the rows' parameters, likewise
 
     def _host_buffer(self, s: int):
         pool = self._host_pool.setdefault(s, [])
@@ -88,7 +93,8 @@ class Sampler:
             ev.record()
             return Pending(out[0].view(torch.int32), out[1], host, ev, pool)
         # one packed upload: temperature, top_p, uniform, penalty (float32) and top_k (int32 bits)
-        meta = torch.empty((5, s), dtype=torch.float32, pin_memory=True)
+        meta_pool = self._meta_pool.setdefault(s, [])
+        meta = meta_pool.pop() if meta_pool else torch.empty((5, s), dtype=torch.float32, pin_memory=True)
         mn = meta.numpy()
         top_k = mn[4].view(np.int32)
         for i, pl in enumerate(plans):
@@ -114,7 +120,8 @@ class Sampler:
         ev = torch.cuda.Event()
         ev.record()
         pending = Pending(tok, lg, host, ev, pool)
-        pending._meta = meta          # pinned memory must outlive the copy that reads it
+        # (pinned memory must outlive the copy that reads it; a greedy batch's copy is kept, and its buffer with it)
+        pending._meta, pending._meta_pool = meta, (None if all_greedy else meta_pool)
         return pending
 
     def sample(self, logits: torch.Tensor, plans: Sequence[SamplingPlan], steps: Sequence[int],
